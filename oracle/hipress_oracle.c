@@ -1,0 +1,521 @@
+/*
+ * CPU oracle for the HiPress gradient-compression hot path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing in the shipped package may link, import or
+ * call this file: it exists so that tests, the smoke check and the benchmark's
+ * CPU-baseline leg have a scalar, obviously-sequential statement of every
+ * operator to compare the HIP kernels with.
+ *
+ * Provenance of the arithmetic.  The reference checkout carries source for one
+ * compressor only, the CompLL-generated min/max stochastic quantiser
+ *   /root/reference/src/CompLL/GCGen/output/TernGradEncode/TernGradEncode_body.h:99-126
+ *   /root/reference/src/CompLL/GCGen/output/TernGradDecode/TernGradDecode_body.h:48-74
+ * and names the five built-in algorithms (onebit, TBQ, TernGrad, DGC, GradDrop,
+ * /root/reference/README.md:9) whose operator sources live in submodules that
+ * are empty directories here (/root/reference/.gitmodules:1-12:
+ * torch-hipress-extension, hipress-mxnet, tensorflow-ops, CCO; no pinned
+ * revision is recoverable).  What the checkout does fix, and what every
+ * function below follows, is
+ *   - the bit-placement rule for packed codes: code i of width b sits at bit
+ *     (i mod 8/b)*b of byte floor(i*b/8), i.e. least-significant first
+ *     (TernGradDecode_body.h:44).  hpo_get_code()/hpo_put_code() restate it on
+ *     little-endian uint32 words, which is the same byte image;
+ *   - header-then-codes payloads sized by the caller
+ *     (TernGradEncode_body.h:114,120-123);
+ *   - in-place operators over caller-allocated buffers, encode
+ *     (gradient, compressed, params), decode (compressed, gradient)
+ *     (TernGradEncode.cc:10-24, TernGradDecode.cc:10-24).
+ * The arithmetic of the five built-in compressors and of the decode-and-merge
+ * step is restated from their published algorithms (1-bit SGD, threshold
+ * two-bit quantisation, TernGrad, Deep Gradient Compression, Gradient
+ * Dropping) with the choices listed beside each function.
+ *
+ * PARITY STATUS.  The reference holds no test, golden vector or fixture for
+ * this path, and the operator sources are absent, so with respect to the
+ * reference's numbers every function here except the bit-placement helpers is
+ * "parity unpinned".  They are pinned instead by hand-worked known answers,
+ * closed forms, invariants and brute force in tests/test_oracle_*.py.
+ * hpo_get_code/hpo_put_code and hpo_compll_decode are pinned against the
+ * reference text (TernGradDecode_body.h:44,65-72).
+ *
+ * Build: gcc -O2 -ffp-contract=off -fno-fast-math (see oracle/Makefile).  All
+ * arithmetic is IEEE binary32 round-to-nearest with no contraction.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define HPO_HEADER_BYTES 16
+
+/* ------------------------------------------------------------------ */
+/* wire rule                                                          */
+/* ------------------------------------------------------------------ */
+
+/* Code i of width b: bits [b*(i mod 32/b), +b) of little-endian word
+ * floor(i*b/32).  Same byte image as TernGradDecode_body.h:44
+ * (byte floor(i*b/8), shift (i mod 8/b)*b). */
+uint32_t hpo_get_code(const uint32_t *words, int64_t i, int b)
+{
+    int per = 32 / b;
+    return (words[i / per] >> ((i % per) * b)) & ((1u << b) - 1u);
+}
+
+void hpo_put_code(uint32_t *words, int64_t i, int b, uint32_t code)
+{
+    int per = 32 / b;
+    uint32_t mask = ((1u << b) - 1u) << ((i % per) * b);
+    words[i / per] = (words[i / per] & ~mask) | ((code << ((i % per) * b)) & mask);
+}
+
+static int64_t words_for(int64_t n, int b)
+{
+    int per = 32 / b;
+    return (n + per - 1) / per;
+}
+
+static int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+/* ------------------------------------------------------------------ */
+/* payload sizes                                                      */
+/* ------------------------------------------------------------------ */
+
+int64_t hpo_onebit_payload_bytes(int64_t n) { return HPO_HEADER_BYTES + 4 * words_for(n, 1); }
+int64_t hpo_tbq_payload_bytes(int64_t n) { return HPO_HEADER_BYTES + 4 * words_for(n, 2); }
+
+int64_t hpo_terngrad_scale_bytes(int64_t n, int64_t bucket)
+{
+    int64_t nb = (n + bucket - 1) / bucket;
+    return round_up(4 * nb, 16);
+}
+
+int64_t hpo_terngrad_payload_bytes(int64_t n, int64_t bucket)
+{
+    return HPO_HEADER_BYTES + hpo_terngrad_scale_bytes(n, bucket) + 4 * words_for(n, 2);
+}
+
+/* Slots reserved for (index, value) pairs: four times the expected count,
+ * never fewer than 64 and never more than n, rounded up to a multiple of 64. */
+int64_t hpo_sparse_capacity(int64_t n, double ratio)
+{
+    int64_t want = (int64_t)ceil(4.0 * ratio * (double)n);
+    if (want > n) want = n;
+    if (want < 64) want = 64;
+    return round_up(want, 64);
+}
+
+int64_t hpo_sparse_payload_bytes(int64_t n, double ratio)
+{
+    return HPO_HEADER_BYTES + 8 * hpo_sparse_capacity(n, ratio);
+}
+
+/* ------------------------------------------------------------------ */
+/* TBQ: threshold two-bit quantisation with error feedback            */
+/* ------------------------------------------------------------------ */
+
+/* v = r + g; v >= tau -> code 1, r' = v - tau; v <= -tau -> code 2,
+ * r' = v + tau; otherwise code 0, r' = v.  NaN compares false -> code 0.
+ * Payload: {f32 tau, u32 n, 0, 0} then ceil(n/16) words, pad codes 0. */
+void hpo_tbq_encode(const float *g, float *r, int64_t n, uint8_t *payload, float tau)
+{
+    uint32_t *hdr = (uint32_t *)payload;
+    uint32_t *w = (uint32_t *)(payload + HPO_HEADER_BYTES);
+    memcpy(&hdr[0], &tau, 4);
+    hdr[1] = (uint32_t)n;
+    hdr[2] = 0;
+    hdr[3] = 0;
+    memset(w, 0, 4 * words_for(n, 2));
+    for (int64_t i = 0; i < n; ++i) {
+        float v = r[i] + g[i];
+        uint32_t code = 0;
+        if (v >= tau) {
+            code = 1;
+            v = v - tau;
+        } else if (v <= -tau) {
+            code = 2;
+            v = v + tau;
+        }
+        r[i] = v;
+        hpo_put_code(w, i, 2, code);
+    }
+}
+
+static float tbq_value(uint32_t code, float tau)
+{
+    return code == 1 ? tau : (code == 2 ? -tau : 0.0f);
+}
+
+/* code 0 -> 0, 1 -> +tau, 2 -> -tau, 3 -> 0; tau comes from the header. */
+void hpo_tbq_decode(const uint8_t *payload, float *out, int64_t n)
+{
+    float tau;
+    const uint32_t *w = (const uint32_t *)(payload + HPO_HEADER_BYTES);
+    memcpy(&tau, payload, 4);
+    for (int64_t i = 0; i < n; ++i)
+        out[i] = tbq_value(hpo_get_code(w, i, 2), tau);
+}
+
+/* ------------------------------------------------------------------ */
+/* onebit: sign quantisation, per-tensor mean-magnitude scale         */
+/* ------------------------------------------------------------------ */
+
+/* Scale s = (sum |r+g|) / n, accumulated in double and rounded once to
+ * binary32 (any summation order is acceptable to within 1e-5 relative);
+ * n = 0 gives 0. */
+float hpo_onebit_scale(const float *g, const float *r, int64_t n)
+{
+    double acc = 0.0;
+    for (int64_t i = 0; i < n; ++i) {
+        float v = r[i] + g[i];
+        acc += (double)fabsf(v);
+    }
+    return n > 0 ? (float)(acc / (double)n) : 0.0f;
+}
+
+/* Given the scale: bit = (v >= 0); d = bit ? +s : -s; r' = v - d.
+ * Payload {f32 s, u32 n, 0, 0} then ceil(n/32) words, pad bits 0. */
+void hpo_onebit_encode_with_scale(const float *g, float *r, int64_t n, uint8_t *payload, float s)
+{
+    uint32_t *hdr = (uint32_t *)payload;
+    uint32_t *w = (uint32_t *)(payload + HPO_HEADER_BYTES);
+    memcpy(&hdr[0], &s, 4);
+    hdr[1] = (uint32_t)n;
+    hdr[2] = 0;
+    hdr[3] = 0;
+    memset(w, 0, 4 * words_for(n, 1));
+    for (int64_t i = 0; i < n; ++i) {
+        float v = r[i] + g[i];
+        uint32_t bit = v >= 0.0f ? 1u : 0u;
+        float d = bit ? s : -s;
+        r[i] = v - d;
+        hpo_put_code(w, i, 1, bit);
+    }
+}
+
+void hpo_onebit_encode(const float *g, float *r, int64_t n, uint8_t *payload)
+{
+    hpo_onebit_encode_with_scale(g, r, n, payload, hpo_onebit_scale(g, r, n));
+}
+
+void hpo_onebit_decode(const uint8_t *payload, float *out, int64_t n)
+{
+    float s;
+    const uint32_t *w = (const uint32_t *)(payload + HPO_HEADER_BYTES);
+    memcpy(&s, payload, 4);
+    for (int64_t i = 0; i < n; ++i)
+        out[i] = hpo_get_code(w, i, 1) ? s : -s;
+}
+
+/* ------------------------------------------------------------------ */
+/* TernGrad: stochastic ternarisation, per-bucket max-abs scale       */
+/* ------------------------------------------------------------------ */
+
+/* Buckets of `bucket` consecutive elements over the flattened tensor (last
+ * one may be short).  s_k = max |g_i| over bucket k (NaN never wins a
+ * comparison).  Element i is kept iff u_i * s_k < |g_i| (one binary32
+ * multiply), so P(keep) = |g_i| / s_k for u uniform on [0,1).
+ * code = keep ? (g_i < 0 ? 2 : 1) : 0.  No residual.
+ * Payload {u32 n, u32 bucket, 0, 0}, f32 scale[nb] padded to 16 B, words. */
+void hpo_terngrad_encode(const float *g, const float *u, int64_t n, uint8_t *payload, int64_t bucket)
+{
+    uint32_t *hdr = (uint32_t *)payload;
+    float *scale = (float *)(payload + HPO_HEADER_BYTES);
+    int64_t sb = hpo_terngrad_scale_bytes(n, bucket);
+    uint32_t *w = (uint32_t *)(payload + HPO_HEADER_BYTES + sb);
+    int64_t nb = (n + bucket - 1) / bucket;
+    hdr[0] = (uint32_t)n;
+    hdr[1] = (uint32_t)bucket;
+    hdr[2] = 0;
+    hdr[3] = 0;
+    memset(scale, 0, sb);
+    memset(w, 0, 4 * words_for(n, 2));
+    for (int64_t k = 0; k < nb; ++k) {
+        int64_t lo = k * bucket, hi = lo + bucket < n ? lo + bucket : n;
+        float s = 0.0f;
+        for (int64_t i = lo; i < hi; ++i) {
+            float a = fabsf(g[i]);
+            if (a > s) s = a;
+        }
+        scale[k] = s;
+        for (int64_t i = lo; i < hi; ++i) {
+            float a = fabsf(g[i]);
+            float t = u[i] * s;
+            uint32_t code = 0;
+            if (t < a) code = g[i] < 0.0f ? 2u : 1u;
+            hpo_put_code(w, i, 2, code);
+        }
+    }
+}
+
+void hpo_terngrad_decode(const uint8_t *payload, float *out, int64_t n)
+{
+    const uint32_t *hdr = (const uint32_t *)payload;
+    int64_t bucket = hdr[1];
+    const float *scale = (const float *)(payload + HPO_HEADER_BYTES);
+    const uint32_t *w = (const uint32_t *)(payload + HPO_HEADER_BYTES + hpo_terngrad_scale_bytes(n, bucket));
+    for (int64_t i = 0; i < n; ++i) {
+        float s = scale[i / bucket];
+        out[i] = tbq_value(hpo_get_code(w, i, 2), s);
+    }
+}
+
+/* ------------------------------------------------------------------ */
+/* DGC / GradDrop: sampled-threshold top-k sparsification             */
+/* ------------------------------------------------------------------ */
+
+static uint32_t abs_key(float x)
+{
+    uint32_t k;
+    memcpy(&k, &x, 4);
+    return k & 0x7fffffffu; /* |x| as an order-preserving integer (NaN sorts above inf) */
+}
+
+static float key_value(uint32_t k)
+{
+    float x;
+    memcpy(&x, &k, 4);
+    return x;
+}
+
+/* k-th largest (k >= 1) of m unsigned keys by counting on 8-bit digits from
+ * the top; the result is a value, so it does not depend on any ordering of
+ * equal keys.  keys[] is overwritten. */
+static uint32_t kth_largest(uint32_t *keys, int64_t m, int64_t k)
+{
+    uint32_t prefix = 0;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        int64_t hist[256];
+        int64_t kept = 0;
+        int d;
+        memset(hist, 0, sizeof hist);
+        for (int64_t i = 0; i < m; ++i) hist[(keys[i] >> shift) & 255u]++;
+        for (d = 255; d > 0; --d) {
+            if (k <= hist[d]) break;
+            k -= hist[d];
+        }
+        prefix |= (uint32_t)d << shift;
+        for (int64_t i = 0; i < m; ++i)
+            if (((keys[i] >> shift) & 255u) == (uint32_t)d) keys[kept++] = keys[i];
+        m = kept;
+    }
+    return prefix;
+}
+
+/* Sample stride: every 100th element (a 1 % sample) once the tensor reaches
+ * 262144 elements, the compression threshold the reference's launch lines use
+ * (/root/reference/README.md:45); smaller tensors are their own sample. */
+int64_t hpo_sparse_sample_stride(int64_t n) { return n >= 262144 ? 100 : 1; }
+
+int64_t hpo_sparse_sample_count(int64_t n)
+{
+    int64_t S = hpo_sparse_sample_stride(n);
+    return n / S;
+}
+
+int64_t hpo_sparse_sample_k(int64_t n, double ratio)
+{
+    int64_t ns = hpo_sparse_sample_count(n);
+    int64_t k = (int64_t)ceil(ratio * (double)ns);
+    if (k < 1) k = 1;
+    if (k > ns) k = ns;
+    return k;
+}
+
+/* Threshold = k_s-th largest |a| over sample positions j*S + S/2. */
+float hpo_sparse_threshold(const float *a, int64_t n, double ratio)
+{
+    int64_t S = hpo_sparse_sample_stride(n);
+    int64_t ns = n / S;
+    uint32_t *keys;
+    uint32_t t;
+    if (ns <= 0) return 0.0f;
+    keys = (uint32_t *)malloc(sizeof(uint32_t) * (size_t)ns);
+    for (int64_t j = 0; j < ns; ++j) keys[j] = abs_key(a[j * S + S / 2]);
+    t = kth_largest(keys, ns, hpo_sparse_sample_k(n, ratio));
+    free(keys);
+    return key_value(t);
+}
+
+/* Select every i with |a_i| >= thr and |a_i| > 0, in ascending i.  If more
+ * than `capacity` qualify, thr becomes the capacity-th largest |a| of the
+ * whole tensor; everything above it is kept and elements equal to it are
+ * kept in ascending index order until the slots are full.  Selected
+ * positions are zeroed in a[] and, when given, in mom[] (momentum-factor
+ * masking).  Payload {u32 nnz, u32 n, u32 capacity, f32 thr}, i32
+ * idx[capacity], f32 val[capacity]; unused slots are left untouched. */
+static void sparse_select(float *a, float *mom, int64_t n, uint8_t *payload, double ratio)
+{
+    uint32_t *hdr = (uint32_t *)payload;
+    int64_t cap = hpo_sparse_capacity(n, ratio);
+    int32_t *idx = (int32_t *)(payload + HPO_HEADER_BYTES);
+    float *val = (float *)(payload + HPO_HEADER_BYTES + 4 * cap);
+    float thr = hpo_sparse_threshold(a, n, ratio);
+    uint32_t tk = abs_key(thr);
+    int64_t count = 0, eq_quota = INT64_MAX, nnz = 0;
+
+    for (int64_t i = 0; i < n; ++i) {
+        uint32_t k = abs_key(a[i]);
+        if (k >= tk && k > 0) count++;
+    }
+    if (count > cap) {
+        uint32_t *keys = (uint32_t *)malloc(sizeof(uint32_t) * (size_t)n);
+        int64_t gt = 0;
+        for (int64_t i = 0; i < n; ++i) keys[i] = abs_key(a[i]);
+        tk = kth_largest(keys, n, cap);
+        free(keys);
+        thr = key_value(tk);
+        for (int64_t i = 0; i < n; ++i)
+            if (abs_key(a[i]) > tk) gt++;
+        eq_quota = cap - gt;
+    }
+    for (int64_t i = 0; i < n; ++i) {
+        uint32_t k = abs_key(a[i]);
+        int take = 0;
+        if (k == 0) continue;
+        if (k > tk) take = 1;
+        else if (k == tk && eq_quota > 0) {
+            take = 1;
+            eq_quota--;
+        }
+        if (take) {
+            idx[nnz] = (int32_t)i;
+            val[nnz] = a[i];
+            nnz++;
+            a[i] = 0.0f;
+            if (mom) mom[i] = 0.0f;
+        }
+    }
+    hdr[0] = (uint32_t)nnz;
+    hdr[1] = (uint32_t)n;
+    hdr[2] = (uint32_t)cap;
+    memcpy(&hdr[3], &thr, 4);
+}
+
+/* DGC with momentum correction: mom' = m*mom + g (a multiply rounded to
+ * binary32, then an add rounded to binary32), acc' = acc + mom', then
+ * sampled-threshold selection on acc' with momentum-factor masking. */
+void hpo_dgc_encode(const float *g, float *mom, float *acc, int64_t n, uint8_t *payload, float m,
+                    double ratio)
+{
+    for (int64_t i = 0; i < n; ++i) {
+        float p = m * mom[i]; /* rounded product: the build disables contraction */
+        float u = p + g[i];
+        mom[i] = u;
+        acc[i] = acc[i] + u;
+    }
+    sparse_select(acc, mom, n, payload, ratio);
+}
+
+/* GradDrop: acc' = acc + g, same selection, `ratio` is the kept fraction
+ * (drop ratio 0.99 = ratio 0.01). */
+void hpo_graddrop_encode(const float *g, float *acc, int64_t n, uint8_t *payload, double ratio)
+{
+    for (int64_t i = 0; i < n; ++i) acc[i] = acc[i] + g[i];
+    sparse_select(acc, NULL, n, payload, ratio);
+}
+
+/* Zero-fill then scatter; entries past n or past capacity are ignored. */
+void hpo_sparse_decode(const uint8_t *payload, float *out, int64_t n)
+{
+    const uint32_t *hdr = (const uint32_t *)payload;
+    int64_t nnz = hdr[0], cap = hdr[2];
+    const int32_t *idx = (const int32_t *)(payload + HPO_HEADER_BYTES);
+    const float *val = (const float *)(payload + HPO_HEADER_BYTES + 4 * cap);
+    if (nnz > cap) nnz = cap;
+    memset(out, 0, sizeof(float) * (size_t)n);
+    for (int64_t j = 0; j < nnz; ++j)
+        if (idx[j] >= 0 && idx[j] < n) out[idx[j]] = val[j];
+}
+
+/* ------------------------------------------------------------------ */
+/* decode-and-merge                                                   */
+/* ------------------------------------------------------------------ */
+
+/* agg[i] = ((0 + d_1[i]) + d_2[i]) + ... in peer order, binary32.  If r is
+ * not NULL the aggregate is re-encoded for the next hop with the
+ * aggregator's own residual r and threshold tau into out_payload. */
+void hpo_tbq_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n, float *r,
+                          uint8_t *out_payload, float tau)
+{
+    for (int64_t i = 0; i < n; ++i) agg[i] = 0.0f;
+    for (int p = 0; p < npeers; ++p) {
+        float t;
+        const uint32_t *w = (const uint32_t *)(payloads[p] + HPO_HEADER_BYTES);
+        memcpy(&t, payloads[p], 4);
+        for (int64_t i = 0; i < n; ++i) agg[i] = agg[i] + tbq_value(hpo_get_code(w, i, 2), t);
+    }
+    if (r) hpo_tbq_encode(agg, r, n, out_payload, tau);
+}
+
+void hpo_onebit_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n)
+{
+    for (int64_t i = 0; i < n; ++i) agg[i] = 0.0f;
+    for (int p = 0; p < npeers; ++p) {
+        float s;
+        const uint32_t *w = (const uint32_t *)(payloads[p] + HPO_HEADER_BYTES);
+        memcpy(&s, payloads[p], 4);
+        for (int64_t i = 0; i < n; ++i) agg[i] = agg[i] + (hpo_get_code(w, i, 1) ? s : -s);
+    }
+}
+
+void hpo_terngrad_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n)
+{
+    for (int64_t i = 0; i < n; ++i) agg[i] = 0.0f;
+    for (int p = 0; p < npeers; ++p) {
+        const uint32_t *hdr = (const uint32_t *)payloads[p];
+        int64_t bucket = hdr[1];
+        const float *scale = (const float *)(payloads[p] + HPO_HEADER_BYTES);
+        const uint32_t *w =
+            (const uint32_t *)(payloads[p] + HPO_HEADER_BYTES + hpo_terngrad_scale_bytes(n, bucket));
+        for (int64_t i = 0; i < n; ++i)
+            agg[i] = agg[i] + tbq_value(hpo_get_code(w, i, 2), scale[i / bucket]);
+    }
+}
+
+/* Zero-fill, then scatter-ADD every peer's pairs in peer order and slot
+ * order (duplicates across peers sum).  If acc is not NULL the aggregate is
+ * re-sparsified for the next hop GradDrop-style with the aggregator's
+ * residual acc: acc' = acc + agg, select, zero. */
+void hpo_sparse_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n,
+                             float *acc, uint8_t *out_payload, double ratio)
+{
+    memset(agg, 0, sizeof(float) * (size_t)n);
+    for (int p = 0; p < npeers; ++p) {
+        const uint32_t *hdr = (const uint32_t *)payloads[p];
+        int64_t nnz = hdr[0], cap = hdr[2];
+        const int32_t *idx = (const int32_t *)(payloads[p] + HPO_HEADER_BYTES);
+        const float *val = (const float *)(payloads[p] + HPO_HEADER_BYTES + 4 * cap);
+        if (nnz > cap) nnz = cap;
+        for (int64_t j = 0; j < nnz; ++j)
+            if (idx[j] >= 0 && idx[j] < n) agg[idx[j]] = agg[idx[j]] + val[j];
+    }
+    if (acc) hpo_graddrop_encode(agg, acc, n, out_payload, ratio);
+}
+
+/* ------------------------------------------------------------------ */
+/* CompLL generated-operator wire format (10-byte header)             */
+/* ------------------------------------------------------------------ */
+
+/* Decode of the in-tree generated operator, as written
+ * (TernGradDecode_body.h:48-74): header [bitwidth:u8][tail:u8][min:f32]
+ * [max:f32] at byte offsets 0,1,2,6, codes from byte 10;
+ * gap = (max-min)/((1<<b)-1); count = (8*csz - 80)/b - tail;
+ * out[i] = code_i*gap + min with code_i at bit (i mod 8/b)*b of byte
+ * floor(i*b/8).  Returns the element count written (at most out_cap). */
+int64_t hpo_compll_decode(const uint8_t *compressed, int64_t csz, float *out, int64_t out_cap)
+{
+    uint8_t b = compressed[0], tail = compressed[1];
+    float mn, mx, gap;
+    const uint8_t *Q = compressed + 10;
+    int64_t count;
+    memcpy(&mn, compressed + 2, 4);
+    memcpy(&mx, compressed + 6, 4);
+    gap = (mx - mn) / (float)((1 << b) - 1);
+    count = (8 * csz - 80) / b - tail;
+    if (count > out_cap) count = out_cap;
+    for (int64_t i = 0; i < count; ++i) {
+        uint32_t code = (Q[i * b / 8] >> ((i % (8 / b)) * b)) & ((1u << b) - 1u);
+        out[i] = (float)code * gap + mn;
+    }
+    return count < 0 ? 0 : count;
+}
