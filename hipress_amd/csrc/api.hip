@@ -1,0 +1,780 @@
+// C ABI of libhipress_amd.so: argument validation, tensor descriptors, batched
+// launch objects.  Kernels live in dense.hip, sparse.hip and merge.hip.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "../../include/hipress_amd.h"
+#include "common.h"
+#include "launch.h"
+
+using namespace hp;
+
+namespace {
+
+constexpr int64_t kSampleFrom = 262144;  // tensors at least this large are sampled at stride 100
+constexpr int64_t kSampleStride = 100;
+
+inline bool mis(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
+inline bool al16(const void* p) { return !mis(p, 16); }
+inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+inline unsigned tiles_of(int64_t n) { return n <= 0 ? 1u : (unsigned)((n + kTile - 1) / kTile); }
+inline bool bad_n(int64_t n) { return n < 0 || n > HIPRESS_MAX_N; }
+
+inline int64_t words_bytes(int64_t n, int bits) {
+    int per = 32 / bits;
+    return 4 * ((n + per - 1) / per);
+}
+
+inline int64_t tg_scale_bytes(int64_t n, int64_t bucket) { return round_up(4 * ((n + bucket - 1) / bucket), 16); }
+
+struct SparsePlan {
+    int64_t cap, stride, ns, ks;
+};
+
+inline SparsePlan sparse_plan(int64_t n, double ratio) {
+    SparsePlan p;
+    int64_t want = (int64_t)std::ceil(4.0 * ratio * (double)n);
+    if (want > n) want = n;
+    if (want < 64) want = 64;
+    p.cap = round_up(want, 64);
+    p.stride = n >= kSampleFrom ? kSampleStride : 1;
+    p.ns = n / p.stride;
+    p.ks = (int64_t)std::ceil(ratio * (double)p.ns);
+    if (p.ks < 1) p.ks = 1;
+    if (p.ks > p.ns) p.ks = p.ns;
+    return p;
+}
+
+inline bool bad_ratio(double r) { return !(r > 0.0 && r <= 1.0); }
+
+// Workspace of a sparse launch: four uint32 arrays, each starting on a 256-byte boundary.
+struct SparseWsLayout {
+    int64_t sample_off, gmax_off, counts_off, thr_off, bytes;
+};
+
+inline SparseWsLayout sparse_ws_layout(int64_t total_ns, int64_t total_tiles, int64_t nsegs) {
+    SparseWsLayout l;
+    int64_t off = 0;
+    l.sample_off = off;
+    off += round_up(4 * total_ns, 256);
+    l.gmax_off = off;
+    off += round_up(4 * 64 * total_tiles, 256);
+    l.counts_off = off;
+    off += round_up(4 * 8 * total_tiles, 256);
+    l.thr_off = off;
+    off += round_up(4 * 2 * nsegs, 256);
+    l.bytes = off;
+    return l;
+}
+
+inline SparseWs sparse_ws_at(void* base, const SparseWsLayout& l) {
+    uint8_t* b = static_cast<uint8_t*>(base);
+    SparseWs w;
+    w.sample = reinterpret_cast<uint32_t*>(b + l.sample_off);
+    w.gmax = reinterpret_cast<uint32_t*>(b + l.gmax_off);
+    w.counts = reinterpret_cast<uint32_t*>(b + l.counts_off);
+    w.thr = reinterpret_cast<uint32_t*>(b + l.thr_off);
+    return w;
+}
+
+inline int hiperr(hipError_t e) { return e == hipSuccess ? HIPRESS_OK : HIPRESS_ERR_HIP; }
+
+// ---- descriptor builders: validate one tensor and fill its Seg -------------------------
+
+int payload_need(int alg, int64_t n, const hipress_params& pr, int64_t* need) {
+    switch (alg) {
+        case HIPRESS_ONEBIT: *need = HIPRESS_HEADER_BYTES + words_bytes(n, 1); return HIPRESS_OK;
+        case HIPRESS_TBQ: *need = HIPRESS_HEADER_BYTES + words_bytes(n, 2); return HIPRESS_OK;
+        case HIPRESS_TERNGRAD:
+            if (pr.bucket < 1) return HIPRESS_ERR_PARAM;
+            *need = HIPRESS_HEADER_BYTES + tg_scale_bytes(n, pr.bucket) + words_bytes(n, 2);
+            return HIPRESS_OK;
+        case HIPRESS_DGC:
+        case HIPRESS_GRADDROP:
+            if (bad_ratio(pr.ratio)) return HIPRESS_ERR_PARAM;
+            *need = HIPRESS_HEADER_BYTES + 8 * sparse_plan(n, pr.ratio).cap;
+            return HIPRESS_OK;
+    }
+    return HIPRESS_ERR_PARAM;
+}
+
+int check_params(int alg, const hipress_params& pr) {
+    switch (alg) {
+        case HIPRESS_ONEBIT: return HIPRESS_OK;
+        case HIPRESS_TBQ: return (pr.threshold >= 0.f && std::isfinite(pr.threshold)) ? HIPRESS_OK : HIPRESS_ERR_PARAM;
+        case HIPRESS_TERNGRAD: return pr.bucket >= 1 ? HIPRESS_OK : HIPRESS_ERR_PARAM;
+        case HIPRESS_DGC:
+            if (!std::isfinite(pr.momentum_factor)) return HIPRESS_ERR_PARAM;
+            return bad_ratio(pr.ratio) ? HIPRESS_ERR_PARAM : HIPRESS_OK;
+        case HIPRESS_GRADDROP: return bad_ratio(pr.ratio) ? HIPRESS_ERR_PARAM : HIPRESS_OK;
+    }
+    return HIPRESS_ERR_PARAM;
+}
+
+// Fills the fields of `s` that do not depend on the tensor's place in a launch.
+int build_encode_seg(int alg, const hipress_tensor& t, const hipress_params& pr, Seg* s) {
+    std::memset(s, 0, sizeof(Seg));
+    if (bad_n(t.n)) return HIPRESS_ERR_SIZE;
+    int rc = check_params(alg, pr);
+    if (rc) return rc;
+    if (!t.payload) return HIPRESS_ERR_NULL;
+    if (mis(t.payload, 16)) return HIPRESS_ERR_ALIGN;
+    int64_t need;
+    if ((rc = payload_need(alg, t.n, pr, &need))) return rc;
+    if (t.payload_bytes < need) return HIPRESS_ERR_SIZE;
+    const bool need_s0 = alg == HIPRESS_ONEBIT || alg == HIPRESS_TBQ || alg == HIPRESS_DGC || alg == HIPRESS_GRADDROP;
+    const bool need_s1 = alg == HIPRESS_DGC;
+    const bool need_u = alg == HIPRESS_TERNGRAD;
+    if (t.n > 0) {
+        if (!t.grad || (need_s0 && !t.state0) || (need_s1 && !t.state1) || (need_u && !t.uniform)) return HIPRESS_ERR_NULL;
+    }
+    if (mis(t.grad, 4) || mis(t.state0, 4) || mis(t.state1, 4) || mis(t.uniform, 4)) return HIPRESS_ERR_ALIGN;
+    s->g = t.grad;
+    s->pay = static_cast<uint8_t*>(t.payload);
+    s->n = (unsigned long long)t.n;
+    s->ntiles = tiles_of(t.n);
+    s->aligned = al16(t.grad);
+    switch (alg) {
+        case HIPRESS_ONEBIT:
+        case HIPRESS_TBQ:
+            s->s0 = t.state0;
+            s->aligned = s->aligned && al16(t.state0);
+            s->f0 = pr.threshold;
+            s->words_off = HIPRESS_HEADER_BYTES;
+            break;
+        case HIPRESS_TERNGRAD: {
+            s->u = t.uniform;
+            s->aligned = s->aligned && al16(t.uniform);
+            s->bucket = (unsigned)pr.bucket;
+            int64_t off = HIPRESS_HEADER_BYTES + tg_scale_bytes(t.n, pr.bucket);
+            if (off > 0xffffffffLL) return HIPRESS_ERR_SIZE;
+            s->words_off = (unsigned)off;
+            break;
+        }
+        case HIPRESS_DGC:
+        case HIPRESS_GRADDROP: {
+            if (alg == HIPRESS_DGC) {
+                s->s0 = t.state0;
+                s->s1 = t.state1;
+                s->f0 = pr.momentum_factor;
+                s->aligned = s->aligned && al16(t.state0) && al16(t.state1);
+            } else {
+                s->s0 = nullptr;
+                s->s1 = t.state0;
+                s->aligned = s->aligned && al16(t.state0);
+            }
+            SparsePlan p = sparse_plan(t.n, pr.ratio);
+            s->cap = (unsigned)p.cap;
+            s->sstride = (unsigned)p.stride;
+            s->ns = (unsigned)p.ns;
+            s->ks = (unsigned)p.ks;
+            break;
+        }
+    }
+    return HIPRESS_OK;
+}
+
+int build_decode_seg(int alg, const void* payload, int64_t payload_bytes, float* out, int64_t n, Seg* s) {
+    std::memset(s, 0, sizeof(Seg));
+    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (!payload || (n > 0 && !out)) return HIPRESS_ERR_NULL;
+    if (mis(payload, 16) || mis(out, 4)) return HIPRESS_ERR_ALIGN;
+    if (payload_bytes < HIPRESS_HEADER_BYTES) return HIPRESS_ERR_SIZE;
+    s->pay = const_cast<uint8_t*>(static_cast<const uint8_t*>(payload));
+    s->pay_bytes = (unsigned long long)payload_bytes;
+    s->out = out;
+    s->n = (unsigned long long)n;
+    s->ntiles = tiles_of(n);
+    s->aligned = al16(out);
+    s->words_off = HIPRESS_HEADER_BYTES;
+    switch (alg) {
+        case HIPRESS_ONEBIT:
+            if (payload_bytes < HIPRESS_HEADER_BYTES + words_bytes(n, 1)) return HIPRESS_ERR_SIZE;
+            break;
+        case HIPRESS_TBQ:
+            if (payload_bytes < HIPRESS_HEADER_BYTES + words_bytes(n, 2)) return HIPRESS_ERR_SIZE;
+            break;
+        case HIPRESS_TERNGRAD:
+            // the bucket size lives in the header on the device; the caller-side
+            // size check is done by the variant that knows the bucket
+            break;
+        case HIPRESS_DGC:
+        case HIPRESS_GRADDROP: {
+            int64_t slots = (payload_bytes - HIPRESS_HEADER_BYTES) / 8;
+            s->cap = (unsigned)(slots > 0xffffffffLL ? 0xffffffffLL : slots);
+            break;
+        }
+        default: return HIPRESS_ERR_PARAM;
+    }
+    return HIPRESS_OK;
+}
+
+// TernGrad decode needs the bucket size to place the words; the host passes it.
+int finish_terngrad_decode_seg(Seg* s, int64_t payload_bytes, int32_t bucket) {
+    if (bucket < 1) return HIPRESS_ERR_PARAM;
+    int64_t off = HIPRESS_HEADER_BYTES + tg_scale_bytes((int64_t)s->n, bucket);
+    if (off > 0xffffffffLL) return HIPRESS_ERR_SIZE;
+    if (payload_bytes < off + words_bytes((int64_t)s->n, 2)) return HIPRESS_ERR_SIZE;
+    s->bucket = (unsigned)bucket;
+    s->words_off = (unsigned)off;
+    return HIPRESS_OK;
+}
+
+Launch single_launch(const Seg& s) {
+    Launch L;
+    std::memset(&L, 0, sizeof L);
+    L.single = true;
+    L.seg = s;
+    L.seg.tile0 = 0;
+    L.seg.id = 0;
+    L.seg.ws0 = 0;
+    L.ntiles = s.ntiles;
+    L.nsegs = 1;
+    return L;
+}
+
+template <class T>
+int upload(const std::vector<T>& v, T** dptr) {
+    *dptr = nullptr;
+    if (v.empty()) return HIPRESS_OK;
+    if (hipMalloc(reinterpret_cast<void**>(dptr), v.size() * sizeof(T)) != hipSuccess) return HIPRESS_ERR_HIP;
+    if (hipMemcpy(*dptr, v.data(), v.size() * sizeof(T), hipMemcpyHostToDevice) != hipSuccess) return HIPRESS_ERR_HIP;
+    return HIPRESS_OK;
+}
+
+// Assigns tile ranges to the tensors of a launch and builds the workgroup -> (tensor, tile) map.
+template <class S, class GetSeg>
+int layout_tiles(std::vector<S>& segs, GetSeg seg_of, std::vector<uint2>& map, unsigned* total) {
+    uint64_t t = 0;
+    for (size_t i = 0; i < segs.size(); ++i) {
+        Seg& s = seg_of(segs[i]);
+        s.tile0 = (unsigned)t;
+        s.id = (unsigned)i;
+        t += s.ntiles;
+        if (t > 0x7fffffffull) return HIPRESS_ERR_SIZE;
+    }
+    map.resize((size_t)t);
+    size_t k = 0;
+    for (size_t i = 0; i < segs.size(); ++i) {
+        Seg& s = seg_of(segs[i]);
+        for (unsigned j = 0; j < s.ntiles; ++j) map[k++] = make_uint2((unsigned)i, j);
+    }
+    *total = (unsigned)t;
+    return HIPRESS_OK;
+}
+
+}  // namespace
+
+// ============================================================================
+// batch objects
+// ============================================================================
+
+struct hipress_batch {
+    int alg = 0;
+    hipress_params params{};
+    std::vector<Seg> enc, dec;
+    bool can_encode = false, can_decode = false;
+    Seg* d_enc = nullptr;
+    Seg* d_dec = nullptr;
+    uint2* d_map = nullptr;
+    unsigned ntiles = 0;
+    void* ws = nullptr;  // onebit: one float per tile; sparse: SparseWsLayout
+    SparseWsLayout swl{};
+};
+
+struct hipress_merge_batch {
+    int alg = 0;
+    hipress_params params{};
+    int npeers = 0;
+    bool reencode = false;
+    std::vector<MergeSeg> segs;
+    std::vector<Seg> renc;  // sparse re-encode descriptors
+    MergeSeg* d_segs = nullptr;
+    Seg* d_renc = nullptr;
+    uint2* d_map = nullptr;
+    unsigned ntiles = 0;
+    void* ws = nullptr;
+    SparseWsLayout swl{};
+};
+
+extern "C" {
+
+int hipress_version(void) { return 100; }
+
+const char* hipress_strerror(int code) {
+    switch (code) {
+        case HIPRESS_OK: return "ok";
+        case HIPRESS_ERR_NULL: return "a required pointer is NULL";
+        case HIPRESS_ERR_SIZE: return "element count out of range or buffer too small";
+        case HIPRESS_ERR_ALIGN: return "pointer not sufficiently aligned";
+        case HIPRESS_ERR_PARAM: return "parameter out of range";
+        case HIPRESS_ERR_HIP: return "HIP runtime error";
+        case HIPRESS_ERR_WORKSPACE: return "workspace missing or too small";
+    }
+    return "unknown error";
+}
+
+// ---- sizes -----------------------------------------------------------------------
+
+int64_t hipress_onebit_payload_bytes(int64_t n) {
+    return bad_n(n) ? HIPRESS_ERR_SIZE : HIPRESS_HEADER_BYTES + words_bytes(n, 1);
+}
+int64_t hipress_tbq_payload_bytes(int64_t n) {
+    return bad_n(n) ? HIPRESS_ERR_SIZE : HIPRESS_HEADER_BYTES + words_bytes(n, 2);
+}
+int64_t hipress_terngrad_payload_bytes(int64_t n, int32_t bucket) {
+    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (bucket < 1) return HIPRESS_ERR_PARAM;
+    return HIPRESS_HEADER_BYTES + tg_scale_bytes(n, bucket) + words_bytes(n, 2);
+}
+int64_t hipress_sparse_capacity(int64_t n, double ratio) {
+    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (bad_ratio(ratio)) return HIPRESS_ERR_PARAM;
+    return sparse_plan(n, ratio).cap;
+}
+int64_t hipress_sparse_payload_bytes(int64_t n, double ratio) {
+    int64_t c = hipress_sparse_capacity(n, ratio);
+    return c < 0 ? c : HIPRESS_HEADER_BYTES + 8 * c;
+}
+int64_t hipress_onebit_workspace_bytes(int64_t n) {
+    return bad_n(n) ? HIPRESS_ERR_SIZE : round_up(4 * (int64_t)tiles_of(n), 256);
+}
+int64_t hipress_sparse_workspace_bytes(int64_t n, double ratio) {
+    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (bad_ratio(ratio)) return HIPRESS_ERR_PARAM;
+    return sparse_ws_layout(sparse_plan(n, ratio).ns, tiles_of(n), 1).bytes;
+}
+
+// ---- TBQ -------------------------------------------------------------------------
+
+int hipress_tbq_encode(const float* grad, float* residual, int64_t n, void* payload, int64_t payload_bytes,
+                       float threshold, void* stream) {
+    hipress_tensor t{grad, residual, nullptr, nullptr, payload, nullptr, n, payload_bytes};
+    hipress_params pr{};
+    pr.threshold = threshold;
+    Seg s;
+    int rc = build_encode_seg(HIPRESS_TBQ, t, pr, &s);
+    if (rc) return rc;
+    return hiperr(launch_tbq_encode(single_launch(s), static_cast<hipStream_t>(stream)));
+}
+
+int hipress_tbq_decode(const void* payload, int64_t payload_bytes, float* out, int64_t n, void* stream) {
+    Seg s;
+    int rc = build_decode_seg(HIPRESS_TBQ, payload, payload_bytes, out, n, &s);
+    if (rc) return rc;
+    return hiperr(launch_tbq_decode(single_launch(s), static_cast<hipStream_t>(stream)));
+}
+
+// ---- onebit ------------------------------------------------------------------------
+
+int hipress_onebit_encode(const float* grad, float* residual, int64_t n, void* payload, int64_t payload_bytes,
+                          void* workspace, int64_t workspace_bytes, void* stream) {
+    hipress_tensor t{grad, residual, nullptr, nullptr, payload, nullptr, n, payload_bytes};
+    hipress_params pr{};
+    Seg s;
+    int rc = build_encode_seg(HIPRESS_ONEBIT, t, pr, &s);
+    if (rc) return rc;
+    if (!workspace || workspace_bytes < hipress_onebit_workspace_bytes(n)) return HIPRESS_ERR_WORKSPACE;
+    if (mis(workspace, 16)) return HIPRESS_ERR_ALIGN;
+    return hiperr(launch_onebit_encode(single_launch(s), static_cast<float*>(workspace), static_cast<hipStream_t>(stream)));
+}
+
+int hipress_onebit_decode(const void* payload, int64_t payload_bytes, float* out, int64_t n, void* stream) {
+    Seg s;
+    int rc = build_decode_seg(HIPRESS_ONEBIT, payload, payload_bytes, out, n, &s);
+    if (rc) return rc;
+    return hiperr(launch_onebit_decode(single_launch(s), static_cast<hipStream_t>(stream)));
+}
+
+// ---- TernGrad ----------------------------------------------------------------------
+
+int hipress_terngrad_encode(const float* grad, const float* uniform, int64_t n, void* payload,
+                            int64_t payload_bytes, int32_t bucket, void* stream) {
+    hipress_tensor t{grad, nullptr, nullptr, uniform, payload, nullptr, n, payload_bytes};
+    hipress_params pr{};
+    pr.bucket = bucket;
+    Seg s;
+    int rc = build_encode_seg(HIPRESS_TERNGRAD, t, pr, &s);
+    if (rc) return rc;
+    return hiperr(launch_terngrad_encode(single_launch(s), (unsigned)bucket, static_cast<hipStream_t>(stream)));
+}
+
+// The bucket size is read from the payload header on the device and the scale
+// array that precedes the words is located with it there (checked against
+// payload_bytes on the device); the host-side check covers header and words.
+int hipress_terngrad_decode(const void* payload, int64_t payload_bytes, float* out, int64_t n, void* stream) {
+    Seg s;
+    int rc = build_decode_seg(HIPRESS_TERNGRAD, payload, payload_bytes, out, n, &s);
+    if (rc) return rc;
+    if (payload_bytes < HIPRESS_HEADER_BYTES + words_bytes(n, 2)) return HIPRESS_ERR_SIZE;
+    return hiperr(launch_terngrad_decode(single_launch(s), static_cast<hipStream_t>(stream)));
+}
+
+// ---- DGC / GradDrop ------------------------------------------------------------------
+
+static int sparse_encode_single(int alg, const hipress_tensor& t, const hipress_params& pr, void* workspace,
+                                int64_t workspace_bytes, void* stream) {
+    Seg s;
+    int rc = build_encode_seg(alg, t, pr, &s);
+    if (rc) return rc;
+    SparseWsLayout l = sparse_ws_layout(s.ns, s.ntiles, 1);
+    if (!workspace || workspace_bytes < l.bytes) return HIPRESS_ERR_WORKSPACE;
+    if (mis(workspace, 16)) return HIPRESS_ERR_ALIGN;
+    return hiperr(launch_sparse_encode(single_launch(s), alg == HIPRESS_DGC, sparse_ws_at(workspace, l),
+                                       static_cast<hipStream_t>(stream)));
+}
+
+int hipress_dgc_encode(const float* grad, float* momentum, float* accumulator, int64_t n, void* payload,
+                       int64_t payload_bytes, float momentum_factor, double ratio, void* workspace,
+                       int64_t workspace_bytes, void* stream) {
+    hipress_tensor t{grad, momentum, accumulator, nullptr, payload, nullptr, n, payload_bytes};
+    hipress_params pr{};
+    pr.momentum_factor = momentum_factor;
+    pr.ratio = ratio;
+    return sparse_encode_single(HIPRESS_DGC, t, pr, workspace, workspace_bytes, stream);
+}
+
+int hipress_graddrop_encode(const float* grad, float* accumulator, int64_t n, void* payload,
+                            int64_t payload_bytes, double ratio, void* workspace, int64_t workspace_bytes,
+                            void* stream) {
+    hipress_tensor t{grad, accumulator, nullptr, nullptr, payload, nullptr, n, payload_bytes};
+    hipress_params pr{};
+    pr.ratio = ratio;
+    return sparse_encode_single(HIPRESS_GRADDROP, t, pr, workspace, workspace_bytes, stream);
+}
+
+int hipress_sparse_decode(const void* payload, int64_t payload_bytes, float* out, int64_t n, void* stream) {
+    Seg s;
+    int rc = build_decode_seg(HIPRESS_DGC, payload, payload_bytes, out, n, &s);
+    if (rc) return rc;
+    return hiperr(launch_sparse_decode(single_launch(s), static_cast<hipStream_t>(stream)));
+}
+
+// ---- decode-and-merge ------------------------------------------------------------------
+
+static int build_merge_seg(int alg, const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
+                           float* aggregate, int64_t n, MergeSeg* m) {
+    std::memset(m, 0, sizeof(MergeSeg));
+    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (npeers < 1 || npeers > HIPRESS_MAX_PEERS) return HIPRESS_ERR_PARAM;
+    if (!payloads || !payload_bytes || (n > 0 && !aggregate)) return HIPRESS_ERR_NULL;
+    if (mis(aggregate, 4)) return HIPRESS_ERR_ALIGN;
+    for (int p = 0; p < npeers; ++p) {
+        if (!payloads[p]) return HIPRESS_ERR_NULL;
+        if (mis(payloads[p], 16)) return HIPRESS_ERR_ALIGN;
+        int64_t need = HIPRESS_HEADER_BYTES;
+        if (alg == HIPRESS_ONEBIT) need += words_bytes(n, 1);
+        else if (alg == HIPRESS_TBQ || alg == HIPRESS_TERNGRAD) need += words_bytes(n, 2);
+        if (payload_bytes[p] < need) return HIPRESS_ERR_SIZE;
+        m->peer[p] = static_cast<const uint8_t*>(payloads[p]);
+        m->peer_bytes[p] = (unsigned long long)payload_bytes[p];
+        int64_t slots = (payload_bytes[p] - HIPRESS_HEADER_BYTES) / 8;
+        m->peer_slots[p] = (unsigned)(slots > 0xffffffffLL ? 0xffffffffLL : slots);
+    }
+    m->s.out = aggregate;
+    m->s.n = (unsigned long long)n;
+    m->s.ntiles = tiles_of(n);
+    m->s.aligned = al16(aggregate);
+    return HIPRESS_OK;
+}
+
+static MergeLaunch single_merge_launch(const MergeSeg& m, int npeers, bool reencode) {
+    MergeLaunch L;
+    std::memset(&L, 0, sizeof L);
+    L.single = true;
+    L.seg = m;
+    L.ntiles = m.s.ntiles;
+    L.nsegs = 1;
+    L.npeers = npeers;
+    L.reencode = reencode;
+    return L;
+}
+
+static int add_tbq_reencode(MergeSeg* m, float* residual, void* out_payload, int64_t out_payload_bytes, float threshold) {
+    if (!out_payload) return HIPRESS_ERR_NULL;
+    if (mis(out_payload, 16) || mis(residual, 4)) return HIPRESS_ERR_ALIGN;
+    if (!(threshold >= 0.f && std::isfinite(threshold))) return HIPRESS_ERR_PARAM;
+    if (out_payload_bytes < HIPRESS_HEADER_BYTES + words_bytes((int64_t)m->s.n, 2)) return HIPRESS_ERR_SIZE;
+    m->s.s0 = residual;
+    m->s.pay = static_cast<uint8_t*>(out_payload);
+    m->s.f0 = threshold;
+    m->s.aligned = m->s.aligned && al16(residual);
+    return HIPRESS_OK;
+}
+
+int hipress_tbq_decode_merge(const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
+                             float* aggregate, int64_t n, float* residual, void* out_payload,
+                             int64_t out_payload_bytes, float threshold, void* stream) {
+    MergeSeg m;
+    int rc = build_merge_seg(HIPRESS_TBQ, payloads, payload_bytes, npeers, aggregate, n, &m);
+    if (rc) return rc;
+    if (residual && (rc = add_tbq_reencode(&m, residual, out_payload, out_payload_bytes, threshold))) return rc;
+    return hiperr(launch_dense_merge(single_merge_launch(m, npeers, residual != nullptr), HIPRESS_TBQ,
+                                     static_cast<hipStream_t>(stream)));
+}
+
+int hipress_onebit_decode_merge(const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
+                                float* aggregate, int64_t n, void* stream) {
+    MergeSeg m;
+    int rc = build_merge_seg(HIPRESS_ONEBIT, payloads, payload_bytes, npeers, aggregate, n, &m);
+    if (rc) return rc;
+    return hiperr(launch_dense_merge(single_merge_launch(m, npeers, false), HIPRESS_ONEBIT,
+                                     static_cast<hipStream_t>(stream)));
+}
+
+int hipress_terngrad_decode_merge(const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
+                                  float* aggregate, int64_t n, void* stream) {
+    MergeSeg m;
+    int rc = build_merge_seg(HIPRESS_TERNGRAD, payloads, payload_bytes, npeers, aggregate, n, &m);
+    if (rc) return rc;
+    return hiperr(launch_dense_merge(single_merge_launch(m, npeers, false), HIPRESS_TERNGRAD,
+                                     static_cast<hipStream_t>(stream)));
+}
+
+int hipress_sparse_decode_merge(const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
+                                float* aggregate, int64_t n, float* accumulator, void* out_payload,
+                                int64_t out_payload_bytes, double ratio, void* workspace,
+                                int64_t workspace_bytes, void* stream) {
+    MergeSeg m;
+    int rc = build_merge_seg(HIPRESS_DGC, payloads, payload_bytes, npeers, aggregate, n, &m);
+    if (rc) return rc;
+    Seg s;
+    SparseWsLayout l{};
+    if (accumulator) {
+        hipress_tensor t{aggregate, accumulator, nullptr, nullptr, out_payload, nullptr, n, out_payload_bytes};
+        hipress_params pr{};
+        pr.ratio = ratio;
+        if ((rc = build_encode_seg(HIPRESS_GRADDROP, t, pr, &s))) return rc;
+        l = sparse_ws_layout(s.ns, s.ntiles, 1);
+        if (!workspace || workspace_bytes < l.bytes) return HIPRESS_ERR_WORKSPACE;
+        if (mis(workspace, 16)) return HIPRESS_ERR_ALIGN;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipError_t e = launch_sparse_merge_scatter(single_merge_launch(m, npeers, false), st);
+    if (e != hipSuccess) return HIPRESS_ERR_HIP;
+    if (accumulator) e = launch_sparse_encode(single_launch(s), false, sparse_ws_at(workspace, l), st);
+    return hiperr(e);
+}
+
+// ---- batches ---------------------------------------------------------------------------
+
+int hipress_batch_destroy(hipress_batch* b) {
+    if (!b) return HIPRESS_OK;
+    (void)hipFree(b->d_enc);
+    (void)hipFree(b->d_dec);
+    (void)hipFree(b->d_map);
+    (void)hipFree(b->ws);
+    delete b;
+    return HIPRESS_OK;
+}
+
+int hipress_batch_create(hipress_batch** out, int32_t alg, const hipress_tensor* tensors, int32_t count,
+                         const hipress_params* params) {
+    if (!out || !params || (count > 0 && !tensors)) return HIPRESS_ERR_NULL;
+    *out = nullptr;
+    if (count < 0) return HIPRESS_ERR_SIZE;
+    if (alg < HIPRESS_ONEBIT || alg > HIPRESS_GRADDROP) return HIPRESS_ERR_PARAM;
+    int rc = check_params(alg, *params);
+    if (rc) return rc;
+    hipress_batch* b = new (std::nothrow) hipress_batch;
+    if (!b) return HIPRESS_ERR_HIP;
+    b->alg = alg;
+    b->params = *params;
+    const bool sparse = alg == HIPRESS_DGC || alg == HIPRESS_GRADDROP;
+    // A batch may be built for encode, for decode, or for both: a side is enabled
+    // when every tensor carries the buffers that side needs.
+    bool enc_ok = true, dec_ok = true;
+    for (int i = 0; i < count; ++i) {
+        const hipress_tensor& t = tensors[i];
+        if (t.n > 0 && !t.grad) enc_ok = false;
+        if (t.n > 0 && !t.out) dec_ok = false;
+    }
+    if (!enc_ok && !dec_ok) { delete b; return HIPRESS_ERR_NULL; }
+    b->can_encode = enc_ok;
+    b->can_decode = dec_ok;
+    auto fail = [&](int code) { hipress_batch_destroy(b); return code; };
+    for (int i = 0; i < count; ++i) {
+        const hipress_tensor& t = tensors[i];
+        Seg s;
+        if (enc_ok) {
+            if ((rc = build_encode_seg(alg, t, *params, &s))) return fail(rc);
+            b->enc.push_back(s);
+        }
+        if (dec_ok) {
+            if ((rc = build_decode_seg(alg, t.payload, t.payload_bytes, t.out, t.n, &s))) return fail(rc);
+            if (alg == HIPRESS_TERNGRAD && (rc = finish_terngrad_decode_seg(&s, t.payload_bytes, params->bucket))) return fail(rc);
+            b->dec.push_back(s);
+        }
+    }
+    std::vector<uint2> map;
+    auto ident = [](Seg& s) -> Seg& { return s; };
+    if (enc_ok && (rc = layout_tiles(b->enc, ident, map, &b->ntiles))) return fail(rc);
+    if (dec_ok && (rc = layout_tiles(b->dec, ident, map, &b->ntiles))) return fail(rc);
+    if (enc_ok && sparse) {
+        uint64_t off = 0;
+        for (Seg& s : b->enc) {
+            s.ws0 = off;
+            off += (s.ns + 3u) & ~3ull;
+        }
+        b->swl = sparse_ws_layout((int64_t)off, b->ntiles, count);
+        if (b->swl.bytes && hipMalloc(&b->ws, (size_t)b->swl.bytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
+    } else if (enc_ok && alg == HIPRESS_ONEBIT) {
+        if (hipMalloc(&b->ws, (size_t)round_up(4 * (int64_t)(b->ntiles ? b->ntiles : 1), 256)) != hipSuccess) return fail(HIPRESS_ERR_HIP);
+    }
+    if ((rc = upload(b->enc, &b->d_enc))) return fail(rc);
+    if ((rc = upload(b->dec, &b->d_dec))) return fail(rc);
+    if ((rc = upload(map, &b->d_map))) return fail(rc);
+    *out = b;
+    return HIPRESS_OK;
+}
+
+static Launch batch_launch(const hipress_batch* b, bool encode) {
+    Launch L;
+    std::memset(&L, 0, sizeof L);
+    L.single = false;
+    L.dsegs = encode ? b->d_enc : b->d_dec;
+    L.dmap = b->d_map;
+    L.ntiles = b->ntiles;
+    L.nsegs = (unsigned)(encode ? b->enc.size() : b->dec.size());
+    return L;
+}
+
+int hipress_batch_encode(hipress_batch* b, void* stream) {
+    if (!b) return HIPRESS_ERR_NULL;
+    if (!b->can_encode) return HIPRESS_ERR_NULL;
+    if (b->enc.empty()) return HIPRESS_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    Launch L = batch_launch(b, true);
+    switch (b->alg) {
+        case HIPRESS_ONEBIT: return hiperr(launch_onebit_encode(L, static_cast<float*>(b->ws), st));
+        case HIPRESS_TBQ: return hiperr(launch_tbq_encode(L, st));
+        case HIPRESS_TERNGRAD: return hiperr(launch_terngrad_encode(L, (unsigned)b->params.bucket, st));
+        case HIPRESS_DGC:
+        case HIPRESS_GRADDROP:
+            return hiperr(launch_sparse_encode(L, b->alg == HIPRESS_DGC, sparse_ws_at(b->ws, b->swl), st));
+    }
+    return HIPRESS_ERR_PARAM;
+}
+
+int hipress_batch_decode(hipress_batch* b, void* stream) {
+    if (!b) return HIPRESS_ERR_NULL;
+    if (!b->can_decode) return HIPRESS_ERR_NULL;
+    if (b->dec.empty()) return HIPRESS_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    Launch L = batch_launch(b, false);
+    switch (b->alg) {
+        case HIPRESS_ONEBIT: return hiperr(launch_onebit_decode(L, st));
+        case HIPRESS_TBQ: return hiperr(launch_tbq_decode(L, st));
+        case HIPRESS_TERNGRAD: return hiperr(launch_terngrad_decode(L, st));
+        case HIPRESS_DGC:
+        case HIPRESS_GRADDROP: return hiperr(launch_sparse_decode(L, st));
+    }
+    return HIPRESS_ERR_PARAM;
+}
+
+// ---- merge batches ---------------------------------------------------------------------
+
+int hipress_merge_batch_destroy(hipress_merge_batch* b) {
+    if (!b) return HIPRESS_OK;
+    (void)hipFree(b->d_segs);
+    (void)hipFree(b->d_renc);
+    (void)hipFree(b->d_map);
+    (void)hipFree(b->ws);
+    delete b;
+    return HIPRESS_OK;
+}
+
+int hipress_merge_batch_create(hipress_merge_batch** out, int32_t alg, const hipress_merge_chunk* chunks,
+                               int32_t count, int32_t npeers, const hipress_params* params) {
+    if (!out || !params || (count > 0 && !chunks)) return HIPRESS_ERR_NULL;
+    *out = nullptr;
+    if (count < 0) return HIPRESS_ERR_SIZE;
+    if (alg < HIPRESS_ONEBIT || alg > HIPRESS_GRADDROP) return HIPRESS_ERR_PARAM;
+    hipress_merge_batch* b = new (std::nothrow) hipress_merge_batch;
+    if (!b) return HIPRESS_ERR_HIP;
+    b->alg = alg;
+    b->params = *params;
+    b->npeers = npeers;
+    const bool sparse = alg == HIPRESS_DGC || alg == HIPRESS_GRADDROP;
+    auto fail = [&](int code) { hipress_merge_batch_destroy(b); return code; };
+    int rc;
+    bool any_state = false, all_state = true;
+    for (int i = 0; i < count; ++i) {
+        if (chunks[i].state) any_state = true;
+        else all_state = false;
+    }
+    if (any_state && !all_state) return fail(HIPRESS_ERR_NULL);  // re-encode is all chunks or none
+    if (any_state && (alg == HIPRESS_ONEBIT || alg == HIPRESS_TERNGRAD)) return fail(HIPRESS_ERR_PARAM);
+    b->reencode = any_state;
+    for (int i = 0; i < count; ++i) {
+        const hipress_merge_chunk& c = chunks[i];
+        MergeSeg m;
+        if ((rc = build_merge_seg(alg, c.payloads, c.payload_bytes, npeers, c.aggregate, c.n, &m))) return fail(rc);
+        if (b->reencode && alg == HIPRESS_TBQ) {
+            if ((rc = add_tbq_reencode(&m, c.state, c.out_payload, c.out_payload_bytes, params->threshold))) return fail(rc);
+        }
+        if (b->reencode && sparse) {
+            hipress_tensor t{c.aggregate, c.state, nullptr, nullptr, c.out_payload, nullptr, c.n, c.out_payload_bytes};
+            Seg s;
+            if ((rc = build_encode_seg(HIPRESS_GRADDROP, t, *params, &s))) return fail(rc);
+            b->renc.push_back(s);
+        }
+        b->segs.push_back(m);
+    }
+    std::vector<uint2> map;
+    if ((rc = layout_tiles(b->segs, [](MergeSeg& m) -> Seg& { return m.s; }, map, &b->ntiles))) return fail(rc);
+    if (!b->renc.empty()) {
+        std::vector<uint2> map2;
+        unsigned nt2;
+        if ((rc = layout_tiles(b->renc, [](Seg& s) -> Seg& { return s; }, map2, &nt2))) return fail(rc);
+        uint64_t off = 0;
+        for (Seg& s : b->renc) {
+            s.ws0 = off;
+            off += (s.ns + 3u) & ~3ull;
+        }
+        b->swl = sparse_ws_layout((int64_t)off, b->ntiles, count);
+        if (b->swl.bytes && hipMalloc(&b->ws, (size_t)b->swl.bytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
+    }
+    if ((rc = upload(b->segs, &b->d_segs))) return fail(rc);
+    if ((rc = upload(b->renc, &b->d_renc))) return fail(rc);
+    if ((rc = upload(map, &b->d_map))) return fail(rc);
+    *out = b;
+    return HIPRESS_OK;
+}
+
+int hipress_merge_batch_run(hipress_merge_batch* b, void* stream) {
+    if (!b) return HIPRESS_ERR_NULL;
+    if (b->segs.empty()) return HIPRESS_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    MergeLaunch L;
+    std::memset(&L, 0, sizeof L);
+    L.single = false;
+    L.dsegs = b->d_segs;
+    L.dmap = b->d_map;
+    L.ntiles = b->ntiles;
+    L.nsegs = (unsigned)b->segs.size();
+    L.npeers = b->npeers;
+    L.reencode = b->reencode;
+    if (b->alg == HIPRESS_DGC || b->alg == HIPRESS_GRADDROP) {
+        hipError_t e = launch_sparse_merge_scatter(L, st);
+        if (e != hipSuccess) return HIPRESS_ERR_HIP;
+        if (b->reencode) {
+            Launch R;
+            std::memset(&R, 0, sizeof R);
+            R.single = false;
+            R.dsegs = b->d_renc;
+            R.dmap = b->d_map;  // same tensors, same tile numbering
+            R.ntiles = b->ntiles;
+            R.nsegs = (unsigned)b->renc.size();
+            e = launch_sparse_encode(R, false, sparse_ws_at(b->ws, b->swl), st);
+        }
+        return hiperr(e);
+    }
+    return hiperr(launch_dense_merge(L, b->alg, st));
+}
+
+}  // extern "C"

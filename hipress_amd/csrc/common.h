@@ -1,0 +1,209 @@
+// Shared device/host definitions for the gfx950 gradient-compression kernels.
+//
+// Work decomposition used by every dense kernel: a tensor is cut into tiles of
+// kTile = 4096 consecutive elements; one 256-thread workgroup (four wave64
+// wavefronts) owns a tile, wavefront w owns the 1024 consecutive elements
+// [w*1024, +1024) of it, and in step j (0..3) lane l of that wavefront holds the
+// four elements at offset j*256 + 4*l as one 16-byte vector.  Every global
+// access of a wavefront is therefore one contiguous, fully used 1 KiB row, and
+// the 2-bit (1-bit) codes of four (eight) neighbouring lanes form one dense
+// uint32 word.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace hp {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+constexpr int kBlock = 256;       // threads per workgroup
+constexpr int kWaveTile = 1024;   // elements per wavefront per tile
+constexpr int kTile = 4096;       // elements per workgroup
+constexpr int kHeaderBytes = 16;
+constexpr int kMaxPeers = 16;
+
+// One tensor (or one chunk) as the kernels see it.  Batched launches index a
+// device-resident array of these through a tile map; single-tensor launches
+// carry one by value in the kernel arguments.
+struct Seg {
+    const float* g;    // gradient in
+    float* s0;         // residual (onebit, tbq) | momentum (dgc; NULL for graddrop)
+    float* s1;         // accumulator (dgc, graddrop)
+    const float* u;    // uniform noise (terngrad)
+    uint8_t* pay;      // payload base (header)
+    float* out;        // decode output / aggregate
+    unsigned long long n;
+    unsigned int tile0;      // index of this tensor's first tile among all tiles of the launch
+    unsigned int ntiles;     // tiles of this tensor
+    unsigned int words_off;  // byte offset of the packed words from the payload base
+    unsigned int bucket;     // terngrad bucket size
+    unsigned int aligned;    // 1 when every pointer used is 16-byte aligned
+    unsigned int cap;        // sparse capacity
+    float f0;                // tbq threshold | dgc momentum factor
+    unsigned int ks;         // sparse: rank of the threshold inside the sample
+    unsigned int sstride;    // sparse: sample stride
+    unsigned int ns;         // sparse: sample count
+    unsigned long long ws0;  // sparse: element offset of this tensor's sample slice
+    unsigned int id;         // index of this tensor in the launch's table
+    unsigned int pad0;
+    unsigned long long pay_bytes;  // size of the payload buffer (decode-side bounds checks)
+};
+
+// Peers of one chunk for decode-and-merge.
+struct MergeSeg {
+    const uint8_t* peer[kMaxPeers];
+    unsigned long long peer_bytes[kMaxPeers];  // size of each peer's buffer
+    unsigned int peer_slots[kMaxPeers];  // sparse: pairs each peer's buffer has room for
+    Seg s;  // out = aggregate, s0 = aggregator residual (tbq), pay = re-encoded payload
+};
+
+struct SingleSrc {
+    Seg seg;
+    __device__ __forceinline__ const Seg& get(unsigned& tile, unsigned blk) const {
+        tile = blk;
+        return seg;
+    }
+};
+
+struct BatchSrc {
+    const Seg* segs;
+    const uint2* map;  // per workgroup: {tensor index, tile index inside the tensor}
+    __device__ __forceinline__ const Seg& get(unsigned& tile, unsigned blk) const {
+        uint2 m = map[blk];
+        tile = m.y;
+        return segs[m.x];
+    }
+};
+
+// Per-tensor (not per-tile) launches: workgroup i works on tensor i.
+struct SingleSegSrc {
+    Seg seg;
+    __device__ __forceinline__ const Seg& at(unsigned) const { return seg; }
+};
+
+struct BatchSegSrc {
+    const Seg* segs;
+    __device__ __forceinline__ const Seg& at(unsigned i) const { return segs[i]; }
+};
+
+struct MergeSingleSrc {
+    MergeSeg seg;
+    __device__ __forceinline__ const MergeSeg& get(unsigned& tile, unsigned blk) const {
+        tile = blk;
+        return seg;
+    }
+};
+
+struct MergeBatchSrc {
+    const MergeSeg* segs;
+    const uint2* map;
+    __device__ __forceinline__ const MergeSeg& get(unsigned& tile, unsigned blk) const {
+        uint2 m = map[blk];
+        tile = m.y;
+        return segs[m.x];
+    }
+};
+
+#ifdef __HIPCC__
+// ---- memory access ---------------------------------------------------------
+// Streaming data is touched exactly once, so loads and stores carry the
+// non-temporal hint.
+__device__ __forceinline__ f4 ld4(const float* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const f4*>(p));
+}
+__device__ __forceinline__ void st4(float* p, f4 v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<f4*>(p));
+}
+// Element-wise variants for partial tiles and pointers that are only 4-byte aligned.
+__device__ __forceinline__ f4 ld4_guard(const float* p, long long e, long long n) {
+    f4 v = {0.f, 0.f, 0.f, 0.f};
+    if (e < n) v.x = p[e];
+    if (e + 1 < n) v.y = p[e + 1];
+    if (e + 2 < n) v.z = p[e + 2];
+    if (e + 3 < n) v.w = p[e + 3];
+    return v;
+}
+__device__ __forceinline__ void st4_guard(float* p, long long e, long long n, f4 v) {
+    if (e < n) p[e] = v.x;
+    if (e + 1 < n) p[e + 1] = v.y;
+    if (e + 2 < n) p[e + 2] = v.z;
+    if (e + 3 < n) p[e + 3] = v.w;
+}
+template <bool FAST>
+__device__ __forceinline__ f4 load4(const float* p, long long e, long long n) {
+    if (FAST) return ld4(p + e);
+    return ld4_guard(p, e, n);
+}
+template <bool FAST>
+__device__ __forceinline__ void store4(float* p, long long e, long long n, f4 v) {
+    if (FAST) st4(p + e, v);
+    else st4_guard(p, e, n, v);
+}
+// bit k set when element e+k exists
+__device__ __forceinline__ unsigned valid4(long long e, long long n) {
+    long long left = n - e;
+    return left >= 4 ? 0xfu : (left <= 0 ? 0u : ((1u << left) - 1u));
+}
+
+// ---- cross-lane -------------------------------------------------------------
+// quad_perm broadcast of lane k of every group of four lanes (DPP, no LDS traffic)
+template <int K>
+__device__ __forceinline__ unsigned quad_bcast(unsigned x) {
+    return (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, K * 0x55, 0xf, 0xf, false);
+}
+// Four neighbouring lanes each hold 8 bits; all four receive the 32-bit word
+// with lane (4q+k)'s byte at bits [8k, 8k+8).
+__device__ __forceinline__ unsigned quad_pack8(unsigned byte) {
+    return quad_bcast<0>(byte) | (quad_bcast<1>(byte) << 8) | (quad_bcast<2>(byte) << 16) |
+           (quad_bcast<3>(byte) << 24);
+}
+// Eight neighbouring lanes each hold 4 bits; all eight receive the word with
+// lane (8o+k)'s nibble at bits [4k, 4k+4).
+__device__ __forceinline__ unsigned oct_pack4(unsigned nib, unsigned lane) {
+    unsigned h = quad_bcast<0>(nib) | (quad_bcast<1>(nib) << 4) | (quad_bcast<2>(nib) << 8) |
+                 (quad_bcast<3>(nib) << 12);
+    unsigned o = (unsigned)__shfl_xor((int)h, 4, 64);
+    return (lane & 4u) ? (o | (h << 16)) : (h | (o << 16));
+}
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) x += __shfl_xor(x, m, 64);
+    return x;
+}
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        float y = __shfl_xor(x, m, 64);
+        x = y > x ? y : x;
+    }
+    return x;
+}
+__device__ __forceinline__ unsigned wave_sum_u(unsigned x) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) x += (unsigned)__shfl_xor((int)x, m, 64);
+    return x;
+}
+#endif  // __HIPCC__
+
+// ---- host-side launch description -----------------------------------------------
+struct Launch {
+    bool single;          // true: seg by value, grid = seg.ntiles
+    Seg seg;              // single
+    const Seg* dsegs;     // batch: device table
+    const uint2* dmap;    // batch: device tile map
+    unsigned ntiles;      // workgroups to launch
+    unsigned nsegs;       // tensors in the table (1 for single)
+};
+
+struct MergeLaunch {
+    bool single;
+    MergeSeg seg;
+    const MergeSeg* dsegs;
+    const uint2* dmap;
+    unsigned ntiles;
+    unsigned nsegs;
+    int npeers;
+    bool reencode;
+};
+
+}  // namespace hp

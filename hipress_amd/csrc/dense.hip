@@ -1,0 +1,559 @@
+// Dense quantisers for gfx950: TBQ, onebit and TernGrad encode/decode.
+// Every kernel is a streaming pass bounded by HBM bandwidth; see common.h for the
+// tile / wavefront / lane decomposition all of them share.
+#include "common.h"
+#include "launch.h"
+
+namespace hp {
+
+// =============================================================================
+// TBQ
+// =============================================================================
+
+// v -> code (0, 1 = +tau, 2 = -tau) and the residual that stays behind.
+__device__ __forceinline__ unsigned tbq_quant(float v, float tau, float& keep) {
+    unsigned c = v >= tau ? 1u : (v <= -tau ? 2u : 0u);
+    keep = c == 1u ? v - tau : (c == 2u ? v + tau : v);
+    return c;
+}
+
+__device__ __forceinline__ float code_value(unsigned c, float s) {
+    return c == 1u ? s : (c == 2u ? -s : 0.f);
+}
+
+// Quantises the four elements of one lane, returns their 8 code bits.
+template <bool FAST>
+__device__ __forceinline__ unsigned tbq_quant4(f4 v, float tau, unsigned valid, f4& keep) {
+    unsigned byte = 0;
+    float k;
+    unsigned c;
+    c = tbq_quant(v.x, tau, k); keep.x = k; byte |= c;
+    c = tbq_quant(v.y, tau, k); keep.y = k; byte |= c << 2;
+    c = tbq_quant(v.z, tau, k); keep.z = k; byte |= c << 4;
+    c = tbq_quant(v.w, tau, k); keep.w = k; byte |= c << 6;
+    if (!FAST) {  // elements past the end produce pad code 0
+        unsigned m = ((valid & 1u) * 0x03u) | ((valid >> 1 & 1u) * 0x0cu) | ((valid >> 2 & 1u) * 0x30u) |
+                     ((valid >> 3 & 1u) * 0xc0u);
+        byte &= m;
+    }
+    return byte;
+}
+
+// Shared tail of TBQ encode and of the fused re-encode in decode-and-merge:
+// v[j] are this lane's 16 values; writes residual and packed words.
+template <bool FAST>
+__device__ __forceinline__ void tbq_emit(const f4 (&v)[4], float tau, float* res, uint32_t* words,
+                                         long long wbase_elem, long long n, unsigned lane) {
+    unsigned myword = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = wbase_elem + j * 256 + lane * 4;
+        f4 keep;
+        unsigned byte = tbq_quant4<FAST>(v[j], tau, FAST ? 0xfu : valid4(e, n), keep);
+        store4<FAST>(res, e, n, keep);
+        unsigned w = quad_pack8(byte);
+        myword = ((lane & 3u) == (unsigned)j) ? w : myword;
+    }
+    // lane 4q+j holds the word of step j, quad q
+    long long widx = (wbase_elem >> 4) + (lane & 3u) * 16 + (lane >> 2);
+    if (FAST || widx < (long long)((n + 15) >> 4)) words[widx] = myword;
+}
+
+template <bool FAST>
+__device__ __forceinline__ void tbq_encode_tile(const Seg& s, unsigned tile) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    const float tau = s.f0;
+    f4 g[4], r[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        g[j] = load4<FAST>(s.g, e, n);
+        r[j] = load4<FAST>(s.s0, e, n);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) r[j] = r[j] + g[j];
+    tbq_emit<FAST>(r, tau, s.s0, reinterpret_cast<uint32_t*>(s.pay + kHeaderBytes), base, n, lane);
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void tbq_encode_kernel(Src src) {
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    if (tile == 0 && threadIdx.x == 0) {
+        uint32_t* h = reinterpret_cast<uint32_t*>(s.pay);
+        h[0] = __float_as_uint(s.f0);
+        h[1] = (uint32_t)s.n;
+        h[2] = 0;
+        h[3] = 0;
+    }
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) tbq_encode_tile<true>(s, tile);
+    else tbq_encode_tile<false>(s, tile);
+}
+
+// Expands the 8 code bits of one lane to four values of magnitude sc.
+__device__ __forceinline__ f4 expand2(unsigned byte, float sc) {
+    f4 o;
+    o.x = code_value(byte & 3u, sc);
+    o.y = code_value((byte >> 2) & 3u, sc);
+    o.z = code_value((byte >> 4) & 3u, sc);
+    o.w = code_value((byte >> 6) & 3u, sc);
+    return o;
+}
+
+// The byte of 2-bit codes that lane `lane` needs in step j of a wavefront whose
+// first element is wbase_elem (a multiple of 1024).
+template <bool FAST>
+__device__ __forceinline__ unsigned fetch_byte2(const uint32_t* words, long long wbase_elem, int j,
+                                                unsigned lane, long long nwords) {
+    long long widx = (wbase_elem >> 4) + j * 16 + (lane >> 2);
+    uint32_t w = (FAST || widx < nwords) ? words[widx] : 0u;
+    return (w >> (8 * (lane & 3u))) & 0xffu;
+}
+
+template <bool FAST>
+__device__ __forceinline__ void tbq_decode_tile(const Seg& s, unsigned tile) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    const uint32_t* words = reinterpret_cast<const uint32_t*>(s.pay + kHeaderBytes);
+    const float tau = *reinterpret_cast<const float*>(s.pay);
+    const long long nwords = (n + 15) >> 4;
+    unsigned b[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) b[j] = fetch_byte2<FAST>(words, base, j, lane, nwords);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) store4<FAST>(s.out, base + j * 256 + lane * 4, n, expand2(b[j], tau));
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void tbq_decode_kernel(Src src) {
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) tbq_decode_tile<true>(s, tile);
+    else tbq_decode_tile<false>(s, tile);
+}
+
+// =============================================================================
+// onebit
+// =============================================================================
+
+__device__ __forceinline__ float abs4sum(f4 v) {
+    return (fabsf(v.x) + fabsf(v.y)) + (fabsf(v.z) + fabsf(v.w));
+}
+
+// Pass 1: one partial sum of |r+g| per tile, in a fixed order (deterministic).
+template <bool FAST>
+__device__ __forceinline__ float onebit_abs_tile(const Seg& s, unsigned tile) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    f4 g[4], r[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        g[j] = load4<FAST>(s.g, e, n);
+        r[j] = load4<FAST>(s.s0, e, n);
+    }
+    float a = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) a += abs4sum(r[j] + g[j]);
+    return a;
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void onebit_abs_kernel(Src src, float* partial) {
+    __shared__ float wsum[4];
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    float a;
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) a = onebit_abs_tile<true>(s, tile);
+    else a = onebit_abs_tile<false>(s, tile);
+    a = wave_sum(a);
+    if ((threadIdx.x & 63u) == 0) wsum[threadIdx.x >> 6] = a;
+    __syncthreads();
+    if (threadIdx.x == 0) partial[s.tile0 + tile] = (wsum[0] + wsum[1]) + (wsum[2] + wsum[3]);
+}
+
+// Pass 2: one workgroup per tensor adds that tensor's partials in double, in a
+// fixed order, and writes the header {scale, n, 0, 0}.
+template <class Src>
+__global__ __launch_bounds__(kBlock) void onebit_scale_kernel(Src src, const float* partial) {
+    __shared__ double red[kBlock];
+    const Seg& s = src.at(blockIdx.x);
+    double a = 0.0;
+    for (unsigned t = threadIdx.x; t < s.ntiles; t += kBlock) a += (double)partial[s.tile0 + t];
+    red[threadIdx.x] = a;
+    __syncthreads();
+    for (int w = kBlock / 2; w >= 1; w >>= 1) {
+        if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        float sc = s.n ? (float)(red[0] / (double)s.n) : 0.f;
+        uint32_t* h = reinterpret_cast<uint32_t*>(s.pay);
+        h[0] = __float_as_uint(sc);
+        h[1] = (uint32_t)s.n;
+        h[2] = 0;
+        h[3] = 0;
+    }
+}
+
+template <bool FAST>
+__device__ __forceinline__ void onebit_quant_tile(const Seg& s, unsigned tile) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    const float sc = *reinterpret_cast<const float*>(s.pay);
+    uint32_t* words = reinterpret_cast<uint32_t*>(s.pay + kHeaderBytes);
+    f4 g[4], r[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        g[j] = load4<FAST>(s.g, e, n);
+        r[j] = load4<FAST>(s.s0, e, n);
+    }
+    unsigned myword = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        f4 v = r[j] + g[j];
+        unsigned b0 = v.x >= 0.f, b1 = v.y >= 0.f, b2 = v.z >= 0.f, b3 = v.w >= 0.f;
+        f4 keep;
+        keep.x = v.x - (b0 ? sc : -sc);
+        keep.y = v.y - (b1 ? sc : -sc);
+        keep.z = v.z - (b2 ? sc : -sc);
+        keep.w = v.w - (b3 ? sc : -sc);
+        unsigned nib = b0 | (b1 << 1) | (b2 << 2) | (b3 << 3);
+        if (!FAST) nib &= valid4(e, n);
+        store4<FAST>(s.s0, e, n, keep);
+        unsigned w = oct_pack4(nib, lane);
+        myword = ((lane & 7u) == (unsigned)j) ? w : myword;
+    }
+    // lane 8o+j (j < 4) holds the word of step j, octet o
+    long long widx = (base >> 5) + (lane & 7u) * 8 + (lane >> 3);
+    if ((lane & 7u) < 4u && (FAST || widx < (long long)((n + 31) >> 5))) words[widx] = myword;
+}
+
+// Tiles are walked from the end of each tensor towards its start: the pass that
+// summed |r+g| finished there, so the most recently read lines are still in cache.
+template <class Src>
+__global__ __launch_bounds__(kBlock) void onebit_quant_kernel(Src src) {
+    unsigned tile;
+    const Seg& s = src.get(tile, gridDim.x - 1 - blockIdx.x);
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) onebit_quant_tile<true>(s, tile);
+    else onebit_quant_tile<false>(s, tile);
+}
+
+template <bool FAST>
+__device__ __forceinline__ void onebit_decode_tile(const Seg& s, unsigned tile) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    const uint32_t* words = reinterpret_cast<const uint32_t*>(s.pay + kHeaderBytes);
+    const float sc = *reinterpret_cast<const float*>(s.pay);
+    const long long nwords = (n + 31) >> 5;
+    unsigned nib[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long widx = (base >> 5) + j * 8 + (lane >> 3);
+        uint32_t w = (FAST || widx < nwords) ? words[widx] : 0u;
+        nib[j] = (w >> (4 * (lane & 7u))) & 0xfu;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        f4 o;
+        o.x = (nib[j] & 1u) ? sc : -sc;
+        o.y = (nib[j] & 2u) ? sc : -sc;
+        o.z = (nib[j] & 4u) ? sc : -sc;
+        o.w = (nib[j] & 8u) ? sc : -sc;
+        store4<FAST>(s.out, base + j * 256 + lane * 4, n, o);
+    }
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void onebit_decode_kernel(Src src) {
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) onebit_decode_tile<true>(s, tile);
+    else onebit_decode_tile<false>(s, tile);
+}
+
+// =============================================================================
+// TernGrad
+// =============================================================================
+
+__device__ __forceinline__ float absmax4(f4 v) {
+    return fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+}
+
+__device__ __forceinline__ unsigned tern_code(float g, float u, float s) {
+    float t = u * s;
+    return t < fabsf(g) ? (g < 0.f ? 2u : 1u) : 0u;
+}
+
+__device__ __forceinline__ unsigned tern_code4(f4 g, f4 u, float s) {
+    return tern_code(g.x, u.x, s) | (tern_code(g.y, u.y, s) << 2) | (tern_code(g.z, u.z, s) << 4) |
+           (tern_code(g.w, u.w, s) << 6);
+}
+
+// Bucket sizes 256, 512 and 1024 divide a wavefront's 1024 elements, so the
+// bucket maximum is a wavefront reduction over values already in registers and
+// the whole encode is a single pass.  BPW = buckets per wavefront tile.
+template <bool FAST, int BPW>
+__device__ __forceinline__ void terngrad_encode_tile(const Seg& s, unsigned tile) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    if (base >= n) return;
+    float* scales = reinterpret_cast<float*>(s.pay + kHeaderBytes);
+    uint32_t* words = reinterpret_cast<uint32_t*>(s.pay + s.words_off);
+    f4 g[4], u[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        g[j] = load4<FAST>(s.g, e, n);
+        u[j] = load4<FAST>(s.u, e, n);
+    }
+    float sc[4];
+    constexpr int SPB = 4 / BPW;  // steps per bucket
+#pragma unroll
+    for (int b = 0; b < BPW; ++b) {
+        float m = 0.f;
+#pragma unroll
+        for (int k = 0; k < SPB; ++k) m = fmaxf(m, absmax4(g[b * SPB + k]));
+        m = wave_max(m);
+#pragma unroll
+        for (int k = 0; k < SPB; ++k) sc[b * SPB + k] = m;
+        long long bidx = (base / (256 * SPB)) + b;
+        if (lane == 0 && bidx * (256 * SPB) < n) scales[bidx] = m;
+    }
+    unsigned myword = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        unsigned byte = tern_code4(g[j], u[j], sc[j]);  // pad elements are 0: u*s < 0 is false
+        unsigned w = quad_pack8(byte);
+        myword = ((lane & 3u) == (unsigned)j) ? w : myword;
+    }
+    long long widx = (base >> 4) + (lane & 3u) * 16 + (lane >> 2);
+    if (FAST || widx < (long long)((n + 15) >> 4)) words[widx] = myword;
+}
+
+// The scale array is padded to 16 bytes; the pad entries are written as zero.
+__device__ __forceinline__ void terngrad_zero_scale_pad(const Seg& s, unsigned tile) {
+    if (tile == 0 && threadIdx.x < 4) {
+        unsigned long long nb = (s.n + s.bucket - 1) / s.bucket;
+        unsigned long long i = nb + threadIdx.x;
+        if (i < ((nb + 3) & ~3ull)) reinterpret_cast<float*>(s.pay + kHeaderBytes)[i] = 0.f;
+    }
+}
+
+template <class Src, int BPW>
+__global__ __launch_bounds__(kBlock) void terngrad_encode_kernel(Src src) {
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    if (tile == 0 && threadIdx.x == 0) {
+        uint32_t* h = reinterpret_cast<uint32_t*>(s.pay);
+        h[0] = (uint32_t)s.n;
+        h[1] = s.bucket;
+        h[2] = 0;
+        h[3] = 0;
+    }
+    terngrad_zero_scale_pad(s, tile);
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) terngrad_encode_tile<true, BPW>(s, tile);
+    else terngrad_encode_tile<false, BPW>(s, tile);
+}
+
+// Any other bucket size: one wavefront per bucket writes the scale ...
+template <class Src>
+__global__ __launch_bounds__(kBlock) void terngrad_scale_generic_kernel(Src src) {
+    // grid: tiles of the tensor; each workgroup walks the buckets that START in its tile
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n, B = s.bucket;
+    const long long lo = (long long)tile * kTile, hi = lo + kTile < n ? lo + kTile : n;
+    float* scales = reinterpret_cast<float*>(s.pay + kHeaderBytes);
+    if (tile == 0 && threadIdx.x == 0) {
+        uint32_t* h = reinterpret_cast<uint32_t*>(s.pay);
+        h[0] = (uint32_t)s.n;
+        h[1] = s.bucket;
+        h[2] = 0;
+        h[3] = 0;
+    }
+    terngrad_zero_scale_pad(s, tile);
+    long long first = (lo + B - 1) / B;  // first bucket starting at or after lo
+    for (long long b = first + wave; b * B < hi; b += 4) {
+        long long e0 = b * B, e1 = e0 + B < n ? e0 + B : n;
+        float m = 0.f;
+        for (long long e = e0 + lane; e < e1; e += 64) m = fmaxf(m, fabsf(s.g[e]));
+        m = wave_max(m);
+        if (lane == 0) scales[b] = m;
+    }
+}
+
+// ... and a second pass quantises with a per-element scale lookup.
+template <class Src>
+__global__ __launch_bounds__(kBlock) void terngrad_quant_generic_kernel(Src src) {
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n, B = s.bucket;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    const float* scales = reinterpret_cast<const float*>(s.pay + kHeaderBytes);
+    uint32_t* words = reinterpret_cast<uint32_t*>(s.pay + s.words_off);
+    unsigned myword = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        unsigned byte = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            long long i = e + k;
+            if (i < n) byte |= tern_code(s.g[i], s.u[i], scales[i / B]) << (2 * k);
+        }
+        unsigned w = quad_pack8(byte);
+        myword = ((lane & 3u) == (unsigned)j) ? w : myword;
+    }
+    long long widx = (base >> 4) + (lane & 3u) * 16 + (lane >> 2);
+    if (widx < (long long)((n + 15) >> 4)) words[widx] = myword;
+}
+
+// Decode.  The bucket size comes from the payload header, and with it the place
+// of the packed words behind the scale array; a header that does not fit the
+// buffer decodes to zeros.  BUCKET256 means the bucket size is a multiple of 256,
+// so one step of a wavefront (256 aligned elements) lies inside one bucket.
+template <bool FAST, bool BUCKET256>
+__device__ __forceinline__ void terngrad_decode_tile(const Seg& s, unsigned tile, long long B,
+                                                     const uint32_t* words) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    if (base >= n) return;
+    const float* scales = reinterpret_cast<const float*>(s.pay + kHeaderBytes);
+    const long long nwords = words ? (n + 15) >> 4 : 0;
+    unsigned b[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long widx = (base >> 4) + j * 16 + (lane >> 2);
+        uint32_t w = widx < nwords ? words[widx] : 0u;
+        b[j] = (w >> (8 * (lane & 3u))) & 0xffu;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        f4 o;
+        if (BUCKET256) {
+            long long e0 = base + j * 256;
+            float sc = (e0 < n && words) ? scales[e0 / B] : 0.f;
+            o = expand2(b[j], sc);
+        } else {
+            o.x = (e < n && b[j]) ? code_value(b[j] & 3u, scales[e / B]) : 0.f;
+            o.y = (e + 1 < n && b[j]) ? code_value((b[j] >> 2) & 3u, scales[(e + 1) / B]) : 0.f;
+            o.z = (e + 2 < n && b[j]) ? code_value((b[j] >> 4) & 3u, scales[(e + 2) / B]) : 0.f;
+            o.w = (e + 3 < n && b[j]) ? code_value((b[j] >> 6) & 3u, scales[(e + 3) / B]) : 0.f;
+        }
+        store4<FAST>(s.out, e, n, o);
+    }
+}
+
+// Where the packed words of a TernGrad payload start, or NULL when the header's
+// bucket size does not fit the buffer.
+__device__ __forceinline__ const uint32_t* terngrad_words(const uint8_t* pay, unsigned long long pay_bytes,
+                                                           unsigned long long n, long long& B) {
+    const uint32_t* h = reinterpret_cast<const uint32_t*>(pay);
+    B = h[1];
+    if (B < 1) { B = 1; return nullptr; }
+    unsigned long long nb = (n + B - 1) / B;
+    unsigned long long off = kHeaderBytes + ((4 * nb + 15) & ~15ull);
+    if (off + 4 * ((n + 15) >> 4) > pay_bytes) return nullptr;
+    return reinterpret_cast<const uint32_t*>(pay + off);
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void terngrad_decode_kernel(Src src) {
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    long long B;
+    const uint32_t* words = terngrad_words(s.pay, s.pay_bytes, s.n, B);
+    const bool fast = s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n;
+    const bool b256 = (B & 255) == 0;
+    if (fast && b256) terngrad_decode_tile<true, true>(s, tile, B, words);
+    else if (b256) terngrad_decode_tile<false, true>(s, tile, B, words);
+    else terngrad_decode_tile<false, false>(s, tile, B, words);
+}
+
+// =============================================================================
+// launchers
+// =============================================================================
+
+#define HP_LAUNCH(KERNEL, L, st, ...)                                                         \
+    do {                                                                                      \
+        if ((L).ntiles == 0) return hipSuccess;                                               \
+        if ((L).single) {                                                                     \
+            SingleSrc src{(L).seg};                                                           \
+            hipLaunchKernelGGL((KERNEL<SingleSrc>), dim3((L).ntiles), dim3(kBlock), 0, st, src, \
+                               ##__VA_ARGS__);                                                \
+        } else {                                                                              \
+            BatchSrc src{(L).dsegs, (L).dmap};                                                \
+            hipLaunchKernelGGL((KERNEL<BatchSrc>), dim3((L).ntiles), dim3(kBlock), 0, st, src, \
+                               ##__VA_ARGS__);                                                \
+        }                                                                                     \
+        return hipGetLastError();                                                             \
+    } while (0)
+
+hipError_t launch_tbq_encode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_encode_kernel, L, st); }
+hipError_t launch_tbq_decode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_decode_kernel, L, st); }
+hipError_t launch_onebit_decode(const Launch& L, hipStream_t st) { HP_LAUNCH(onebit_decode_kernel, L, st); }
+hipError_t launch_terngrad_decode(const Launch& L, hipStream_t st) { HP_LAUNCH(terngrad_decode_kernel, L, st); }
+
+static hipError_t onebit_abs(const Launch& L, float* partial, hipStream_t st) {
+    HP_LAUNCH(onebit_abs_kernel, L, st, partial);
+}
+static hipError_t onebit_quant(const Launch& L, hipStream_t st) { HP_LAUNCH(onebit_quant_kernel, L, st); }
+
+static hipError_t onebit_scale(const Launch& L, const float* partial, hipStream_t st) {
+    if (L.single) {
+        SingleSegSrc src{L.seg};
+        hipLaunchKernelGGL((onebit_scale_kernel<SingleSegSrc>), dim3(1), dim3(kBlock), 0, st, src, partial);
+    } else {
+        BatchSegSrc src{L.dsegs};
+        hipLaunchKernelGGL((onebit_scale_kernel<BatchSegSrc>), dim3(L.nsegs), dim3(kBlock), 0, st, src, partial);
+    }
+    return hipGetLastError();
+}
+
+// partial: one float per tile of the launch
+hipError_t launch_onebit_encode(const Launch& L, float* partial, hipStream_t st) {
+    hipError_t e;
+    if (L.ntiles) {
+        if ((e = onebit_abs(L, partial, st)) != hipSuccess) return e;
+    }
+    if ((e = onebit_scale(L, partial, st)) != hipSuccess) return e;  // also writes headers of empty tensors
+    if (L.ntiles) {
+        if ((e = onebit_quant(L, st)) != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+template <class Src>
+static hipError_t terngrad_encode_src(const Src& src, unsigned ntiles, unsigned bucket, hipStream_t st) {
+    if (bucket == 256) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 4>), dim3(ntiles), dim3(kBlock), 0, st, src);
+    else if (bucket == 512) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 2>), dim3(ntiles), dim3(kBlock), 0, st, src);
+    else if (bucket == 1024) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 1>), dim3(ntiles), dim3(kBlock), 0, st, src);
+    else {
+        hipLaunchKernelGGL((terngrad_scale_generic_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);
+        hipLaunchKernelGGL((terngrad_quant_generic_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);
+    }
+    return hipGetLastError();
+}
+
+// All tensors of one launch share the bucket size.
+hipError_t launch_terngrad_encode(const Launch& L, unsigned bucket, hipStream_t st) {
+    if (L.ntiles == 0) return hipSuccess;
+    if (L.single) return terngrad_encode_src(SingleSrc{L.seg}, L.ntiles, bucket, st);
+    return terngrad_encode_src(BatchSrc{L.dsegs, L.dmap}, L.ntiles, bucket, st);
+}
+
+}  // namespace hp

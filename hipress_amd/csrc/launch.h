@@ -1,0 +1,28 @@
+// Host-callable launchers; each one only enqueues kernels on the given stream.
+#pragma once
+#include "common.h"
+
+namespace hp {
+
+hipError_t launch_tbq_encode(const Launch& L, hipStream_t st);
+hipError_t launch_tbq_decode(const Launch& L, hipStream_t st);
+hipError_t launch_onebit_encode(const Launch& L, float* partial, hipStream_t st);
+hipError_t launch_onebit_decode(const Launch& L, hipStream_t st);
+hipError_t launch_terngrad_encode(const Launch& L, unsigned bucket, hipStream_t st);
+hipError_t launch_terngrad_decode(const Launch& L, hipStream_t st);
+
+// Dense decode-and-merge; alg is a hipress_alg value (onebit, tbq, terngrad).
+hipError_t launch_dense_merge(const MergeLaunch& L, int alg, hipStream_t st);
+
+// Sparse (DGC / GradDrop) pipeline.  ws is the launch's workspace.
+struct SparseWs {
+    uint32_t* sample;   // |acc'| keys at the sample positions, all tensors back to back
+    uint32_t* gmax;     // max |acc'| key of every 64-element group: 64 per tile
+    uint32_t* counts;   // per wavefront-tile {above, equal} counts, then their exclusive scans
+    uint32_t* thr;      // per tensor {threshold key, equal-quota}
+};
+hipError_t launch_sparse_encode(const Launch& L, bool dgc, const SparseWs& ws, hipStream_t st);
+hipError_t launch_sparse_decode(const Launch& L, hipStream_t st);
+hipError_t launch_sparse_merge_scatter(const MergeLaunch& L, hipStream_t st);
+
+}  // namespace hp

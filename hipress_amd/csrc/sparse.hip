@@ -1,0 +1,491 @@
+// Sampled-threshold sparsifiers for gfx950: DGC and GradDrop encode, the shared
+// sparse decode, and the scatter-add half of sparse decode-and-merge.
+//
+// Encode is five launches over the whole tensor set:
+//   1. accumulate   one streaming pass: mom' = m*mom + g, acc' = acc + mom'
+//                   (GradDrop: acc' = acc + g), written back; the |acc'| keys at
+//                   the sample positions are gathered and the maximum key of
+//                   every 64-element group is recorded on the way;
+//   2. threshold    one workgroup per tensor selects the k-th largest sample key;
+//   3. count        only groups whose maximum reaches the threshold are read
+//                   again; per wavefront-tile counts of keys above / equal to it;
+//   4. scan         one workgroup per tensor turns the counts into output
+//                   offsets, writes the header and, if more than `capacity`
+//                   elements qualify, re-thresholds on the whole tensor;
+//   5. emit         the flagged groups are read once more and the selected
+//                   (index, value) pairs are written in ascending index order,
+//                   the accumulator (and momentum) being zeroed at those places.
+// |x| is handled as the integer key bits(x) & 0x7fffffff, which orders like |x|.
+#include "common.h"
+#include "launch.h"
+
+namespace hp {
+
+constexpr unsigned kNoQuota = 0xffffffffu;
+
+__device__ __forceinline__ unsigned key_of(float x) { return __float_as_uint(x) & 0x7fffffffu; }
+
+__device__ __forceinline__ unsigned umax(unsigned a, unsigned b) { return a > b ? a : b; }
+
+// max over the 16 lanes of a DPP row; every lane of the row gets the result
+__device__ __forceinline__ unsigned row_max16(unsigned x) {
+    x = umax(x, (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+    x = umax(x, (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+    x = umax(x, (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x141, 0xf, 0xf, false));  // row_half_mirror
+    x = umax(x, (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x140, 0xf, 0xf, false));  // row_mirror
+    return x;
+}
+
+__device__ __forceinline__ unsigned popc_lt(unsigned long long m, unsigned lane) {
+    return __popcll(m & ((1ull << lane) - 1ull));
+}
+
+// ---- 1. accumulate -------------------------------------------------------------
+
+template <bool FAST, bool DGC>
+__device__ __forceinline__ void sparse_accum_tile(const Seg& s, unsigned tile, const SparseWs& ws) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    const float mf = s.f0;
+    uint32_t* sample = ws.sample + s.ws0;
+    f4 g[4], a[4], m[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        g[j] = load4<FAST>(s.g, e, n);
+        a[j] = load4<FAST>(s.s1, e, n);
+        if (DGC) m[j] = load4<FAST>(s.s0, e, n);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        f4 acc;
+        if (DGC) {
+            f4 mm;  // a rounded product, then a rounded sum: never a fused multiply-add
+            mm.x = __fadd_rn(__fmul_rn(mf, m[j].x), g[j].x);
+            mm.y = __fadd_rn(__fmul_rn(mf, m[j].y), g[j].y);
+            mm.z = __fadd_rn(__fmul_rn(mf, m[j].z), g[j].z);
+            mm.w = __fadd_rn(__fmul_rn(mf, m[j].w), g[j].w);
+            store4<FAST>(s.s0, e, n, mm);
+            acc = a[j] + mm;
+        } else {
+            acc = a[j] + g[j];
+        }
+        store4<FAST>(s.s1, e, n, acc);
+        unsigned k0 = key_of(acc.x), k1 = key_of(acc.y), k2 = key_of(acc.z), k3 = key_of(acc.w);
+        if (!FAST) {
+            unsigned v = valid4(e, n);
+            k0 = (v & 1u) ? k0 : 0u;
+            k1 = (v & 2u) ? k1 : 0u;
+            k2 = (v & 4u) ? k2 : 0u;
+            k3 = (v & 8u) ? k3 : 0u;
+        }
+        unsigned gm = row_max16(umax(umax(k0, k1), umax(k2, k3)));
+        if ((lane & 15u) == 0)
+            ws.gmax[(unsigned long long)(s.tile0 + tile) * 64 + wave * 16 + j * 4 + (lane >> 4)] = gm;
+        if (s.sstride == 1) {  // small tensor: every element is a sample
+            if (e < n) sample[e] = k0;
+            if (e + 1 < n) sample[e + 1] = k1;
+            if (e + 2 < n) sample[e + 2] = k2;
+            if (e + 3 < n) sample[e + 3] = k3;
+        } else {  // sample positions are q*S + S/2; at most one falls into [e, e+4)
+            const unsigned long long S = s.sstride, h = S / 2;
+            unsigned long long q = ((unsigned long long)e + (S - 1 - h)) / S;  // first q with q*S+h >= e
+            unsigned long long p = q * S + h;
+            if (p < (unsigned long long)e + 4 && q < s.ns) {
+                unsigned d = (unsigned)(p - (unsigned long long)e);
+                sample[q] = d == 0 ? k0 : (d == 1 ? k1 : (d == 2 ? k2 : k3));
+            }
+        }
+    }
+}
+
+template <class Src, bool DGC>
+__global__ __launch_bounds__(kBlock) void sparse_accum_kernel(Src src, SparseWs ws) {
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) sparse_accum_tile<true, DGC>(s, tile, ws);
+    else sparse_accum_tile<false, DGC>(s, tile, ws);
+}
+
+// ---- radix selection helper (one workgroup) ----------------------------------------
+
+// Finds the k-th largest (k >= 1) key among the keys a workgroup enumerates with
+// `visit(f)` (which must call f(key) for every candidate, the same set each time
+// it is invoked).  8-bit digits from the top; 16 interleaved histograms keep the
+// LDS atomics of neighbouring lanes apart.
+struct RadixScratch {
+    unsigned hist[16][257];
+    unsigned prefix, k;
+};
+
+template <class Visit>
+__device__ __forceinline__ unsigned block_kth_largest(RadixScratch& sc, unsigned k, Visit visit) {
+    unsigned prefix = 0, mask = 0;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        for (unsigned i = threadIdx.x; i < 16 * 257; i += kBlock) (&sc.hist[0][0])[i] = 0;
+        __syncthreads();
+        visit([&](unsigned key) {
+            if ((key & mask) == prefix) atomicAdd(&sc.hist[threadIdx.x & 15u][(key >> shift) & 255u], 1u);
+        });
+        __syncthreads();
+        // fold the 16 copies
+        {
+            unsigned t = threadIdx.x;  // kBlock == 256 bins
+            unsigned c = 0;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) c += sc.hist[r][t];
+            __syncthreads();
+            sc.hist[0][t] = c;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            unsigned kk = k;
+            int d = 255;
+            for (; d > 0; --d) {
+                unsigned c = sc.hist[0][d];
+                if (kk <= c) break;
+                kk -= c;
+            }
+            sc.prefix = prefix | ((unsigned)d << shift);
+            sc.k = kk;
+        }
+        __syncthreads();
+        prefix = sc.prefix;
+        k = sc.k;
+        mask |= 0xffu << shift;
+        __syncthreads();
+    }
+    return prefix;
+}
+
+// ---- 2. threshold ----------------------------------------------------------------
+
+template <class SegSrc>
+__global__ __launch_bounds__(kBlock) void sparse_threshold_kernel(SegSrc src, SparseWs ws) {
+    __shared__ RadixScratch sc;
+    const Seg& s = src.at(blockIdx.x);
+    const uint32_t* keys = ws.sample + s.ws0;
+    const unsigned ns = s.ns;
+    unsigned thr = 0;
+    if (ns > 0) {
+        thr = block_kth_largest(sc, s.ks, [&](auto f) {
+            for (unsigned i = threadIdx.x; i < ns; i += kBlock) f(keys[i]);
+        });
+    }
+    if (threadIdx.x == 0) {
+        ws.thr[2 * s.id] = thr;
+        ws.thr[2 * s.id + 1] = kNoQuota;
+    }
+}
+
+// ---- 3. count ---------------------------------------------------------------------
+
+// Counts, for the wavefront-tile wt (1024 elements) of tensor s, the keys above
+// and equal to thr; only 64-element groups whose maximum reaches thr are read.
+// Wavefront-uniform result.
+__device__ __forceinline__ void count_wavetile(const Seg& s, const SparseWs& ws, unsigned long long wt,
+                                               unsigned thr, unsigned lane, unsigned& gt, unsigned& eq) {
+    const long long n = (long long)s.n;
+    const unsigned long long g0 = (unsigned long long)s.tile0 * 64 + wt * 16;
+    unsigned gm = lane < 16 ? ws.gmax[g0 + lane] : 0u;
+    unsigned long long mask = __ballot(gm >= thr && gm > 0u);
+    gt = 0;
+    eq = 0;
+    while (mask) {
+        unsigned gi = __ffsll((long long)mask) - 1;
+        mask &= mask - 1;
+        long long e = (long long)wt * kWaveTile + gi * 64 + lane;
+        unsigned key = e < n ? key_of(s.s1[e]) : 0u;
+        gt += __popcll(__ballot(key > thr));
+        eq += __popcll(__ballot(key == thr && key > 0u));
+    }
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void sparse_count_kernel(Src src, SparseWs ws) {
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned thr = ws.thr[2 * s.id];
+    unsigned gt, eq;
+    const unsigned long long wt = (unsigned long long)tile * 4 + wave;
+    count_wavetile(s, ws, wt, thr, lane, gt, eq);
+    if (lane == 0) {
+        unsigned long long c = ((unsigned long long)s.tile0 * 4 + wt) * 2;
+        ws.counts[c] = gt;
+        ws.counts[c + 1] = eq;
+    }
+}
+
+// ---- 4. scan ----------------------------------------------------------------------
+
+// In-place exclusive scan of nw {above, equal} pairs by one workgroup; returns
+// the totals to every thread.
+__device__ __forceinline__ void block_scan_pairs(uint32_t* c, unsigned nw, unsigned (&sh)[2][kBlock],
+                                                 unsigned& tot_gt, unsigned& tot_eq) {
+    const unsigned t = threadIdx.x;
+    const unsigned per = (nw + kBlock - 1) / kBlock;
+    const unsigned lo = t * per, hi = lo + per < nw ? lo + per : nw;
+    unsigned sg = 0, se = 0;
+    for (unsigned i = lo; i < hi; ++i) {
+        sg += c[2 * i];
+        se += c[2 * i + 1];
+    }
+    sh[0][t] = sg;
+    sh[1][t] = se;
+    __syncthreads();
+    // Hillis-Steele inclusive scan over the 256 thread sums
+    for (int d = 1; d < kBlock; d <<= 1) {
+        unsigned ag = 0, ae = 0;
+        if ((int)t >= d) {
+            ag = sh[0][t - d];
+            ae = sh[1][t - d];
+        }
+        __syncthreads();
+        sh[0][t] += ag;
+        sh[1][t] += ae;
+        __syncthreads();
+    }
+    tot_gt = sh[0][kBlock - 1];
+    tot_eq = sh[1][kBlock - 1];
+    unsigned og = sh[0][t] - sg, oe = sh[1][t] - se;  // exclusive offsets of this thread's chunk
+    for (unsigned i = lo; i < hi; ++i) {
+        unsigned cg = c[2 * i], ce = c[2 * i + 1];
+        c[2 * i] = og;
+        c[2 * i + 1] = oe;
+        og += cg;
+        oe += ce;
+    }
+    __syncthreads();
+}
+
+template <class SegSrc>
+__global__ __launch_bounds__(kBlock) void sparse_scan_kernel(SegSrc src, SparseWs ws) {
+    __shared__ unsigned sh[2][kBlock];
+    __shared__ RadixScratch sc;
+    const Seg& s = src.at(blockIdx.x);
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned nw = s.ntiles * 4;
+    uint32_t* c = ws.counts + (unsigned long long)s.tile0 * 8;
+    unsigned thr = ws.thr[2 * s.id];
+    unsigned quota = kNoQuota;
+    unsigned tot_gt, tot_eq;
+    block_scan_pairs(c, nw, sh, tot_gt, tot_eq);
+    unsigned long long total = (unsigned long long)tot_gt + tot_eq;
+    if (total > s.cap) {
+        // More candidates than slots: the threshold becomes the capacity-th largest
+        // key of the whole tensor (all of those keys are >= the sampled threshold,
+        // hence inside flagged groups); ties at the new threshold are taken in
+        // ascending index order until the slots are full.
+        const unsigned old = thr;
+        const long long n = (long long)s.n;
+        const unsigned long long ngroups = (unsigned long long)s.ntiles * 64;
+        const uint32_t* gmax = ws.gmax + (unsigned long long)s.tile0 * 64;
+        thr = block_kth_largest(sc, s.cap, [&](auto f) {
+            for (unsigned long long g = wave; g < ngroups; g += 4) {
+                unsigned gm = gmax[g];
+                if (gm >= old && gm > 0u) {
+                    long long e = (long long)g * 64 + lane;
+                    unsigned key = e < n ? key_of(s.s1[e]) : 0u;
+                    if (key >= old && key > 0u) f(key);
+                }
+            }
+        });
+        for (unsigned long long wt = wave; wt < nw; wt += 4) {
+            unsigned gt, eq;
+            count_wavetile(s, ws, wt, thr, lane, gt, eq);
+            if (lane == 0) {
+                c[2 * wt] = gt;
+                c[2 * wt + 1] = eq;
+            }
+        }
+        __syncthreads();
+        block_scan_pairs(c, nw, sh, tot_gt, tot_eq);
+        quota = s.cap - tot_gt;
+        total = s.cap;
+    }
+    if (threadIdx.x == 0) {
+        ws.thr[2 * s.id] = thr;
+        ws.thr[2 * s.id + 1] = quota;
+        uint32_t* h = reinterpret_cast<uint32_t*>(s.pay);
+        h[0] = (uint32_t)total;
+        h[1] = (uint32_t)s.n;
+        h[2] = s.cap;
+        h[3] = thr;  // bit pattern of the threshold value
+    }
+}
+
+// ---- 5. emit ----------------------------------------------------------------------
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void sparse_emit_kernel(Src src, SparseWs ws) {
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const unsigned thr = ws.thr[2 * s.id], quota = ws.thr[2 * s.id + 1];
+    const unsigned long long wt = (unsigned long long)tile * 4 + wave;
+    const unsigned long long ci = ((unsigned long long)s.tile0 * 4 + wt) * 2;
+    const unsigned G = ws.counts[ci], E = ws.counts[ci + 1];
+    unsigned pos = G + (E < quota ? E : quota);  // pairs written by earlier wavefront-tiles
+    unsigned eq_seen = E;
+    int32_t* idx = reinterpret_cast<int32_t*>(s.pay + kHeaderBytes);
+    float* val = reinterpret_cast<float*>(s.pay + kHeaderBytes + 4ull * s.cap);
+    const unsigned long long g0 = (unsigned long long)s.tile0 * 64 + wt * 16;
+    unsigned gm = lane < 16 ? ws.gmax[g0 + lane] : 0u;
+    unsigned long long mask = __ballot(gm >= thr && gm > 0u);
+    while (mask) {
+        unsigned gi = __ffsll((long long)mask) - 1;
+        mask &= mask - 1;
+        long long e = (long long)wt * kWaveTile + gi * 64 + lane;
+        float v = e < n ? s.s1[e] : 0.f;
+        unsigned key = key_of(v);
+        bool is_eq = key == thr && key > 0u;
+        unsigned long long m_eq = __ballot(is_eq);
+        bool sel = key > thr || (is_eq && eq_seen + popc_lt(m_eq, lane) < quota);
+        unsigned long long m_sel = __ballot(sel);
+        if (sel) {
+            unsigned p = pos + popc_lt(m_sel, lane);
+            if (p < s.cap) {
+                idx[p] = (int32_t)e;
+                val[p] = v;
+                s.s1[e] = 0.f;
+                if (s.s0) s.s0[e] = 0.f;
+            }
+        }
+        pos += __popcll(m_sel);
+        eq_seen += __popcll(m_eq);
+    }
+}
+
+// ---- decode: zero fill + scatter ------------------------------------------------------
+
+template <bool FAST>
+__device__ __forceinline__ void zero_tile(float* out, long long n, unsigned tile) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    const f4 z = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) store4<FAST>(out, base + j * 256 + lane * 4, n, z);
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void zero_fill_kernel(Src src) {
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) zero_tile<true>(s.out, (long long)s.n, tile);
+    else zero_tile<false>(s.out, (long long)s.n, tile);
+}
+
+// Reads the header of a sparse payload that has room for `slots` pairs; returns
+// the number of usable pairs (0 when the header does not fit the buffer).
+__device__ __forceinline__ unsigned sparse_header(const uint8_t* pay, unsigned slots, const int32_t*& idx,
+                                                  const float*& val) {
+    const uint32_t* h = reinterpret_cast<const uint32_t*>(pay);
+    unsigned nnz = h[0], cap = h[2];
+    if (cap > slots) return 0;
+    idx = reinterpret_cast<const int32_t*>(pay + kHeaderBytes);
+    val = reinterpret_cast<const float*>(pay + kHeaderBytes + 4ull * cap);
+    return nnz < cap ? nnz : cap;
+}
+
+// The slots of a tensor are dealt out evenly over that tensor's tiles.
+template <class Src>
+__global__ __launch_bounds__(kBlock) void sparse_scatter_kernel(Src src) {
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    const int32_t* idx;
+    const float* val;
+    const unsigned nnz = sparse_header(s.pay, s.cap, idx, val);
+    const unsigned per = (s.cap + s.ntiles - 1) / s.ntiles;
+    const unsigned long long lo = (unsigned long long)tile * per;
+    unsigned long long hi = lo + per;
+    if (hi > nnz) hi = nnz;
+    for (unsigned long long j = lo + threadIdx.x; j < hi; j += kBlock) {
+        long long i = idx[j];
+        if (i >= 0 && i < (long long)s.n) s.out[i] = val[j];
+    }
+}
+
+// Scatter-ADD of every peer of a chunk into its (already zeroed) aggregate.
+template <class MSrc>
+__global__ __launch_bounds__(kBlock) void sparse_scatter_add_kernel(MSrc src, int npeers) {
+    unsigned tile;
+    const MergeSeg& m = src.get(tile, blockIdx.x);
+    for (int p = 0; p < npeers; ++p) {
+        const int32_t* idx;
+        const float* val;
+        const unsigned slots = m.peer_slots[p];
+        const unsigned nnz = sparse_header(m.peer[p], slots, idx, val);
+        const unsigned per = (slots + m.s.ntiles - 1) / m.s.ntiles;
+        const unsigned long long lo = (unsigned long long)tile * per;
+        unsigned long long hi = lo + per;
+        if (hi > nnz) hi = nnz;
+        for (unsigned long long j = lo + threadIdx.x; j < hi; j += kBlock) {
+            long long i = idx[j];
+            if (i >= 0 && i < (long long)m.s.n) atomicAdd(&m.s.out[i], val[j]);
+        }
+    }
+}
+
+template <class MSrc>
+__global__ __launch_bounds__(kBlock) void merge_zero_fill_kernel(MSrc src) {
+    unsigned tile;
+    const MergeSeg& m = src.get(tile, blockIdx.x);
+    if (m.s.aligned && (unsigned long long)(tile + 1) * kTile <= m.s.n) zero_tile<true>(m.s.out, (long long)m.s.n, tile);
+    else zero_tile<false>(m.s.out, (long long)m.s.n, tile);
+}
+
+// =============================================================================
+// launchers
+// =============================================================================
+
+template <class Src, class SegSrcT>
+static hipError_t sparse_encode_src(const Src& src, const SegSrcT& ssrc, unsigned ntiles, unsigned nsegs,
+                                    bool dgc, const SparseWs& ws, hipStream_t st) {
+    if (dgc) hipLaunchKernelGGL((sparse_accum_kernel<Src, true>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
+    else hipLaunchKernelGGL((sparse_accum_kernel<Src, false>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
+    hipLaunchKernelGGL((sparse_threshold_kernel<SegSrcT>), dim3(nsegs), dim3(kBlock), 0, st, ssrc, ws);
+    hipLaunchKernelGGL((sparse_count_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
+    hipLaunchKernelGGL((sparse_scan_kernel<SegSrcT>), dim3(nsegs), dim3(kBlock), 0, st, ssrc, ws);
+    hipLaunchKernelGGL((sparse_emit_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
+    return hipGetLastError();
+}
+
+hipError_t launch_sparse_encode(const Launch& L, bool dgc, const SparseWs& ws, hipStream_t st) {
+    if (L.ntiles == 0) return hipSuccess;
+    if (L.single) return sparse_encode_src(SingleSrc{L.seg}, SingleSegSrc{L.seg}, L.ntiles, 1, dgc, ws, st);
+    return sparse_encode_src(BatchSrc{L.dsegs, L.dmap}, BatchSegSrc{L.dsegs}, L.ntiles, L.nsegs, dgc, ws, st);
+}
+
+hipError_t launch_sparse_decode(const Launch& L, hipStream_t st) {
+    if (L.ntiles == 0) return hipSuccess;
+    if (L.single) {
+        SingleSrc src{L.seg};
+        hipLaunchKernelGGL((zero_fill_kernel<SingleSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
+        hipLaunchKernelGGL((sparse_scatter_kernel<SingleSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
+    } else {
+        BatchSrc src{L.dsegs, L.dmap};
+        hipLaunchKernelGGL((zero_fill_kernel<BatchSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
+        hipLaunchKernelGGL((sparse_scatter_kernel<BatchSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_sparse_merge_scatter(const MergeLaunch& L, hipStream_t st) {
+    if (L.ntiles == 0) return hipSuccess;
+    if (L.single) {
+        MergeSingleSrc src{L.seg};
+        hipLaunchKernelGGL((merge_zero_fill_kernel<MergeSingleSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
+        hipLaunchKernelGGL((sparse_scatter_add_kernel<MergeSingleSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src, L.npeers);
+    } else {
+        MergeBatchSrc src{L.dsegs, L.dmap};
+        hipLaunchKernelGGL((merge_zero_fill_kernel<MergeBatchSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
+        hipLaunchKernelGGL((sparse_scatter_add_kernel<MergeBatchSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src, L.npeers);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace hp

@@ -1,0 +1,436 @@
+"""In-place PyTorch operators over the C ABI.
+
+The surface follows the reference's operator convention
+(/root/reference/src/CompLL/GCGen/output/TernGradEncode/TernGradEncode.cc:10-24,
+ /root/reference/src/CompLL/GCGen/output/TernGradDecode/TernGradDecode.cc:10-24):
+encode takes ``(gradient, [state...], compressed, *scalars)``, decode takes
+``(compressed, gradient)``; every buffer is allocated by the caller, updated in
+place, and nothing is returned.  ``gradient`` must be float32 and ``compressed``
+uint8, the two type checks the reference makes
+(TernGradEncode_wrapper.h:35-38); here a violation raises ``TypeError`` instead
+of aborting the process.
+
+Operator names are ``<alg>_encode`` / ``<alg>_decode`` / ``<alg>_decode_merge``
+for the algorithm tokens the reference's launch lines use (onebit, tbq,
+terngrad, dgc, graddrop; /root/reference/README.md:9,45,160,276), with
+CompLL-style aliases (``TernGradEncode`` ...: TernGradEncode.cc:10) kept in
+``ALIASES``.  All of them are also registered as ``torch.ops.hipress.<name>``.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import ALG_IDS, MAX_PEERS, MergeChunk, Params, Tensor, check, size
+
+__all__ = [
+    "onebit_payload_bytes", "tbq_payload_bytes", "terngrad_payload_bytes", "sparse_capacity",
+    "sparse_payload_bytes", "dgc_payload_bytes", "graddrop_payload_bytes",
+    "onebit_encode", "onebit_decode", "tbq_encode", "tbq_decode", "terngrad_encode", "terngrad_decode",
+    "dgc_encode", "dgc_decode", "graddrop_encode", "graddrop_decode",
+    "onebit_decode_merge", "tbq_decode_merge", "terngrad_decode_merge", "dgc_decode_merge",
+    "graddrop_decode_merge", "Batch", "MergeBatch", "ALIASES",
+]
+
+
+# ---------------------------------------------------------------- sizes
+def onebit_payload_bytes(n):
+    return size(_lib.lib().hipress_onebit_payload_bytes(n), "onebit_payload_bytes")
+
+
+def tbq_payload_bytes(n):
+    return size(_lib.lib().hipress_tbq_payload_bytes(n), "tbq_payload_bytes")
+
+
+def terngrad_payload_bytes(n, bucket=512):
+    return size(_lib.lib().hipress_terngrad_payload_bytes(n, bucket), "terngrad_payload_bytes")
+
+
+def sparse_capacity(n, ratio):
+    return size(_lib.lib().hipress_sparse_capacity(n, ratio), "sparse_capacity")
+
+
+def sparse_payload_bytes(n, ratio):
+    return size(_lib.lib().hipress_sparse_payload_bytes(n, ratio), "sparse_payload_bytes")
+
+
+dgc_payload_bytes = sparse_payload_bytes
+graddrop_payload_bytes = sparse_payload_bytes
+
+
+# ---------------------------------------------------------------- argument checks
+def _f32(t, name, like=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if t.dtype != torch.float32:
+        raise TypeError(f"type of {name} should be float")
+    _common(t, name, like)
+    return t
+
+
+def _u8(t, name, like=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if t.dtype != torch.uint8:
+        raise TypeError(f"type of {name} should be uint8")
+    _common(t, name, like)
+    return t
+
+
+def _common(t, name, like):
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (hipress_amd has no CPU path)")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if like is not None:
+        if t.device != like.device:
+            raise ValueError(f"{name} is on {t.device}, expected {like.device}")
+
+
+def _same_numel(a, b, na, nb):
+    if a.numel() != b.numel():
+        raise ValueError(f"{na} has {a.numel()} elements, {nb} has {b.numel()}")
+
+
+def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+_workspaces = {}
+
+
+def _workspace(t, nbytes):
+    """Scratch buffer per (device, stream), grown on demand and reused."""
+    key = (t.device.index, _stream(t))
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(int(nbytes), 1 << 16), dtype=torch.uint8, device=t.device)
+        _workspaces[key] = ws
+    return ws
+
+
+def _p(t):
+    return t.data_ptr() if t is not None else None
+
+
+# ---------------------------------------------------------------- TBQ
+def tbq_encode(gradient, residual, compressed, threshold):
+    """Threshold two-bit quantisation with error feedback; residual is updated in place."""
+    _f32(gradient, "gradient"); _f32(residual, "residual", gradient); _u8(compressed, "compressed", gradient)
+    _same_numel(gradient, residual, "gradient", "residual")
+    with torch.cuda.device(gradient.device):
+        check(_lib.lib().hipress_tbq_encode(_p(gradient), _p(residual), gradient.numel(), _p(compressed),
+                                            compressed.numel(), float(threshold), _stream(gradient)), "tbq_encode")
+
+
+def tbq_decode(compressed, gradient):
+    _u8(compressed, "compressed"); _f32(gradient, "gradient", compressed)
+    with torch.cuda.device(gradient.device):
+        check(_lib.lib().hipress_tbq_decode(_p(compressed), compressed.numel(), _p(gradient), gradient.numel(),
+                                            _stream(gradient)), "tbq_decode")
+
+
+# ---------------------------------------------------------------- onebit
+def onebit_encode(gradient, residual, compressed):
+    """Sign bits + mean-magnitude scale with error feedback; residual is updated in place."""
+    _f32(gradient, "gradient"); _f32(residual, "residual", gradient); _u8(compressed, "compressed", gradient)
+    _same_numel(gradient, residual, "gradient", "residual")
+    L = _lib.lib()
+    n = gradient.numel()
+    with torch.cuda.device(gradient.device):
+        need = size(L.hipress_onebit_workspace_bytes(n), "onebit_workspace_bytes")
+        ws = _workspace(gradient, need)
+        check(L.hipress_onebit_encode(_p(gradient), _p(residual), n, _p(compressed), compressed.numel(),
+                                      _p(ws), ws.numel(), _stream(gradient)), "onebit_encode")
+
+
+def onebit_decode(compressed, gradient):
+    _u8(compressed, "compressed"); _f32(gradient, "gradient", compressed)
+    with torch.cuda.device(gradient.device):
+        check(_lib.lib().hipress_onebit_decode(_p(compressed), compressed.numel(), _p(gradient), gradient.numel(),
+                                               _stream(gradient)), "onebit_decode")
+
+
+# ---------------------------------------------------------------- TernGrad
+def terngrad_encode(gradient, uniform, compressed, bucket=512):
+    """Stochastic ternarisation; `uniform` holds one U[0,1) draw per element."""
+    _f32(gradient, "gradient"); _f32(uniform, "uniform", gradient); _u8(compressed, "compressed", gradient)
+    _same_numel(gradient, uniform, "gradient", "uniform")
+    with torch.cuda.device(gradient.device):
+        check(_lib.lib().hipress_terngrad_encode(_p(gradient), _p(uniform), gradient.numel(), _p(compressed),
+                                                 compressed.numel(), int(bucket), _stream(gradient)), "terngrad_encode")
+
+
+def terngrad_decode(compressed, gradient):
+    _u8(compressed, "compressed"); _f32(gradient, "gradient", compressed)
+    with torch.cuda.device(gradient.device):
+        check(_lib.lib().hipress_terngrad_decode(_p(compressed), compressed.numel(), _p(gradient), gradient.numel(),
+                                                 _stream(gradient)), "terngrad_decode")
+
+
+# ---------------------------------------------------------------- DGC / GradDrop
+def dgc_encode(gradient, momentum, accumulator, compressed, momentum_factor=0.9, ratio=0.001):
+    """Deep gradient compression: momentum correction, local accumulation,
+    sampled-threshold top-`ratio` selection; momentum and accumulator are updated in place."""
+    _f32(gradient, "gradient"); _f32(momentum, "momentum", gradient); _f32(accumulator, "accumulator", gradient)
+    _u8(compressed, "compressed", gradient)
+    _same_numel(gradient, momentum, "gradient", "momentum"); _same_numel(gradient, accumulator, "gradient", "accumulator")
+    L = _lib.lib()
+    n = gradient.numel()
+    with torch.cuda.device(gradient.device):
+        need = size(L.hipress_sparse_workspace_bytes(n, float(ratio)), "sparse_workspace_bytes")
+        ws = _workspace(gradient, need)
+        check(L.hipress_dgc_encode(_p(gradient), _p(momentum), _p(accumulator), n, _p(compressed), compressed.numel(),
+                                   float(momentum_factor), float(ratio), _p(ws), ws.numel(), _stream(gradient)), "dgc_encode")
+
+
+def graddrop_encode(gradient, accumulator, compressed, ratio=0.01):
+    """Gradient dropping: `ratio` is the kept fraction (drop ratio 0.99 = ratio 0.01)."""
+    _f32(gradient, "gradient"); _f32(accumulator, "accumulator", gradient); _u8(compressed, "compressed", gradient)
+    _same_numel(gradient, accumulator, "gradient", "accumulator")
+    L = _lib.lib()
+    n = gradient.numel()
+    with torch.cuda.device(gradient.device):
+        need = size(L.hipress_sparse_workspace_bytes(n, float(ratio)), "sparse_workspace_bytes")
+        ws = _workspace(gradient, need)
+        check(L.hipress_graddrop_encode(_p(gradient), _p(accumulator), n, _p(compressed), compressed.numel(),
+                                        float(ratio), _p(ws), ws.numel(), _stream(gradient)), "graddrop_encode")
+
+
+def dgc_decode(compressed, gradient):
+    _u8(compressed, "compressed"); _f32(gradient, "gradient", compressed)
+    with torch.cuda.device(gradient.device):
+        check(_lib.lib().hipress_sparse_decode(_p(compressed), compressed.numel(), _p(gradient), gradient.numel(),
+                                               _stream(gradient)), "sparse_decode")
+
+
+graddrop_decode = dgc_decode
+
+
+# ---------------------------------------------------------------- decode-and-merge
+def _peers(compressed_list, like):
+    if not 1 <= len(compressed_list) <= MAX_PEERS:
+        raise ValueError(f"between 1 and {MAX_PEERS} peer payloads are supported, got {len(compressed_list)}")
+    for i, c in enumerate(compressed_list):
+        _u8(c, f"compressed[{i}]", like)
+    P = len(compressed_list)
+    ptrs = (ctypes.c_void_p * P)(*[c.data_ptr() for c in compressed_list])
+    lens = (ctypes.c_int64 * P)(*[c.numel() for c in compressed_list])
+    return ptrs, lens, P
+
+
+def tbq_decode_merge(compressed_list, aggregate, residual=None, out_compressed=None, threshold=0.0):
+    """aggregate = sum of the decoded peers; with `residual` given the aggregate is
+    re-encoded into `out_compressed` with the aggregator's own residual."""
+    _f32(aggregate, "aggregate")
+    ptrs, lens, P = _peers(compressed_list, aggregate)
+    if residual is not None:
+        _f32(residual, "residual", aggregate); _u8(out_compressed, "out_compressed", aggregate)
+        _same_numel(aggregate, residual, "aggregate", "residual")
+    with torch.cuda.device(aggregate.device):
+        check(_lib.lib().hipress_tbq_decode_merge(
+            ptrs, lens, P, _p(aggregate), aggregate.numel(), _p(residual), _p(out_compressed),
+            out_compressed.numel() if out_compressed is not None else 0, float(threshold), _stream(aggregate)),
+            "tbq_decode_merge")
+
+
+def onebit_decode_merge(compressed_list, aggregate):
+    _f32(aggregate, "aggregate")
+    ptrs, lens, P = _peers(compressed_list, aggregate)
+    with torch.cuda.device(aggregate.device):
+        check(_lib.lib().hipress_onebit_decode_merge(ptrs, lens, P, _p(aggregate), aggregate.numel(),
+                                                     _stream(aggregate)), "onebit_decode_merge")
+
+
+def terngrad_decode_merge(compressed_list, aggregate):
+    _f32(aggregate, "aggregate")
+    ptrs, lens, P = _peers(compressed_list, aggregate)
+    with torch.cuda.device(aggregate.device):
+        check(_lib.lib().hipress_terngrad_decode_merge(ptrs, lens, P, _p(aggregate), aggregate.numel(),
+                                                       _stream(aggregate)), "terngrad_decode_merge")
+
+
+def dgc_decode_merge(compressed_list, aggregate, accumulator=None, out_compressed=None, ratio=0.001):
+    """Scatter-add of the peers' (index, value) pairs; with `accumulator` given the
+    aggregate is re-sparsified into `out_compressed` (accumulator = aggregator residual)."""
+    _f32(aggregate, "aggregate")
+    ptrs, lens, P = _peers(compressed_list, aggregate)
+    L = _lib.lib()
+    n = aggregate.numel()
+    ws = None
+    if accumulator is not None:
+        _f32(accumulator, "accumulator", aggregate); _u8(out_compressed, "out_compressed", aggregate)
+        _same_numel(aggregate, accumulator, "aggregate", "accumulator")
+    with torch.cuda.device(aggregate.device):
+        if accumulator is not None:
+            ws = _workspace(aggregate, size(L.hipress_sparse_workspace_bytes(n, float(ratio)), "sparse_workspace_bytes"))
+        check(L.hipress_sparse_decode_merge(
+            ptrs, lens, P, _p(aggregate), n, _p(accumulator), _p(out_compressed),
+            out_compressed.numel() if out_compressed is not None else 0, float(ratio),
+            _p(ws), ws.numel() if ws is not None else 0, _stream(aggregate)), "sparse_decode_merge")
+
+
+graddrop_decode_merge = dgc_decode_merge
+
+
+# ---------------------------------------------------------------- batched launches
+class Batch:
+    """All tensors of a gradient set behind one launch sequence.
+
+    ``tensors`` is a list of dicts with the keys the algorithm needs:
+    gradient, residual (onebit, tbq), momentum + accumulator (dgc), accumulator
+    (graddrop), uniform (terngrad), compressed, and ``out`` for decode.  The
+    tensors must stay alive and keep their addresses for the life of the batch.
+    """
+
+    def __init__(self, alg, tensors, threshold=0.0, bucket=512, momentum_factor=0.9, ratio=0.001):
+        self.alg = alg
+        self._keep = tensors
+        alg_id = ALG_IDS[alg]
+        arr = (Tensor * max(len(tensors), 1))()
+        dev = None
+        for i, t in enumerate(tensors):
+            c = _u8(t["compressed"], "compressed")
+            dev = dev or c.device
+            g = t.get("gradient")
+            if alg in ("onebit", "tbq"):
+                s0, s1 = t.get("residual"), None
+            elif alg == "dgc":
+                s0, s1 = t.get("momentum"), t.get("accumulator")
+            elif alg == "graddrop":
+                s0, s1 = t.get("accumulator"), None
+            else:
+                s0, s1 = None, None
+            u, o = t.get("uniform"), t.get("out")
+            for name, x in (("gradient", g), ("state", s0), ("state", s1), ("uniform", u), ("out", o)):
+                if x is not None:
+                    _f32(x, name, c)
+            n = (g if g is not None else o).numel()
+            arr[i] = Tensor(_p(g), _p(s0), _p(s1), _p(u), _p(c), _p(o), n, c.numel())
+        self.device = dev
+        pr = Params(float(threshold), int(bucket), float(momentum_factor), 0.0, float(ratio))
+        h = ctypes.c_void_p()
+        with torch.cuda.device(dev):
+            check(_lib.lib().hipress_batch_create(ctypes.byref(h), alg_id, arr, len(tensors), ctypes.byref(pr)), "batch_create")
+        self._h = h
+
+    def encode(self):
+        with torch.cuda.device(self.device):
+            check(_lib.lib().hipress_batch_encode(self._h, torch.cuda.current_stream(self.device).cuda_stream), "batch_encode")
+
+    def decode(self):
+        with torch.cuda.device(self.device):
+            check(_lib.lib().hipress_batch_decode(self._h, torch.cuda.current_stream(self.device).cuda_stream), "batch_decode")
+
+    def close(self):
+        if getattr(self, "_h", None):
+            _lib.lib().hipress_batch_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+
+class MergeBatch:
+    """Decode-and-merge of many chunks in one launch sequence.
+
+    ``chunks``: list of dicts with ``compressed`` (list of peer payload tensors),
+    ``aggregate``, and optionally ``state`` + ``out_compressed`` for the fused
+    re-encode (tbq: aggregator residual; dgc/graddrop: aggregator accumulator).
+    """
+
+    def __init__(self, alg, chunks, threshold=0.0, bucket=512, ratio=0.001):
+        self._keep = chunks
+        npeers = len(chunks[0]["compressed"]) if chunks else 1
+        arr = (MergeChunk * max(len(chunks), 1))()
+        dev = None
+        for i, c in enumerate(chunks):
+            agg = _f32(c["aggregate"], "aggregate")
+            dev = dev or agg.device
+            if len(c["compressed"]) != npeers:
+                raise ValueError("every chunk must have the same number of peers")
+            mc = MergeChunk()
+            for p, pay in enumerate(c["compressed"]):
+                _u8(pay, "compressed", agg)
+                mc.payloads[p] = pay.data_ptr()
+                mc.payload_bytes[p] = pay.numel()
+            mc.aggregate = agg.data_ptr()
+            st, oc = c.get("state"), c.get("out_compressed")
+            if st is not None:
+                _f32(st, "state", agg); _u8(oc, "out_compressed", agg)
+                mc.state, mc.out_payload, mc.out_payload_bytes = st.data_ptr(), oc.data_ptr(), oc.numel()
+            mc.n = agg.numel()
+            arr[i] = mc
+        self.device = dev
+        pr = Params(float(threshold), int(bucket), 0.0, 0.0, float(ratio))
+        h = ctypes.c_void_p()
+        with torch.cuda.device(dev):
+            check(_lib.lib().hipress_merge_batch_create(ctypes.byref(h), ALG_IDS[alg], arr, len(chunks), npeers,
+                                                        ctypes.byref(pr)), "merge_batch_create")
+        self._h = h
+
+    def run(self):
+        with torch.cuda.device(self.device):
+            check(_lib.lib().hipress_merge_batch_run(self._h, torch.cuda.current_stream(self.device).cuda_stream), "merge_batch_run")
+
+    def close(self):
+        if getattr(self, "_h", None):
+            _lib.lib().hipress_merge_batch_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+
+# ---------------------------------------------------------------- aliases + torch.ops registration
+# CompLL names its generated operators <Func>Encode / <Func>Decode
+# (TernGradEncode.cc:10); one line per name maps them onto the operators above.
+ALIASES = {
+    "OnebitEncode": onebit_encode, "OnebitDecode": onebit_decode,
+    "TBQEncode": tbq_encode, "TBQDecode": tbq_decode,
+    "TernGradEncode": terngrad_encode, "TernGradDecode": terngrad_decode,
+    "DGCEncode": dgc_encode, "DGCDecode": dgc_decode,
+    "GradDropEncode": graddrop_encode, "GradDropDecode": graddrop_decode,
+}
+globals().update(ALIASES)
+__all__ += list(ALIASES)
+
+_SCHEMAS = {
+    "onebit_encode": "(Tensor gradient, Tensor(a!) residual, Tensor(b!) compressed) -> ()",
+    "onebit_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
+    "tbq_encode": "(Tensor gradient, Tensor(a!) residual, Tensor(b!) compressed, float threshold) -> ()",
+    "tbq_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
+    "terngrad_encode": "(Tensor gradient, Tensor uniform, Tensor(a!) compressed, int bucket=512) -> ()",
+    "terngrad_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
+    "dgc_encode": "(Tensor gradient, Tensor(a!) momentum, Tensor(b!) accumulator, Tensor(c!) compressed, "
+                  "float momentum_factor=0.9, float ratio=0.001) -> ()",
+    "dgc_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
+    "graddrop_encode": "(Tensor gradient, Tensor(a!) accumulator, Tensor(b!) compressed, float ratio=0.01) -> ()",
+    "graddrop_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
+    "onebit_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate) -> ()",
+    "terngrad_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate) -> ()",
+    "tbq_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate, Tensor(b!)? residual=None, "
+                        "Tensor(c!)? out_compressed=None, float threshold=0.0) -> ()",
+    "dgc_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate, Tensor(b!)? accumulator=None, "
+                        "Tensor(c!)? out_compressed=None, float ratio=0.001) -> ()",
+    "graddrop_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate, Tensor(b!)? accumulator=None, "
+                             "Tensor(c!)? out_compressed=None, float ratio=0.01) -> ()",
+}
+_ALIAS_OF = {
+    "OnebitEncode": "onebit_encode", "OnebitDecode": "onebit_decode", "TBQEncode": "tbq_encode",
+    "TBQDecode": "tbq_decode", "TernGradEncode": "terngrad_encode", "TernGradDecode": "terngrad_decode",
+    "DGCEncode": "dgc_encode", "DGCDecode": "dgc_decode", "GradDropEncode": "graddrop_encode",
+    "GradDropDecode": "graddrop_decode",
+}
+
+
+def _register():
+    lib = torch.library.Library("hipress", "DEF")
+    for name, schema in _SCHEMAS.items():
+        lib.define(name + schema)
+        lib.impl(name, globals()[name], "CUDA")
+    for alias, target in _ALIAS_OF.items():
+        lib.define(alias + _SCHEMAS[target])
+        lib.impl(alias, globals()[target], "CUDA")
+    return lib
+
+
+_torch_lib = _register()

@@ -1,0 +1,196 @@
+/*
+ * hipress_amd — C ABI of the MI355X (gfx950) gradient-compression operators.
+ *
+ * One shared library, libhipress_amd.so, exports everything declared here with
+ * C linkage.  All pointers named grad/residual/momentum/accumulator/uniform/
+ * payload/out/aggregate/workspace are DEVICE pointers owned by the caller;
+ * `stream` is a hipStream_t passed as void* (NULL = the default stream), the
+ * way the reference carries its stream
+ * (/root/reference/src/CompLL/GCGen/output/get_policy_general.h:125-133,
+ *  /root/reference/src/CompLL/GCGen/output/get_stream_mxnet.h:19-25).
+ * Every call only enqueues work on `stream` and returns; nothing here
+ * synchronises with the host or allocates device memory, except
+ * hipress_batch_create / hipress_merge_batch_create (set-up time) and their
+ * destroy calls.
+ *
+ * The per-tensor entry points replace the reference's generated operator body
+ *   void <Func>_body<policy_t>(float* gradient, int32 _gradient_size,
+ *                              uint8* compressed, int32 _compressed_size,
+ *                              <scalars>, policy_t policy, void* stream)
+ * (/root/reference/src/CompLL/GCGen/output/TernGradEncode/TernGradEncode_body.h:99-109,
+ *  /root/reference/src/CompLL/GCGen/output/TernGradDecode/TernGradDecode_body.h:48-57)
+ * which the framework wrappers call with raw pointers and element counts
+ * (TernGradEncode_wrapper.h:42-70, TernGradDecode_wrapper.h:40-67): encode takes
+ * (gradient, [state...], compressed, scalars), decode takes (compressed,
+ * gradient); both buffers are caller-allocated and updated in place
+ * (TernGradEncode.cc:10-24, TernGradDecode.cc:10-24).  Differences: sizes are
+ * int64, error-feedback state buffers are explicit arguments, and errors come
+ * back as negative return codes instead of a fatal CHECK.
+ *
+ * Payload layout (all little-endian, payload base 16-byte aligned):
+ *   16-byte header, then dense uint32 words.  Code i of width b occupies bits
+ *   [b*(i mod 32/b), +b) of word floor(i*b/32) — the byte image the reference
+ *   decoder reads (TernGradDecode_body.h:44).  Pad codes are 0.
+ *     onebit   {f32 scale, u32 n, 0, 0}            words: ceil(n/32)
+ *     tbq      {f32 tau,   u32 n, 0, 0}            words: ceil(n/16)
+ *     terngrad {u32 n, u32 bucket, 0, 0} f32 scale[ceil(n/bucket)] (padded to
+ *              16 B) then words: ceil(n/16)
+ *     dgc/graddrop {u32 nnz, u32 n, u32 capacity, f32 thr} i32 idx[capacity]
+ *              f32 val[capacity]; pairs are in ascending index order
+ *   2-bit codes: 0 -> 0, 1 -> +scale, 2 -> -scale, 3 -> 0 (never produced).
+ */
+#ifndef HIPRESS_AMD_H_
+#define HIPRESS_AMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HIPRESS_OK 0
+#define HIPRESS_ERR_NULL (-1)      /* a required pointer is NULL */
+#define HIPRESS_ERR_SIZE (-2)      /* n out of range, or a buffer is too small */
+#define HIPRESS_ERR_ALIGN (-3)     /* pointer not aligned (fp32: 4 B, payload/workspace: 16 B) */
+#define HIPRESS_ERR_PARAM (-4)     /* scalar parameter out of range */
+#define HIPRESS_ERR_HIP (-5)       /* the HIP runtime reported an error */
+#define HIPRESS_ERR_WORKSPACE (-6) /* workspace missing or too small */
+
+#define HIPRESS_HEADER_BYTES 16
+#define HIPRESS_MAX_PEERS 16
+#define HIPRESS_MAX_N 4294967295LL /* n is carried as u32 in payload headers */
+
+enum hipress_alg {
+    HIPRESS_ONEBIT = 0,
+    HIPRESS_TBQ = 1,
+    HIPRESS_TERNGRAD = 2,
+    HIPRESS_DGC = 3,
+    HIPRESS_GRADDROP = 4
+};
+
+int hipress_version(void);
+const char *hipress_strerror(int code);
+
+/* ---- sizes (host-only arithmetic; negative return = error code) ---------- */
+int64_t hipress_onebit_payload_bytes(int64_t n);
+int64_t hipress_tbq_payload_bytes(int64_t n);
+int64_t hipress_terngrad_payload_bytes(int64_t n, int32_t bucket);
+int64_t hipress_sparse_capacity(int64_t n, double ratio);
+int64_t hipress_sparse_payload_bytes(int64_t n, double ratio);
+int64_t hipress_onebit_workspace_bytes(int64_t n);
+int64_t hipress_sparse_workspace_bytes(int64_t n, double ratio);
+
+/* ---- TBQ: threshold two-bit quantisation with error feedback ------------- */
+/* Replaces <Func>_body for the built-in "tbq" algorithm
+ * (/root/reference/README.md:9,45).  residual is read and overwritten. */
+int hipress_tbq_encode(const float *grad, float *residual, int64_t n, void *payload,
+                       int64_t payload_bytes, float threshold, void *stream);
+int hipress_tbq_decode(const void *payload, int64_t payload_bytes, float *out, int64_t n,
+                       void *stream);
+
+/* ---- onebit: sign bits, per-tensor mean-magnitude scale, error feedback --- */
+/* Replaces <Func>_body for "onebit" (/root/reference/README.md:9).  Where the
+ * reference body blocks the host on each thrust::reduce result
+ * (TernGradEncode_body.h:115-116), the scale here stays on the device. */
+int hipress_onebit_encode(const float *grad, float *residual, int64_t n, void *payload,
+                          int64_t payload_bytes, void *workspace, int64_t workspace_bytes,
+                          void *stream);
+int hipress_onebit_decode(const void *payload, int64_t payload_bytes, float *out, int64_t n,
+                          void *stream);
+
+/* ---- TernGrad: stochastic ternarisation, per-bucket max-abs scale ---------- */
+/* Replaces TernGradEncode_body / TernGradDecode_body for "terngrad"
+ * (/root/reference/README.md:9,276).  The rounding noise is an explicit
+ * uniform[0,1) tensor instead of the body's clock-seeded generator
+ * (TernGradEncode_body.h:49,119). */
+int hipress_terngrad_encode(const float *grad, const float *uniform, int64_t n, void *payload,
+                            int64_t payload_bytes, int32_t bucket, void *stream);
+int hipress_terngrad_decode(const void *payload, int64_t payload_bytes, float *out, int64_t n,
+                            void *stream);
+
+/* ---- DGC / GradDrop: sampled-threshold sparsification ---------------------- */
+/* Replace <Func>_body for "dgc" and "graddrop" (/root/reference/README.md:9,162).
+ * ratio is the kept fraction (DGC 0.001; GradDrop drop ratio 0.99 = 0.01). */
+int hipress_dgc_encode(const float *grad, float *momentum, float *accumulator, int64_t n,
+                       void *payload, int64_t payload_bytes, float momentum_factor, double ratio,
+                       void *workspace, int64_t workspace_bytes, void *stream);
+int hipress_graddrop_encode(const float *grad, float *accumulator, int64_t n, void *payload,
+                            int64_t payload_bytes, double ratio, void *workspace,
+                            int64_t workspace_bytes, void *stream);
+/* One decoder for both: zero-fill out[n], then scatter the pairs. */
+int hipress_sparse_decode(const void *payload, int64_t payload_bytes, float *out, int64_t n,
+                          void *stream);
+
+/* ---- decode-and-merge (the aggregation step of CaSync, README.md:7) -------- */
+/* payloads / payload_bytes are HOST arrays of npeers entries (device pointers
+ * and sizes).  aggregate[n] receives the sum of the decoded peers.  With a
+ * non-NULL residual (tbq) or accumulator (sparse) the aggregate is re-encoded
+ * for the next hop into out_payload in the same pass. */
+int hipress_tbq_decode_merge(const void *const *payloads, const int64_t *payload_bytes,
+                             int32_t npeers, float *aggregate, int64_t n, float *residual,
+                             void *out_payload, int64_t out_payload_bytes, float threshold,
+                             void *stream);
+int hipress_onebit_decode_merge(const void *const *payloads, const int64_t *payload_bytes,
+                                int32_t npeers, float *aggregate, int64_t n, void *stream);
+int hipress_terngrad_decode_merge(const void *const *payloads, const int64_t *payload_bytes,
+                                  int32_t npeers, float *aggregate, int64_t n, void *stream);
+int hipress_sparse_decode_merge(const void *const *payloads, const int64_t *payload_bytes,
+                                int32_t npeers, float *aggregate, int64_t n, float *accumulator,
+                                void *out_payload, int64_t out_payload_bytes, double ratio,
+                                void *workspace, int64_t workspace_bytes, void *stream);
+
+/* ---- batched launches over a whole gradient set ---------------------------- */
+/* A training step compresses every tensor of the model; a batch object holds a
+ * device-resident table of the tensors so that one launch sequence covers all of
+ * them (the per-tensor calls cost one launch sequence each).  Fields a given
+ * algorithm does not use may be NULL. */
+typedef struct hipress_tensor {
+    const float *grad;    /* encode input, fp32[n] */
+    float *state0;        /* residual (onebit, tbq) | momentum (dgc) | accumulator (graddrop) */
+    float *state1;        /* accumulator (dgc) */
+    const float *uniform; /* terngrad rounding noise, fp32[n] */
+    void *payload;        /* compressed buffer */
+    float *out;           /* decode output, fp32[n] */
+    int64_t n;
+    int64_t payload_bytes;
+} hipress_tensor;
+
+typedef struct hipress_params {
+    float threshold;       /* tbq */
+    int32_t bucket;        /* terngrad */
+    float momentum_factor; /* dgc */
+    float reserved;
+    double ratio;          /* dgc, graddrop */
+} hipress_params;
+
+typedef struct hipress_batch hipress_batch;
+
+int hipress_batch_create(hipress_batch **out, int32_t alg, const hipress_tensor *tensors,
+                         int32_t count, const hipress_params *params);
+int hipress_batch_encode(hipress_batch *batch, void *stream);
+int hipress_batch_decode(hipress_batch *batch, void *stream);
+int hipress_batch_destroy(hipress_batch *batch);
+
+/* One chunk of the aggregation step: npeers payloads of the same n. */
+typedef struct hipress_merge_chunk {
+    const void *payloads[HIPRESS_MAX_PEERS];
+    int64_t payload_bytes[HIPRESS_MAX_PEERS];
+    float *aggregate;    /* fp32[n] */
+    float *state;        /* aggregator residual (tbq) / accumulator (sparse), or NULL */
+    void *out_payload;   /* re-encoded payload when state != NULL */
+    int64_t out_payload_bytes;
+    int64_t n;
+} hipress_merge_chunk;
+
+typedef struct hipress_merge_batch hipress_merge_batch;
+
+int hipress_merge_batch_create(hipress_merge_batch **out, int32_t alg,
+                               const hipress_merge_chunk *chunks, int32_t count, int32_t npeers,
+                               const hipress_params *params);
+int hipress_merge_batch_run(hipress_merge_batch *batch, void *stream);
+int hipress_merge_batch_destroy(hipress_merge_batch *batch);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIPRESS_AMD_H_ */

@@ -1,0 +1,85 @@
+"""CPU-side checks of the C ABI: the library loads, exports every function
+include/hipress_amd.h declares, the ctypes binding covers them all, and the
+host-only size arithmetic agrees with the oracle's.  No GPU work is issued."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import oracle
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "hipress_amd.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hipress_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from hipress_amd import _lib
+
+    return _lib
+
+
+def test_header_declares_the_expected_surface():
+    names = declared_functions()
+    for alg in ("onebit", "tbq", "terngrad"):
+        assert f"hipress_{alg}_encode" in names and f"hipress_{alg}_decode" in names
+        assert f"hipress_{alg}_decode_merge" in names
+    for n in ("hipress_dgc_encode", "hipress_graddrop_encode", "hipress_sparse_decode", "hipress_sparse_decode_merge",
+              "hipress_batch_create", "hipress_batch_encode", "hipress_batch_decode", "hipress_merge_batch_run"):
+        assert n in names
+
+
+def test_library_exports_every_declared_symbol(lib):
+    raw = ctypes.CDLL(lib.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(raw, name), f"{name} is declared in the header but not exported"
+        assert name in lib.SIGNATURES, f"{name} has no ctypes signature"
+    assert set(lib.SIGNATURES) == set(declared_functions())
+
+
+def test_version_and_strerror(lib):
+    L = lib.lib()
+    assert L.hipress_version() >= 100
+    assert lib.strerror(0) == "ok"
+    for code in range(-6, 0):
+        assert lib.strerror(code) not in ("ok", "unknown error")
+
+
+@pytest.mark.parametrize("n", [0, 1, 15, 16, 17, 31, 32, 33, 512, 513, 4096, 262143, 262144, 102760448])
+def test_sizes_match_oracle(lib, n):
+    L = lib.lib()
+    assert L.hipress_onebit_payload_bytes(n) == oracle.onebit_payload_bytes(n)
+    assert L.hipress_tbq_payload_bytes(n) == oracle.tbq_payload_bytes(n)
+    for bucket in (1, 16, 100, 512, 1024):
+        assert L.hipress_terngrad_payload_bytes(n, bucket) == oracle.terngrad_payload_bytes(n, bucket)
+    for ratio in (0.001, 0.01, 0.5, 1.0):
+        assert L.hipress_sparse_capacity(n, ratio) == oracle.sparse_capacity(n, ratio)
+        assert L.hipress_sparse_payload_bytes(n, ratio) == oracle.sparse_payload_bytes(n, ratio)
+        assert L.hipress_sparse_workspace_bytes(n, ratio) > 0
+    assert L.hipress_onebit_workspace_bytes(n) >= 4 * max(1, (n + 4095) // 4096)
+
+
+def test_size_errors(lib):
+    L = lib.lib()
+    assert L.hipress_tbq_payload_bytes(-1) == -2
+    assert L.hipress_tbq_payload_bytes(1 << 33) == -2
+    assert L.hipress_terngrad_payload_bytes(10, 0) == -4
+    assert L.hipress_sparse_capacity(10, 0.0) == -4
+    assert L.hipress_sparse_capacity(10, 1.5) == -4
+
+
+def test_null_and_range_checks_need_no_gpu(lib):
+    """Argument validation happens before any HIP call."""
+    L = lib.lib()
+    assert L.hipress_tbq_encode(None, None, 10, None, 100, 0.05, None) == -1
+    assert L.hipress_tbq_encode(None, None, -1, None, 100, 0.05, None) == -2
+    assert L.hipress_tbq_decode(None, 100, None, 10, None) == -1
+    assert L.hipress_batch_encode(None, None) == -1
+    assert L.hipress_merge_batch_run(None, None) == -1

@@ -1,0 +1,459 @@
+"""GPU parity: the HIP operators, called through the C ABI (hipress_amd.ops ->
+ctypes -> libhipress_amd.so), against the CPU oracle on the same seeded inputs.
+
+Bars: packed words, sparse indices / counts, thresholds and residuals are
+bit-exact; the onebit scale (a sum whose order differs) is within 1e-5 relative
+and everything derived from it is bit-exact once the oracle is given the GPU's
+scale."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+F = np.float32
+SIZES = [1, 15, 16, 17, 31, 33, 1000, 4095, 4096, 4097, 12289, 262144, 1000003]
+
+
+@pytest.fixture(scope="module")
+def hp():
+    import hipress_amd
+
+    assert torch.cuda.is_available()
+    hipress_amd._lib.lib()  # fails loudly if the HIP library is missing
+    return hipress_amd
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def payload(nbytes):
+    # poison so that bytes the kernels must write (pad codes, header zeros) are checked
+    return torch.full((nbytes,), 0xAB, dtype=torch.uint8, device="cuda")
+
+
+# ---------------------------------------------------------------- TBQ
+@pytest.mark.parametrize("n", SIZES)
+def test_tbq_encode_decode(hp, n):
+    rng = np.random.default_rng(n)
+    tau = 0.05
+    r_ref = rng.normal(0, 0.02, n).astype(F)
+    r_gpu = dev(r_ref)
+    for step in range(3):
+        g = rng.normal(0, 0.02, n).astype(F)
+        pay = payload(hp.tbq_payload_bytes(n))
+        hp.tbq_encode(dev(g), r_gpu, pay, tau)
+        want_pay, r_ref = oracle.tbq_encode(g, r_ref, tau)
+        np.testing.assert_array_equal(host(pay), want_pay, err_msg=f"payload step {step}")
+        np.testing.assert_array_equal(host(r_gpu), r_ref, err_msg=f"residual step {step}")
+        out = torch.full((n,), 7.0, device="cuda")
+        hp.tbq_decode(pay, out)
+        np.testing.assert_array_equal(host(out), oracle.tbq_decode(want_pay, n))
+
+
+def test_tbq_unaligned_views(hp):
+    n = 9001
+    rng = np.random.default_rng(1)
+    g, r = rng.normal(0, 0.05, n).astype(F), rng.normal(0, 0.05, n).astype(F)
+    gbuf, rbuf, obuf = torch.zeros(n + 3, device="cuda"), torch.zeros(n + 3, device="cuda"), torch.zeros(n + 3, device="cuda")
+    gv, rv, ov = gbuf[1 : n + 1], rbuf[3 : n + 3], obuf[2 : n + 2]
+    gv.copy_(dev(g)); rv.copy_(dev(r))
+    pay = payload(hp.tbq_payload_bytes(n))
+    hp.tbq_encode(gv, rv, pay, 0.05)
+    want_pay, want_r = oracle.tbq_encode(g, r, 0.05)
+    np.testing.assert_array_equal(host(pay), want_pay)
+    np.testing.assert_array_equal(host(rv), want_r)
+    assert host(rbuf)[:3].tolist() == [0, 0, 0]
+    hp.tbq_decode(pay, ov)
+    np.testing.assert_array_equal(host(ov), oracle.tbq_decode(want_pay, n))
+    assert host(obuf)[:2].tolist() == [0, 0] and host(obuf)[-1] == 0
+
+
+def test_tbq_config1_full_size(hp):
+    """262,144 elements, N(0, 0.02), threshold 0.05, residual zeros, seed 0."""
+    n = 262144
+    g = np.random.default_rng(0).normal(0, 0.02, n).astype(F)
+    r = torch.zeros(n, device="cuda")
+    pay = payload(hp.tbq_payload_bytes(n))
+    hp.tbq_encode(dev(g), r, pay, 0.05)
+    want_pay, want_r = oracle.tbq_encode(g, np.zeros(n, F), 0.05)
+    np.testing.assert_array_equal(host(pay), want_pay)
+    np.testing.assert_array_equal(host(r), want_r)
+    out = torch.empty(n, device="cuda")
+    hp.tbq_decode(pay, out)
+    np.testing.assert_array_equal(host(out), oracle.tbq_decode(want_pay, n))
+
+
+# ---------------------------------------------------------------- onebit
+@pytest.mark.parametrize("n", SIZES)
+def test_onebit_encode_decode(hp, n):
+    rng = np.random.default_rng(100 + n)
+    r_ref = rng.normal(0, 1e-3, n).astype(F)
+    r_gpu = dev(r_ref)
+    for step in range(2):
+        g = rng.normal(0, 1e-3, n).astype(F)
+        pay = payload(hp.onebit_payload_bytes(n))
+        hp.onebit_encode(dev(g), r_gpu, pay)
+        got = host(pay)
+        s_gpu = got[:4].view(F)[0]
+        s_ref = oracle.onebit_scale(g, r_ref)
+        assert abs(float(s_gpu) - float(s_ref)) <= 1e-5 * float(s_ref), (s_gpu, s_ref)
+        # with the GPU's scale the oracle must reproduce every byte and every residual bit
+        want_pay, r_next = oracle.onebit_encode(g, r_ref, scale=s_gpu)
+        np.testing.assert_array_equal(got, want_pay, err_msg=f"payload step {step}")
+        np.testing.assert_array_equal(host(r_gpu), r_next, err_msg=f"residual step {step}")
+        # and against the oracle's own scale the residual is within 1e-5 * max(s, |r|)
+        _, r_own = oracle.onebit_encode(g, r_ref)
+        assert np.all(np.abs(r_next - r_own) <= 1e-5 * np.maximum(s_ref, np.abs(r_own)))
+        out = torch.full((n,), 7.0, device="cuda")
+        hp.onebit_decode(pay, out)
+        np.testing.assert_array_equal(host(out), oracle.onebit_decode(want_pay, n))
+        r_ref = r_next
+
+
+def test_onebit_scale_is_deterministic(hp):
+    n = 3_000_000
+    g = dev(np.random.default_rng(2).normal(0, 1e-3, n).astype(F))
+    scales = []
+    for _ in range(3):
+        pay = payload(hp.onebit_payload_bytes(n))
+        hp.onebit_encode(g, torch.zeros(n, device="cuda"), pay)
+        scales.append(host(pay)[:4].view(np.uint32)[0])
+    assert len(set(scales)) == 1
+
+
+def test_onebit_zero_tensor(hp):
+    n = 5000
+    pay = payload(hp.onebit_payload_bytes(n))
+    r = torch.zeros(n, device="cuda")
+    hp.onebit_encode(torch.zeros(n, device="cuda"), r, pay)
+    want_pay, want_r = oracle.onebit_encode(np.zeros(n, F), np.zeros(n, F))
+    np.testing.assert_array_equal(host(pay), want_pay)
+    np.testing.assert_array_equal(host(r), want_r)
+
+
+# ---------------------------------------------------------------- TernGrad
+@pytest.mark.parametrize("bucket", [512, 256, 1024, 100, 16, 2048])
+@pytest.mark.parametrize("n", [1, 17, 511, 512, 513, 4097, 70001, 1000003])
+def test_terngrad_encode_decode(hp, n, bucket):
+    rng = np.random.default_rng(n * 7 + bucket)
+    g = rng.normal(0, 1e-3, n).astype(F)
+    out_l = rng.random(n) < 0.01
+    g[out_l] = rng.laplace(0, 1e-2, out_l.sum()).astype(F)
+    u = rng.random(n, dtype=F)
+    pay = payload(hp.terngrad_payload_bytes(n, bucket))
+    hp.terngrad_encode(dev(g), dev(u), pay, bucket)
+    want = oracle.terngrad_encode(g, u, bucket)
+    np.testing.assert_array_equal(host(pay), want)
+    out = torch.full((n,), 7.0, device="cuda")
+    hp.terngrad_decode(pay, out)
+    np.testing.assert_array_equal(host(out), oracle.terngrad_decode(want, n))
+
+
+def test_terngrad_decode_rejects_header_that_overruns_buffer(hp):
+    n = 5000
+    pay = torch.zeros(hp.terngrad_payload_bytes(n, 512), dtype=torch.uint8, device="cuda")
+    hdr = np.zeros(4, np.uint32)
+    hdr[:2] = [n, 1]  # bucket 1 would need a 20 KB scale array: does not fit
+    pay[:16] = dev(hdr.view(np.uint8))
+    out = torch.full((n,), 7.0, device="cuda")
+    hp.terngrad_decode(pay, out)
+    assert not host(out).any()
+
+
+# ---------------------------------------------------------------- DGC / GradDrop
+def check_sparse(got_pay, want_pay):
+    g = oracle.sparse_unpack(got_pay)
+    w = oracle.sparse_unpack(want_pay)
+    assert g[:3] == w[:3], (g[:3], w[:3])
+    assert g[3].view(np.uint32) == w[3].view(np.uint32), (g[3], w[3])
+    np.testing.assert_array_equal(g[4], w[4])
+    np.testing.assert_array_equal(g[5], w[5])
+
+
+@pytest.mark.parametrize("n", [1, 63, 1000, 4097, 70001, 262143, 262144, 1000003])
+def test_dgc_encode_decode(hp, n):
+    rng = np.random.default_rng(200 + n)
+    m, ratio = 0.9, 0.001
+    mom_ref, acc_ref = np.zeros(n, F), np.zeros(n, F)
+    mom, acc = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    for step in range(3):
+        g = rng.normal(0, 1e-3, n).astype(F)
+        pay = payload(hp.dgc_payload_bytes(n, ratio))
+        hp.dgc_encode(dev(g), mom, acc, pay, m, ratio)
+        want_pay, mom_ref, acc_ref = oracle.dgc_encode(g, mom_ref, acc_ref, m, ratio)
+        check_sparse(host(pay), want_pay)
+        np.testing.assert_array_equal(host(mom), mom_ref, err_msg=f"momentum step {step}")
+        np.testing.assert_array_equal(host(acc), acc_ref, err_msg=f"accumulator step {step}")
+        out = torch.full((n,), 7.0, device="cuda")
+        hp.dgc_decode(pay, out)
+        np.testing.assert_array_equal(host(out), oracle.sparse_decode(want_pay, n))
+
+
+@pytest.mark.parametrize("n", [1, 1000, 4097, 70001, 262144, 1000003])
+def test_graddrop_encode_decode(hp, n):
+    rng = np.random.default_rng(300 + n)
+    ratio = 0.01
+    acc_ref = np.zeros(n, F)
+    acc = torch.zeros(n, device="cuda")
+    for step in range(2):
+        g = rng.normal(0, 1e-3, n).astype(F)
+        pay = payload(hp.graddrop_payload_bytes(n, ratio))
+        hp.graddrop_encode(dev(g), acc, pay, ratio)
+        want_pay, acc_ref = oracle.graddrop_encode(g, acc_ref, ratio)
+        check_sparse(host(pay), want_pay)
+        np.testing.assert_array_equal(host(acc), acc_ref)
+        out = torch.full((n,), 7.0, device="cuda")
+        hp.graddrop_decode(pay, out)
+        np.testing.assert_array_equal(host(out), oracle.sparse_decode(want_pay, n))
+
+
+def test_sparse_overflow_ties(hp):
+    n = 10000
+    g = np.full(n, 0.5, F)
+    acc = torch.zeros(n, device="cuda")
+    pay = payload(hp.graddrop_payload_bytes(n, 0.001))
+    hp.graddrop_encode(dev(g), acc, pay, 0.001)
+    want_pay, want_acc = oracle.graddrop_encode(g, np.zeros(n, F), 0.001)
+    check_sparse(host(pay), want_pay)
+    np.testing.assert_array_equal(host(acc), want_acc)
+    assert oracle.sparse_unpack(want_pay)[0] == 64
+
+
+def test_sparse_overflow_rethreshold(hp):
+    n = 262144
+    rng = np.random.default_rng(11)
+    a = rng.uniform(1.0, 2.0, n).astype(F) * rng.choice([-1, 1], n).astype(F)
+    a[50::100] = rng.uniform(0.001, 0.002, a[50::100].size).astype(F)
+    a[1000:1010] = a[2000]  # some exact ties near the top
+    mom, acc = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    pay = payload(hp.dgc_payload_bytes(n, 0.001))
+    hp.dgc_encode(dev(a), mom, acc, pay, 0.9, 0.001)
+    want_pay, want_mom, want_acc = oracle.dgc_encode(a, np.zeros(n, F), np.zeros(n, F), 0.9, 0.001)
+    check_sparse(host(pay), want_pay)
+    np.testing.assert_array_equal(host(mom), want_mom)
+    np.testing.assert_array_equal(host(acc), want_acc)
+
+
+def test_sparse_all_zero(hp):
+    n = 5000
+    acc = torch.zeros(n, device="cuda")
+    pay = payload(hp.graddrop_payload_bytes(n, 0.01))
+    hp.graddrop_encode(torch.zeros(n, device="cuda"), acc, pay, 0.01)
+    nnz, n_, cap, thr, idx, val = oracle.sparse_unpack(host(pay))
+    assert (nnz, n_, thr) == (0, n, 0)
+    out = torch.full((n,), 7.0, device="cuda")
+    hp.graddrop_decode(pay, out)
+    assert not host(out).any()
+
+
+# ---------------------------------------------------------------- decode-and-merge
+@pytest.mark.parametrize("n", [1, 4097, 1048576])
+@pytest.mark.parametrize("npeers", [1, 8])
+def test_tbq_decode_merge(hp, n, npeers):
+    rng = np.random.default_rng(n + npeers)
+    tau = 0.05
+    pays = [oracle.tbq_encode(rng.normal(0, 0.04, n).astype(F), np.zeros(n, F), tau)[0] for _ in range(npeers)]
+    dpays = [dev(p) for p in pays]
+    agg = torch.full((n,), 7.0, device="cuda")
+    hp.tbq_decode_merge(dpays, agg)
+    np.testing.assert_array_equal(host(agg), oracle.tbq_decode_merge(pays, n))
+    # fused re-encode with the aggregator's residual
+    r0 = rng.normal(0, 0.01, n).astype(F)
+    r = dev(r0)
+    out = payload(hp.tbq_payload_bytes(n))
+    agg.fill_(7.0)
+    hp.tbq_decode_merge(dpays, agg, r, out, tau)
+    want_agg, want_out, want_r = oracle.tbq_decode_merge(pays, n, r0, tau)
+    np.testing.assert_array_equal(host(agg), want_agg)
+    np.testing.assert_array_equal(host(out), want_out)
+    np.testing.assert_array_equal(host(r), want_r)
+
+
+def test_onebit_and_terngrad_decode_merge(hp):
+    n, P = 70001, 5
+    rng = np.random.default_rng(9)
+    ob = [oracle.onebit_encode(rng.normal(0, 1, n).astype(F), np.zeros(n, F))[0] for _ in range(P)]
+    agg = torch.empty(n, device="cuda")
+    hp.onebit_decode_merge([dev(p) for p in ob], agg)
+    np.testing.assert_array_equal(host(agg), oracle.onebit_decode_merge(ob, n))
+    for bucket in (512, 100):
+        tg = [oracle.terngrad_encode(rng.normal(0, 1, n).astype(F), rng.random(n, dtype=F), bucket) for _ in range(P)]
+        hp.terngrad_decode_merge([dev(p) for p in tg], agg)
+        np.testing.assert_array_equal(host(agg), oracle.terngrad_decode_merge(tg, n))
+
+
+@pytest.mark.parametrize("n", [1000, 1048576])
+def test_sparse_decode_merge(hp, n):
+    P, ratio = 8, 0.001
+    rng = np.random.default_rng(n)
+    pays = []
+    for p in range(P):
+        g = rng.normal(0, 1e-3, n).astype(F)
+        g[:20] += 1.0  # duplicates across peers
+        pays.append(oracle.dgc_encode(g, np.zeros(n, F), np.zeros(n, F), 0.9, ratio)[0])
+    dpays = [dev(p) for p in pays]
+    agg = torch.full((n,), 7.0, device="cuda")
+    hp.dgc_decode_merge(dpays, agg)
+    want = oracle.sparse_decode_merge(pays, n)
+    np.testing.assert_allclose(host(agg), want, rtol=1e-5, atol=0)
+    # re-sparsify for the next hop; compare against the oracle run on the GPU's aggregate
+    acc0 = rng.normal(0, 1e-3, n).astype(F)
+    acc = dev(acc0)
+    out = payload(hp.dgc_payload_bytes(n, ratio))
+    hp.dgc_decode_merge(dpays, agg, acc, out, ratio)
+    got_agg = host(agg)
+    np.testing.assert_allclose(got_agg, want, rtol=1e-5, atol=0)
+    want_out, want_acc = oracle.graddrop_encode(got_agg, acc0, ratio)
+    check_sparse(host(out), want_out)
+    np.testing.assert_array_equal(host(acc), want_acc)
+
+
+# ---------------------------------------------------------------- batched launches
+def mixed_sizes():
+    return [1728, 64, 36864, 64, 73728, 128, 4097, 1, 262144, 512, 1000003, 1000]
+
+
+@pytest.mark.parametrize("alg", ["tbq", "onebit", "terngrad", "dgc", "graddrop"])
+def test_batch_matches_oracle(hp, alg):
+    rng = np.random.default_rng(42)
+    tensors, refs = [], []
+    for n in mixed_sizes():
+        g = rng.normal(0, 10 ** rng.uniform(-4, -2), n).astype(F)
+        t = {"gradient": dev(g), "out": torch.full((n,), 7.0, device="cuda")}
+        ref = {"g": g, "n": n}
+        if alg in ("tbq", "onebit"):
+            ref["r"] = rng.normal(0, 1e-3, n).astype(F)
+            t["residual"] = dev(ref["r"])
+            nb = hp.tbq_payload_bytes(n) if alg == "tbq" else hp.onebit_payload_bytes(n)
+        elif alg == "terngrad":
+            ref["u"] = rng.random(n, dtype=F)
+            t["uniform"] = dev(ref["u"])
+            nb = hp.terngrad_payload_bytes(n, 512)
+        elif alg == "dgc":
+            ref["mom"], ref["acc"] = rng.normal(0, 1e-3, n).astype(F), rng.normal(0, 1e-3, n).astype(F)
+            t["momentum"], t["accumulator"] = dev(ref["mom"]), dev(ref["acc"])
+            nb = hp.dgc_payload_bytes(n, 0.001)
+        else:
+            ref["acc"] = rng.normal(0, 1e-3, n).astype(F)
+            t["accumulator"] = dev(ref["acc"])
+            nb = hp.graddrop_payload_bytes(n, 0.01)
+        t["compressed"] = payload(nb)
+        tensors.append(t)
+        refs.append(ref)
+    ratio = 0.001 if alg == "dgc" else 0.01
+    b = hp.Batch(alg, tensors, threshold=0.001, bucket=512, momentum_factor=0.9, ratio=ratio)
+    b.encode()
+    b.decode()
+    for t, ref in zip(tensors, refs):
+        n, g = ref["n"], ref["g"]
+        got = host(t["compressed"])
+        if alg == "tbq":
+            want, r = oracle.tbq_encode(g, ref["r"], 0.001)
+            np.testing.assert_array_equal(got, want)
+            np.testing.assert_array_equal(host(t["residual"]), r)
+            dec = oracle.tbq_decode(want, n)
+        elif alg == "onebit":
+            s = got[:4].view(F)[0]
+            s_ref = oracle.onebit_scale(g, ref["r"])
+            assert abs(float(s) - float(s_ref)) <= 1e-5 * float(s_ref)
+            want, r = oracle.onebit_encode(g, ref["r"], scale=s)
+            np.testing.assert_array_equal(got, want)
+            np.testing.assert_array_equal(host(t["residual"]), r)
+            dec = oracle.onebit_decode(want, n)
+        elif alg == "terngrad":
+            want = oracle.terngrad_encode(g, ref["u"], 512)
+            np.testing.assert_array_equal(got, want)
+            dec = oracle.terngrad_decode(want, n)
+        elif alg == "dgc":
+            want, mom, acc = oracle.dgc_encode(g, ref["mom"], ref["acc"], 0.9, ratio)
+            check_sparse(got, want)
+            np.testing.assert_array_equal(host(t["momentum"]), mom)
+            np.testing.assert_array_equal(host(t["accumulator"]), acc)
+            dec = oracle.sparse_decode(want, n)
+        else:
+            want, acc = oracle.graddrop_encode(g, ref["acc"], ratio)
+            check_sparse(got, want)
+            np.testing.assert_array_equal(host(t["accumulator"]), acc)
+            dec = oracle.sparse_decode(want, n)
+        np.testing.assert_array_equal(host(t["out"]), dec)
+    b.close()
+
+
+@pytest.mark.parametrize("alg", ["tbq", "dgc"])
+def test_merge_batch_matches_oracle(hp, alg):
+    rng = np.random.default_rng(77)
+    P, tau, ratio = 8, 0.05, 0.001
+    chunks, refs = [], []
+    for n in [1048576, 4097, 300000]:
+        if alg == "tbq":
+            pays = [oracle.tbq_encode(rng.normal(0, 0.04, n).astype(F), np.zeros(n, F), tau)[0] for _ in range(P)]
+            nb = hp.tbq_payload_bytes(n)
+        else:
+            pays = [oracle.dgc_encode(rng.normal(0, 1e-3, n).astype(F), np.zeros(n, F), np.zeros(n, F), 0.9, ratio)[0] for _ in range(P)]
+            nb = hp.dgc_payload_bytes(n, ratio)
+        st = rng.normal(0, 1e-3, n).astype(F)
+        chunks.append({"compressed": [dev(p) for p in pays], "aggregate": torch.full((n,), 7.0, device="cuda"),
+                       "state": dev(st), "out_compressed": payload(nb)})
+        refs.append((pays, st, n))
+    mb = hp.MergeBatch(alg, chunks, threshold=tau, ratio=ratio)
+    mb.run()
+    for c, (pays, st, n) in zip(chunks, refs):
+        if alg == "tbq":
+            agg, out, r = oracle.tbq_decode_merge(pays, n, st, tau)
+            np.testing.assert_array_equal(host(c["aggregate"]), agg)
+            np.testing.assert_array_equal(host(c["out_compressed"]), out)
+            np.testing.assert_array_equal(host(c["state"]), r)
+        else:
+            got_agg = host(c["aggregate"])
+            np.testing.assert_allclose(got_agg, oracle.sparse_decode_merge(pays, n), rtol=1e-5, atol=0)
+            want_out, want_acc = oracle.graddrop_encode(got_agg, st, ratio)
+            check_sparse(host(c["out_compressed"]), want_out)
+            np.testing.assert_array_equal(host(c["state"]), want_acc)
+    mb.close()
+
+
+# ---------------------------------------------------------------- error behaviour
+def test_errors_are_raised_not_faulted(hp):
+    g = torch.zeros(100, device="cuda")
+    r = torch.zeros(100, device="cuda")
+    small = torch.zeros(16, dtype=torch.uint8, device="cuda")
+    with pytest.raises(hp._lib.HipressError):
+        hp.tbq_encode(g, r, small, 0.05)  # payload too small
+    with pytest.raises(TypeError):
+        hp.tbq_encode(g.double(), r, small, 0.05)
+    with pytest.raises(TypeError):
+        hp.tbq_encode(g, r, torch.zeros(64, device="cuda"), 0.05)  # compressed must be uint8
+    with pytest.raises(ValueError):
+        hp.tbq_encode(g, r[:50], torch.zeros(64, dtype=torch.uint8, device="cuda"), 0.05)
+    with pytest.raises(hp._lib.HipressError):
+        hp.tbq_encode(g, r, torch.zeros(64, dtype=torch.uint8, device="cuda"), -1.0)
+    with pytest.raises(hp._lib.HipressError):
+        hp.terngrad_encode(g, r, torch.zeros(4096, dtype=torch.uint8, device="cuda"), 0)
+    with pytest.raises(hp._lib.HipressError):
+        hp.graddrop_encode(g, r, torch.zeros(4096, dtype=torch.uint8, device="cuda"), 0.0)
+    ok = torch.zeros(hp.tbq_payload_bytes(100) + 16, dtype=torch.uint8, device="cuda")
+    with pytest.raises(hp._lib.HipressError):
+        hp.tbq_encode(g, r, ok[1:], 0.05)  # payload not 16-byte aligned
+    torch.cuda.synchronize()
+
+
+def test_torch_ops_namespace(hp):
+    n = 1000
+    g = np.random.default_rng(5).normal(0, 0.05, n).astype(F)
+    r = torch.zeros(n, device="cuda")
+    pay = payload(hp.tbq_payload_bytes(n))
+    torch.ops.hipress.tbq_encode(dev(g), r, pay, 0.05)
+    want, want_r = oracle.tbq_encode(g, np.zeros(n, F), 0.05)
+    np.testing.assert_array_equal(host(pay), want)
+    out = torch.empty(n, device="cuda")
+    torch.ops.hipress.TBQDecode(pay, out)
+    np.testing.assert_array_equal(host(out), oracle.tbq_decode(want, n))
