@@ -380,7 +380,7 @@ int hipress_onebit_encode(const float* grad, float* residual, int64_t n, void* p
     if (rc) return rc;
     if (!workspace || workspace_bytes < hipress_onebit_workspace_bytes(n)) return HIPRESS_ERR_WORKSPACE;
     if (mis(workspace, 16)) return HIPRESS_ERR_ALIGN;
-    return hiperr(launch_onebit_encode(single_launch(s), static_cast<float*>(workspace), static_cast<hipStream_t>(stream)));
+    return hiperr(launch_onebit_encode(single_launch(s), static_cast<float*>(workspace), -1, static_cast<hipStream_t>(stream)));
 }
 
 int hipress_onebit_decode(const void* payload, int64_t payload_bytes, float* out, int64_t n, void* stream) {
@@ -424,7 +424,7 @@ static int sparse_encode_single(int alg, const hipress_tensor& t, const hipress_
     SparseWsLayout l = sparse_ws_layout(s.ns, s.ntiles, 1);
     if (!workspace || workspace_bytes < l.bytes) return HIPRESS_ERR_WORKSPACE;
     if (mis(workspace, 16)) return HIPRESS_ERR_ALIGN;
-    return hiperr(launch_sparse_encode(single_launch(s), alg == HIPRESS_DGC, sparse_ws_at(workspace, l),
+    return hiperr(launch_sparse_encode(single_launch(s), alg == HIPRESS_DGC, sparse_ws_at(workspace, l), -1,
                                        static_cast<hipStream_t>(stream)));
 }
 
@@ -556,7 +556,7 @@ int hipress_sparse_decode_merge(const void* const* payloads, const int64_t* payl
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipError_t e = launch_sparse_merge_scatter(single_merge_launch(m, npeers, false), st);
     if (e != hipSuccess) return HIPRESS_ERR_HIP;
-    if (accumulator) e = launch_sparse_encode(single_launch(s), false, sparse_ws_at(workspace, l), st);
+    if (accumulator) e = launch_sparse_encode(single_launch(s), false, sparse_ws_at(workspace, l), -1, st);
     return hiperr(e);
 }
 
@@ -643,21 +643,35 @@ static Launch batch_launch(const hipress_batch* b, bool encode) {
     return L;
 }
 
-int hipress_batch_encode(hipress_batch* b, void* stream) {
+static int batch_encode_impl(hipress_batch* b, int phase, void* stream) {
     if (!b) return HIPRESS_ERR_NULL;
     if (!b->can_encode) return HIPRESS_ERR_NULL;
     if (b->enc.empty()) return HIPRESS_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
     Launch L = batch_launch(b, true);
     switch (b->alg) {
-        case HIPRESS_ONEBIT: return hiperr(launch_onebit_encode(L, static_cast<float*>(b->ws), st));
-        case HIPRESS_TBQ: return hiperr(launch_tbq_encode(L, st));
-        case HIPRESS_TERNGRAD: return hiperr(launch_terngrad_encode(L, (unsigned)b->params.bucket, st));
+        case HIPRESS_ONEBIT:
+            if (phase > 2) return HIPRESS_ERR_PARAM;
+            return hiperr(launch_onebit_encode(L, static_cast<float*>(b->ws), phase, st));
+        case HIPRESS_TBQ:
+            if (phase > 0) return HIPRESS_ERR_PARAM;
+            return hiperr(launch_tbq_encode(L, st));
+        case HIPRESS_TERNGRAD:
+            if (phase > 0) return HIPRESS_ERR_PARAM;
+            return hiperr(launch_terngrad_encode(L, (unsigned)b->params.bucket, st));
         case HIPRESS_DGC:
         case HIPRESS_GRADDROP:
-            return hiperr(launch_sparse_encode(L, b->alg == HIPRESS_DGC, sparse_ws_at(b->ws, b->swl), st));
+            if (phase > 4) return HIPRESS_ERR_PARAM;
+            return hiperr(launch_sparse_encode(L, b->alg == HIPRESS_DGC, sparse_ws_at(b->ws, b->swl), phase, st));
     }
     return HIPRESS_ERR_PARAM;
+}
+
+int hipress_batch_encode(hipress_batch* b, void* stream) { return batch_encode_impl(b, -1, stream); }
+
+int hipress_batch_encode_phase(hipress_batch* b, int32_t phase, void* stream) {
+    if (phase < 0) return HIPRESS_ERR_PARAM;
+    return batch_encode_impl(b, phase, stream);
 }
 
 int hipress_batch_decode(hipress_batch* b, void* stream) {
@@ -770,7 +784,7 @@ int hipress_merge_batch_run(hipress_merge_batch* b, void* stream) {
             R.dmap = b->d_map;  // same tensors, same tile numbering
             R.ntiles = b->ntiles;
             R.nsegs = (unsigned)b->renc.size();
-            e = launch_sparse_encode(R, false, sparse_ws_at(b->ws, b->swl), st);
+            e = launch_sparse_encode(R, false, sparse_ws_at(b->ws, b->swl), -1, st);
         }
         return hiperr(e);
     }

@@ -524,14 +524,17 @@ static hipError_t onebit_scale(const Launch& L, const float* partial, hipStream_
     return hipGetLastError();
 }
 
-// partial: one float per tile of the launch
-hipError_t launch_onebit_encode(const Launch& L, float* partial, hipStream_t st) {
+// partial: one float per tile of the launch.  phase < 0 runs the whole sequence,
+// 0 / 1 / 2 run only the magnitude sum / the scale / the quantisation launch.
+hipError_t launch_onebit_encode(const Launch& L, float* partial, int phase, hipStream_t st) {
     hipError_t e;
-    if (L.ntiles) {
+    if (L.ntiles && (phase < 0 || phase == 0)) {
         if ((e = onebit_abs(L, partial, st)) != hipSuccess) return e;
     }
-    if ((e = onebit_scale(L, partial, st)) != hipSuccess) return e;  // also writes headers of empty tensors
-    if (L.ntiles) {
+    if (phase < 0 || phase == 1) {
+        if ((e = onebit_scale(L, partial, st)) != hipSuccess) return e;
+    }
+    if (L.ntiles && (phase < 0 || phase == 2)) {
         if ((e = onebit_quant(L, st)) != hipSuccess) return e;
     }
     return hipSuccess;

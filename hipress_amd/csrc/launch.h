@@ -6,7 +6,7 @@ namespace hp {
 
 hipError_t launch_tbq_encode(const Launch& L, hipStream_t st);
 hipError_t launch_tbq_decode(const Launch& L, hipStream_t st);
-hipError_t launch_onebit_encode(const Launch& L, float* partial, hipStream_t st);
+hipError_t launch_onebit_encode(const Launch& L, float* partial, int phase, hipStream_t st);
 hipError_t launch_onebit_decode(const Launch& L, hipStream_t st);
 hipError_t launch_terngrad_encode(const Launch& L, unsigned bucket, hipStream_t st);
 hipError_t launch_terngrad_decode(const Launch& L, hipStream_t st);
@@ -21,7 +21,7 @@ struct SparseWs {
     uint32_t* counts;   // per wavefront-tile {above, equal} counts, then their exclusive scans
     uint32_t* thr;      // per tensor {threshold key, equal-quota}
 };
-hipError_t launch_sparse_encode(const Launch& L, bool dgc, const SparseWs& ws, hipStream_t st);
+hipError_t launch_sparse_encode(const Launch& L, bool dgc, const SparseWs& ws, int phase, hipStream_t st);
 hipError_t launch_sparse_decode(const Launch& L, hipStream_t st);
 hipError_t launch_sparse_merge_scatter(const MergeLaunch& L, hipStream_t st);
 

@@ -444,20 +444,25 @@ __global__ __launch_bounds__(kBlock) void merge_zero_fill_kernel(MSrc src) {
 
 template <class Src, class SegSrcT>
 static hipError_t sparse_encode_src(const Src& src, const SegSrcT& ssrc, unsigned ntiles, unsigned nsegs,
-                                    bool dgc, const SparseWs& ws, hipStream_t st) {
-    if (dgc) hipLaunchKernelGGL((sparse_accum_kernel<Src, true>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
-    else hipLaunchKernelGGL((sparse_accum_kernel<Src, false>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
-    hipLaunchKernelGGL((sparse_threshold_kernel<SegSrcT>), dim3(nsegs), dim3(kBlock), 0, st, ssrc, ws);
-    hipLaunchKernelGGL((sparse_count_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
-    hipLaunchKernelGGL((sparse_scan_kernel<SegSrcT>), dim3(nsegs), dim3(kBlock), 0, st, ssrc, ws);
-    hipLaunchKernelGGL((sparse_emit_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
+                                    bool dgc, const SparseWs& ws, int phase, hipStream_t st) {
+    auto on = [&](int p) { return phase < 0 || phase == p; };
+    if (on(0)) {
+        if (dgc) hipLaunchKernelGGL((sparse_accum_kernel<Src, true>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
+        else hipLaunchKernelGGL((sparse_accum_kernel<Src, false>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
+    }
+    if (on(1)) hipLaunchKernelGGL((sparse_threshold_kernel<SegSrcT>), dim3(nsegs), dim3(kBlock), 0, st, ssrc, ws);
+    if (on(2)) hipLaunchKernelGGL((sparse_count_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
+    if (on(3)) hipLaunchKernelGGL((sparse_scan_kernel<SegSrcT>), dim3(nsegs), dim3(kBlock), 0, st, ssrc, ws);
+    if (on(4)) hipLaunchKernelGGL((sparse_emit_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
     return hipGetLastError();
 }
 
-hipError_t launch_sparse_encode(const Launch& L, bool dgc, const SparseWs& ws, hipStream_t st) {
+// phase < 0 runs the whole sequence; 0..4 run one launch of it (accumulate,
+// threshold, count, scan, emit).
+hipError_t launch_sparse_encode(const Launch& L, bool dgc, const SparseWs& ws, int phase, hipStream_t st) {
     if (L.ntiles == 0) return hipSuccess;
-    if (L.single) return sparse_encode_src(SingleSrc{L.seg}, SingleSegSrc{L.seg}, L.ntiles, 1, dgc, ws, st);
-    return sparse_encode_src(BatchSrc{L.dsegs, L.dmap}, BatchSegSrc{L.dsegs}, L.ntiles, L.nsegs, dgc, ws, st);
+    if (L.single) return sparse_encode_src(SingleSrc{L.seg}, SingleSegSrc{L.seg}, L.ntiles, 1, dgc, ws, phase, st);
+    return sparse_encode_src(BatchSrc{L.dsegs, L.dmap}, BatchSegSrc{L.dsegs}, L.ntiles, L.nsegs, dgc, ws, phase, st);
 }
 
 hipError_t launch_sparse_decode(const Launch& L, hipStream_t st) {

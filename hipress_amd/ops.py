@@ -318,6 +318,11 @@ class Batch:
         with torch.cuda.device(self.device):
             check(_lib.lib().hipress_batch_encode(self._h, torch.cuda.current_stream(self.device).cuda_stream), "batch_encode")
 
+    def encode_phase(self, phase):
+        """One launch of the encode sequence (measurement aid)."""
+        with torch.cuda.device(self.device):
+            check(_lib.lib().hipress_batch_encode_phase(self._h, int(phase), torch.cuda.current_stream(self.device).cuda_stream), "batch_encode_phase")
+
     def decode(self):
         with torch.cuda.device(self.device):
             check(_lib.lib().hipress_batch_decode(self._h, torch.cuda.current_stream(self.device).cuda_stream), "batch_decode")

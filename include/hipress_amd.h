@@ -169,6 +169,12 @@ int hipress_batch_create(hipress_batch **out, int32_t alg, const hipress_tensor 
                          int32_t count, const hipress_params *params);
 int hipress_batch_encode(hipress_batch *batch, void *stream);
 int hipress_batch_decode(hipress_batch *batch, void *stream);
+/* Measurement aid: enqueues only launch number `phase` of the encode sequence, so
+ * that a caller can bracket one kernel with events.  onebit: 0 magnitude sum,
+ * 1 scale, 2 quantise; tbq, terngrad: 0; dgc, graddrop: 0 accumulate, 1 threshold,
+ * 2 count, 3 scan, 4 emit.  Running every phase in order equals
+ * hipress_batch_encode.  No counterpart in the reference. */
+int hipress_batch_encode_phase(hipress_batch *batch, int32_t phase, void *stream);
 int hipress_batch_destroy(hipress_batch *batch);
 
 /* One chunk of the aggregation step: npeers payloads of the same n. */
