@@ -202,9 +202,9 @@ def make_workload(name):
         return SetWorkload(name, "terngrad", vgg, "vgg", {"bucket": 512}, 8.2578, 4.2578, 0, "terngrad_encode_kernel", 8.2578)
     if name == "dgc_vgg19":
         return SetWorkload(name, "dgc", vgg, "vgg", {"momentum_factor": 0.9, "ratio": 0.001}, 20.0, 4.0, 0,
-                           "sparse_accum_kernel", 20.0, nphases=5)
+                           "sparse_accum_kernel", 20.0, nphases=7)
     if name == "graddrop_vgg19":
-        return SetWorkload(name, "graddrop", vgg, "vgg", {"ratio": 0.01}, 12.0, 4.0, 0, "sparse_accum_kernel", 12.0, nphases=5)
+        return SetWorkload(name, "graddrop", vgg, "vgg", {"ratio": 0.01}, 12.0, 4.0, 0, "sparse_accum_kernel", 12.0, nphases=7)
     if name == "tbq_262144":
         return SetWorkload(name, "tbq", [262144], "n0.02", {"threshold": 0.05}, 12.25, 4.25, 0, "tbq_encode_kernel", 12.25)
     if name == "tbq_262144_x512":
@@ -214,9 +214,9 @@ def make_workload(name):
                            8.2578, rotate=4)
     if name == "dgc_bert_large":
         return SetWorkload(name, "dgc", bert, "n1e-3", {"momentum_factor": 0.9, "ratio": 0.001}, 20.0, 4.0, 0,
-                           "sparse_accum_kernel", 20.0, nphases=5)
+                           "sparse_accum_kernel", 20.0, nphases=7)
     if name == "graddrop_bert_large":
-        return SetWorkload(name, "graddrop", bert, "n1e-3", {"ratio": 0.01}, 12.0, 4.0, 0, "sparse_accum_kernel", 12.0, nphases=5)
+        return SetWorkload(name, "graddrop", bert, "n1e-3", {"ratio": 0.01}, 12.0, 4.0, 0, "sparse_accum_kernel", 12.0, nphases=7)
     if name == "merge_tbq_vgg19":
         return MergeWorkload(name, "tbq", W.chunk_sizes(vgg))
     if name == "merge_dgc_vgg19":

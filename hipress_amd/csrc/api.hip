@@ -17,6 +17,7 @@ namespace {
 
 constexpr int64_t kSampleFrom = 262144;  // tensors at least this large are sampled at stride 100
 constexpr int64_t kSampleStride = 100;
+constexpr int64_t kSampleTile = 4096;    // sample keys per workgroup of the select passes
 
 inline bool mis(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
 inline bool al16(const void* p) { return !mis(p, 16); }
@@ -51,9 +52,9 @@ inline SparsePlan sparse_plan(int64_t n, double ratio) {
 
 inline bool bad_ratio(double r) { return !(r > 0.0 && r <= 1.0); }
 
-// Workspace of a sparse launch: four uint32 arrays, each starting on a 256-byte boundary.
+// Workspace of a sparse launch: six uint32 arrays, each starting on a 256-byte boundary.
 struct SparseWsLayout {
-    int64_t sample_off, gmax_off, counts_off, thr_off, bytes;
+    int64_t sample_off, gmax_off, counts_off, thr_off, hist_off, ctl_off, bytes;
 };
 
 inline SparseWsLayout sparse_ws_layout(int64_t total_ns, int64_t total_tiles, int64_t nsegs) {
@@ -64,9 +65,13 @@ inline SparseWsLayout sparse_ws_layout(int64_t total_ns, int64_t total_tiles, in
     l.gmax_off = off;
     off += round_up(4 * 64 * total_tiles, 256);
     l.counts_off = off;
-    off += round_up(4 * 8 * total_tiles, 256);
+    off += round_up(4 * 2 * total_tiles, 256);
     l.thr_off = off;
     off += round_up(4 * 2 * nsegs, 256);
+    l.hist_off = off;
+    off += round_up(4 * 3 * 2048 * nsegs, 256);
+    l.ctl_off = off;
+    off += round_up(4 * 8 * nsegs, 256);
     l.bytes = off;
     return l;
 }
@@ -78,6 +83,8 @@ inline SparseWs sparse_ws_at(void* base, const SparseWsLayout& l) {
     w.gmax = reinterpret_cast<uint32_t*>(b + l.gmax_off);
     w.counts = reinterpret_cast<uint32_t*>(b + l.counts_off);
     w.thr = reinterpret_cast<uint32_t*>(b + l.thr_off);
+    w.hist = reinterpret_cast<uint32_t*>(b + l.hist_off);
+    w.ctl = reinterpret_cast<uint32_t*>(b + l.ctl_off);
     return w;
 }
 
@@ -172,6 +179,7 @@ int build_encode_seg(int alg, const hipress_tensor& t, const hipress_params& pr,
             s->sstride = (unsigned)p.stride;
             s->ns = (unsigned)p.ns;
             s->ks = (unsigned)p.ks;
+            s->nsblk = (unsigned)((p.ns + kSampleTile - 1) / kSampleTile);
             break;
         }
     }
@@ -267,6 +275,20 @@ int layout_tiles(std::vector<S>& segs, GetSeg seg_of, std::vector<uint2>& map, u
     return HIPRESS_OK;
 }
 
+// Sparse launches: gives every tensor its slice of the sample array and builds the
+// workgroup -> (tensor, sample tile) map of the select passes.
+int64_t layout_samples(std::vector<Seg>& segs, std::vector<uint2>& smap) {
+    uint64_t off = 0;
+    smap.clear();
+    for (size_t i = 0; i < segs.size(); ++i) {
+        Seg& s = segs[i];
+        s.ws0 = off;
+        off += (s.ns + 3u) & ~3ull;
+        for (unsigned j = 0; j < s.nsblk; ++j) smap.push_back(make_uint2((unsigned)i, j));
+    }
+    return (int64_t)off;
+}
+
 }  // namespace
 
 // ============================================================================
@@ -281,7 +303,8 @@ struct hipress_batch {
     Seg* d_enc = nullptr;
     Seg* d_dec = nullptr;
     uint2* d_map = nullptr;
-    unsigned ntiles = 0;
+    uint2* d_smap = nullptr;  // sparse: sample tiles
+    unsigned ntiles = 0, nstiles = 0;
     void* ws = nullptr;  // onebit: one float per tile; sparse: SparseWsLayout
     SparseWsLayout swl{};
 };
@@ -296,7 +319,8 @@ struct hipress_merge_batch {
     MergeSeg* d_segs = nullptr;
     Seg* d_renc = nullptr;
     uint2* d_map = nullptr;
-    unsigned ntiles = 0;
+    uint2* d_smap = nullptr;
+    unsigned ntiles = 0, nstiles = 0;
     void* ws = nullptr;
     SparseWsLayout swl{};
 };
@@ -567,6 +591,7 @@ int hipress_batch_destroy(hipress_batch* b) {
     (void)hipFree(b->d_enc);
     (void)hipFree(b->d_dec);
     (void)hipFree(b->d_map);
+    (void)hipFree(b->d_smap);
     (void)hipFree(b->ws);
     delete b;
     return HIPRESS_OK;
@@ -615,13 +640,12 @@ int hipress_batch_create(hipress_batch** out, int32_t alg, const hipress_tensor*
     if (enc_ok && (rc = layout_tiles(b->enc, ident, map, &b->ntiles))) return fail(rc);
     if (dec_ok && (rc = layout_tiles(b->dec, ident, map, &b->ntiles))) return fail(rc);
     if (enc_ok && sparse) {
-        uint64_t off = 0;
-        for (Seg& s : b->enc) {
-            s.ws0 = off;
-            off += (s.ns + 3u) & ~3ull;
-        }
-        b->swl = sparse_ws_layout((int64_t)off, b->ntiles, count);
+        std::vector<uint2> smap;
+        int64_t total_ns = layout_samples(b->enc, smap);
+        b->nstiles = (unsigned)smap.size();
+        b->swl = sparse_ws_layout(total_ns, b->ntiles, count);
         if (b->swl.bytes && hipMalloc(&b->ws, (size_t)b->swl.bytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
+        if ((rc = upload(smap, &b->d_smap))) return fail(rc);
     } else if (enc_ok && alg == HIPRESS_ONEBIT) {
         if (hipMalloc(&b->ws, (size_t)round_up(4 * (int64_t)(b->ntiles ? b->ntiles : 1), 256)) != hipSuccess) return fail(HIPRESS_ERR_HIP);
     }
@@ -638,7 +662,9 @@ static Launch batch_launch(const hipress_batch* b, bool encode) {
     L.single = false;
     L.dsegs = encode ? b->d_enc : b->d_dec;
     L.dmap = b->d_map;
+    L.dsmap = b->d_smap;
     L.ntiles = b->ntiles;
+    L.nstiles = b->nstiles;
     L.nsegs = (unsigned)(encode ? b->enc.size() : b->dec.size());
     return L;
 }
@@ -661,7 +687,7 @@ static int batch_encode_impl(hipress_batch* b, int phase, void* stream) {
             return hiperr(launch_terngrad_encode(L, (unsigned)b->params.bucket, st));
         case HIPRESS_DGC:
         case HIPRESS_GRADDROP:
-            if (phase > 4) return HIPRESS_ERR_PARAM;
+            if (phase > 6) return HIPRESS_ERR_PARAM;
             return hiperr(launch_sparse_encode(L, b->alg == HIPRESS_DGC, sparse_ws_at(b->ws, b->swl), phase, st));
     }
     return HIPRESS_ERR_PARAM;
@@ -697,6 +723,7 @@ int hipress_merge_batch_destroy(hipress_merge_batch* b) {
     (void)hipFree(b->d_segs);
     (void)hipFree(b->d_renc);
     (void)hipFree(b->d_map);
+    (void)hipFree(b->d_smap);
     (void)hipFree(b->ws);
     delete b;
     return HIPRESS_OK;
@@ -745,13 +772,12 @@ int hipress_merge_batch_create(hipress_merge_batch** out, int32_t alg, const hip
         std::vector<uint2> map2;
         unsigned nt2;
         if ((rc = layout_tiles(b->renc, [](Seg& s) -> Seg& { return s; }, map2, &nt2))) return fail(rc);
-        uint64_t off = 0;
-        for (Seg& s : b->renc) {
-            s.ws0 = off;
-            off += (s.ns + 3u) & ~3ull;
-        }
-        b->swl = sparse_ws_layout((int64_t)off, b->ntiles, count);
+        std::vector<uint2> smap;
+        int64_t total_ns = layout_samples(b->renc, smap);
+        b->nstiles = (unsigned)smap.size();
+        b->swl = sparse_ws_layout(total_ns, b->ntiles, count);
         if (b->swl.bytes && hipMalloc(&b->ws, (size_t)b->swl.bytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
+        if ((rc = upload(smap, &b->d_smap))) return fail(rc);
     }
     if ((rc = upload(b->segs, &b->d_segs))) return fail(rc);
     if ((rc = upload(b->renc, &b->d_renc))) return fail(rc);
@@ -782,6 +808,8 @@ int hipress_merge_batch_run(hipress_merge_batch* b, void* stream) {
             R.single = false;
             R.dsegs = b->d_renc;
             R.dmap = b->d_map;  // same tensors, same tile numbering
+            R.dsmap = b->d_smap;
+            R.nstiles = b->nstiles;
             R.ntiles = b->ntiles;
             R.nsegs = (unsigned)b->renc.size();
             e = launch_sparse_encode(R, false, sparse_ws_at(b->ws, b->swl), -1, st);

@@ -45,7 +45,7 @@ struct Seg {
     unsigned int ns;         // sparse: sample count
     unsigned long long ws0;  // sparse: element offset of this tensor's sample slice
     unsigned int id;         // index of this tensor in the launch's table
-    unsigned int pad0;
+    unsigned int nsblk;      // sparse: workgroups the select passes spend on this tensor
     unsigned long long pay_bytes;  // size of the payload buffer (decode-side bounds checks)
 };
 
@@ -191,7 +191,9 @@ struct Launch {
     Seg seg;              // single
     const Seg* dsegs;     // batch: device table
     const uint2* dmap;    // batch: device tile map
+    const uint2* dsmap;   // batch, sparse: device map of sample tiles
     unsigned ntiles;      // workgroups to launch
+    unsigned nstiles;     // batch, sparse: sample tiles
     unsigned nsegs;       // tensors in the table (1 for single)
 };
 

@@ -18,8 +18,10 @@ hipError_t launch_dense_merge(const MergeLaunch& L, int alg, hipStream_t st);
 struct SparseWs {
     uint32_t* sample;   // |acc'| keys at the sample positions, all tensors back to back
     uint32_t* gmax;     // max |acc'| key of every 64-element group: 64 per tile
-    uint32_t* counts;   // per wavefront-tile {above, equal} counts, then their exclusive scans
+    uint32_t* counts;   // per tile {above, equal} counts, then their exclusive scans
     uint32_t* thr;      // per tensor {threshold key, equal-quota}
+    uint32_t* hist;     // per tensor 3 x 2048 bins, one histogram per select pass
+    uint32_t* ctl;      // per tensor 8 words: select prefix, remaining rank, done counters
 };
 hipError_t launch_sparse_encode(const Launch& L, bool dgc, const SparseWs& ws, int phase, hipStream_t st);
 hipError_t launch_sparse_decode(const Launch& L, hipStream_t st);

@@ -1,18 +1,22 @@
 // Sampled-threshold sparsifiers for gfx950: DGC and GradDrop encode, the shared
 // sparse decode, and the scatter-add half of sparse decode-and-merge.
 //
-// Encode is five launches over the whole tensor set:
-//   1. accumulate   one streaming pass: mom' = m*mom + g, acc' = acc + mom'
+// Encode is seven launches over the whole tensor set:
+//   0. accumulate   one streaming pass: mom' = m*mom + g, acc' = acc + mom'
 //                   (GradDrop: acc' = acc + g), written back; the |acc'| keys at
 //                   the sample positions are gathered and the maximum key of
 //                   every 64-element group is recorded on the way;
-//   2. threshold    one workgroup per tensor selects the k-th largest sample key;
-//   3. count        only groups whose maximum reaches the threshold are read
-//                   again; per wavefront-tile counts of keys above / equal to it;
-//   4. scan         one workgroup per tensor turns the counts into output
+//   1-3. select     the k-th largest sample key of every tensor by radix
+//                   selection, 11 + 10 + 10 bits from the top: every pass is one
+//                   launch over all sample tiles, LDS histograms merged into a
+//                   per-tensor global one, the last workgroup of a tensor to
+//                   finish picks the digit;
+//   4. count        only groups whose maximum reaches the threshold are read
+//                   again; per-tile counts of keys above / equal to it;
+//   5. scan         one workgroup per tensor turns the counts into output
 //                   offsets, writes the header and, if more than `capacity`
 //                   elements qualify, re-thresholds on the whole tensor;
-//   5. emit         the flagged groups are read once more and the selected
+//   6. emit         the flagged groups are read once more and the selected
 //                   (index, value) pairs are written in ascending index order,
 //                   the accumulator (and momentum) being zeroed at those places.
 // |x| is handled as the integer key bits(x) & 0x7fffffff, which orders like |x|.
@@ -22,6 +26,8 @@
 namespace hp {
 
 constexpr unsigned kNoQuota = 0xffffffffu;
+constexpr int kSampleTile = 4096;  // sample keys per workgroup in the select passes
+constexpr int kBins = 2048;        // histogram bins per select pass (11-bit first digit)
 
 __device__ __forceinline__ unsigned key_of(float x) { return __float_as_uint(x) & 0x7fffffffu; }
 
@@ -40,7 +46,16 @@ __device__ __forceinline__ unsigned popc_lt(unsigned long long m, unsigned lane)
     return __popcll(m & ((1ull << lane) - 1ull));
 }
 
-// ---- 1. accumulate -------------------------------------------------------------
+// per-tensor control words of the select passes
+enum { kCtlPrefix = 0, kCtlK = 1, kCtlDone = 2 /* +pass */, kCtlWords = 8 };
+
+__device__ __forceinline__ unsigned digit_shift(int pass) { return pass == 0 ? 20u : (pass == 1 ? 10u : 0u); }
+__device__ __forceinline__ unsigned digit_bins(int pass) { return pass == 0 ? 2048u : 1024u; }
+__device__ __forceinline__ unsigned digit_mask_above(int pass) {
+    return pass == 0 ? 0u : (pass == 1 ? 0x7ff00000u : 0x7ffffc00u);
+}
+
+// ---- 0. accumulate -------------------------------------------------------------
 
 template <bool FAST, bool DGC>
 __device__ __forceinline__ void sparse_accum_tile(const Seg& s, unsigned tile, const SparseWs& ws) {
@@ -105,121 +120,144 @@ template <class Src, bool DGC>
 __global__ __launch_bounds__(kBlock) void sparse_accum_kernel(Src src, SparseWs ws) {
     unsigned tile;
     const Seg& s = src.get(tile, blockIdx.x);
+    if (tile == 0) {
+        // this tensor's select-pass state starts from zero every call
+        uint32_t* h = ws.hist + (unsigned long long)s.id * (3 * kBins);
+        for (unsigned i = threadIdx.x; i < 3 * kBins; i += kBlock) h[i] = 0;
+        if (threadIdx.x < kCtlWords) ws.ctl[s.id * kCtlWords + threadIdx.x] = threadIdx.x == kCtlK ? s.ks : 0u;
+        if (threadIdx.x == 0) {
+            ws.thr[2 * s.id] = 0;
+            ws.thr[2 * s.id + 1] = kNoQuota;
+        }
+    }
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) sparse_accum_tile<true, DGC>(s, tile, ws);
     else sparse_accum_tile<false, DGC>(s, tile, ws);
 }
 
-// ---- radix selection helper (one workgroup) ----------------------------------------
+// ---- 1-3. select -----------------------------------------------------------------
 
-// Finds the k-th largest (k >= 1) key among the keys a workgroup enumerates with
-// `visit(f)` (which must call f(key) for every candidate, the same set each time
-// it is invoked).  8-bit digits from the top; 16 interleaved histograms keep the
-// LDS atomics of neighbouring lanes apart.
-struct RadixScratch {
-    unsigned hist[16][257];
-    unsigned prefix, k;
-};
-
-template <class Visit>
-__device__ __forceinline__ unsigned block_kth_largest(RadixScratch& sc, unsigned k, Visit visit) {
-    unsigned prefix = 0, mask = 0;
-    for (int shift = 24; shift >= 0; shift -= 8) {
-        for (unsigned i = threadIdx.x; i < 16 * 257; i += kBlock) (&sc.hist[0][0])[i] = 0;
-        __syncthreads();
-        visit([&](unsigned key) {
-            if ((key & mask) == prefix) atomicAdd(&sc.hist[threadIdx.x & 15u][(key >> shift) & 255u], 1u);
-        });
-        __syncthreads();
-        // fold the 16 copies
-        {
-            unsigned t = threadIdx.x;  // kBlock == 256 bins
-            unsigned c = 0;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) c += sc.hist[r][t];
-            __syncthreads();
-            sc.hist[0][t] = c;
-        }
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            unsigned kk = k;
-            int d = 255;
-            for (; d > 0; --d) {
-                unsigned c = sc.hist[0][d];
-                if (kk <= c) break;
-                kk -= c;
-            }
-            sc.prefix = prefix | ((unsigned)d << shift);
-            sc.k = kk;
-        }
-        __syncthreads();
-        prefix = sc.prefix;
-        k = sc.k;
-        mask |= 0xffu << shift;
-        __syncthreads();
-    }
-    return prefix;
-}
-
-// ---- 2. threshold ----------------------------------------------------------------
-
-template <class SegSrc>
-__global__ __launch_bounds__(kBlock) void sparse_threshold_kernel(SegSrc src, SparseWs ws) {
-    __shared__ RadixScratch sc;
-    const Seg& s = src.at(blockIdx.x);
+// One radix pass.  Workgroup = one tile of kSampleTile sample keys of one tensor.
+template <class Src>
+__global__ __launch_bounds__(kBlock) void sparse_select_kernel(Src src, SparseWs ws, int pass) {
+    __shared__ unsigned lh[kBins];
+    __shared__ unsigned chunk[kBlock];
+    __shared__ unsigned is_last;
+    unsigned stile;
+    const Seg& s = src.get(stile, blockIdx.x);
     const uint32_t* keys = ws.sample + s.ws0;
-    const unsigned ns = s.ns;
-    unsigned thr = 0;
-    if (ns > 0) {
-        thr = block_kth_largest(sc, s.ks, [&](auto f) {
-            for (unsigned i = threadIdx.x; i < ns; i += kBlock) f(keys[i]);
-        });
+    uint32_t* ctl = ws.ctl + s.id * kCtlWords;
+    uint32_t* gh = ws.hist + ((unsigned long long)s.id * 3 + pass) * kBins;
+    const unsigned shift = digit_shift(pass), nb = digit_bins(pass), above = digit_mask_above(pass);
+    const unsigned prefix = pass ? ctl[kCtlPrefix] : 0u;
+    for (unsigned i = threadIdx.x; i < nb; i += kBlock) lh[i] = 0;
+    __syncthreads();
+    const unsigned long long lo = (unsigned long long)stile * kSampleTile;
+#pragma unroll 4
+    for (int j = 0; j < kSampleTile / kBlock; ++j) {
+        unsigned long long i = lo + j * kBlock + threadIdx.x;
+        if (i < s.ns) {
+            unsigned key = keys[i];
+            if ((key & above) == prefix) atomicAdd(&lh[(key >> shift) & (nb - 1)], 1u);
+        }
     }
+    __syncthreads();
+    for (unsigned i = threadIdx.x; i < nb; i += kBlock) {
+        unsigned c = lh[i];
+        if (c) atomicAdd(&gh[i], c);
+    }
+    // Everything workgroups exchange here travels through device-scope atomics
+    // (the histogram adds above, the ticket below, the atomic loads after it), so
+    // no cache write-back is needed: the barrier waits until this workgroup's
+    // adds have been performed, and only then is its ticket taken.
+    __syncthreads();
+    if (threadIdx.x == 0) is_last = atomicAdd(&ctl[kCtlDone + pass], 1u) == s.nsblk - 1;
+    __syncthreads();
+    if (!is_last) return;
+    // Every other workgroup of this tensor has merged its histogram: pick the digit
+    // that holds the k-th largest key, walking the bins from the top.
+    for (unsigned i = threadIdx.x; i < nb; i += kBlock)
+        lh[i] = __hip_atomic_load(&gh[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const unsigned per = nb / kBlock;  // bins per thread, thread t owns the t-th chunk from the top
+    {
+        unsigned c = 0;
+        for (unsigned b = 0; b < per; ++b) c += lh[nb - 1 - (threadIdx.x * per + b)];
+        chunk[threadIdx.x] = c;
+    }
+    __syncthreads();
     if (threadIdx.x == 0) {
-        ws.thr[2 * s.id] = thr;
-        ws.thr[2 * s.id + 1] = kNoQuota;
+        unsigned k = pass ? ctl[kCtlK] : s.ks;
+        unsigned t = 0;
+        for (; t < kBlock - 1; ++t) {
+            if (k <= chunk[t]) break;
+            k -= chunk[t];
+        }
+        unsigned d = nb - 1 - t * per;
+        for (unsigned b = 0; b < per - 1; ++b, --d) {
+            unsigned c = lh[d];
+            if (k <= c) break;
+            k -= c;
+        }
+        unsigned np = prefix | (d << shift);
+        ctl[kCtlPrefix] = np;
+        ctl[kCtlK] = k;
+        if (pass == 2) ws.thr[2 * s.id] = np;
     }
 }
 
-// ---- 3. count ---------------------------------------------------------------------
+// ---- 4. count ---------------------------------------------------------------------
 
-// Counts, for the wavefront-tile wt (1024 elements) of tensor s, the keys above
-// and equal to thr; only 64-element groups whose maximum reaches thr are read.
-// Wavefront-uniform result.
-__device__ __forceinline__ void count_wavetile(const Seg& s, const SparseWs& ws, unsigned long long wt,
-                                               unsigned thr, unsigned lane, unsigned& gt, unsigned& eq) {
+// Counts, for tile `tile` (4096 elements) of tensor s, the keys above and equal
+// to thr; lane l looks at the maximum of 64-element group l and only groups
+// whose maximum reaches thr are read.  Wavefront-uniform result.
+__device__ __forceinline__ void count_tile(const Seg& s, const SparseWs& ws, unsigned tile, unsigned thr,
+                                           unsigned lane, unsigned& gt, unsigned& eq) {
     const long long n = (long long)s.n;
-    const unsigned long long g0 = (unsigned long long)s.tile0 * 64 + wt * 16;
-    unsigned gm = lane < 16 ? ws.gmax[g0 + lane] : 0u;
+    unsigned gm = ws.gmax[(unsigned long long)(s.tile0 + tile) * 64 + lane];
     unsigned long long mask = __ballot(gm >= thr && gm > 0u);
+    const long long base = (long long)tile * kTile + lane;
     gt = 0;
     eq = 0;
     while (mask) {
-        unsigned gi = __ffsll((long long)mask) - 1;
-        mask &= mask - 1;
-        long long e = (long long)wt * kWaveTile + gi * 64 + lane;
-        unsigned key = e < n ? key_of(s.s1[e]) : 0u;
-        gt += __popcll(__ballot(key > thr));
-        eq += __popcll(__ballot(key == thr && key > 0u));
+        // up to four flagged groups per round, their loads in flight together
+        unsigned gi[4], key[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            gi[k] = mask ? (unsigned)__ffsll((long long)mask) - 1 : 64u;
+            mask &= mask - 1;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            long long e = base + gi[k] * 64;
+            key[k] = (gi[k] < 64u && e < n) ? key_of(s.s1[e]) : 0u;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            gt += __popcll(__ballot(key[k] > thr));
+            eq += __popcll(__ballot(key[k] == thr && key[k] > 0u));
+        }
     }
 }
 
+// One wavefront per tile, four tiles per workgroup.
 template <class Src>
-__global__ __launch_bounds__(kBlock) void sparse_count_kernel(Src src, SparseWs ws) {
-    unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+__global__ __launch_bounds__(kBlock) void sparse_count_kernel(Src src, SparseWs ws, unsigned total_tiles) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned gt_idx = blockIdx.x * 4 + wave;
+    if (gt_idx >= total_tiles) return;
+    unsigned tile;
+    const Seg& s = src.get(tile, gt_idx);
     const unsigned thr = ws.thr[2 * s.id];
     unsigned gt, eq;
-    const unsigned long long wt = (unsigned long long)tile * 4 + wave;
-    count_wavetile(s, ws, wt, thr, lane, gt, eq);
+    count_tile(s, ws, tile, thr, lane, gt, eq);
     if (lane == 0) {
-        unsigned long long c = ((unsigned long long)s.tile0 * 4 + wt) * 2;
+        unsigned long long c = (unsigned long long)(s.tile0 + tile) * 2;
         ws.counts[c] = gt;
         ws.counts[c + 1] = eq;
     }
 }
 
-// ---- 4. scan ----------------------------------------------------------------------
+// ---- 5. scan ----------------------------------------------------------------------
 
 // In-place exclusive scan of nw {above, equal} pairs by one workgroup; returns
 // the totals to every thread.
@@ -261,14 +299,62 @@ __device__ __forceinline__ void block_scan_pairs(uint32_t* c, unsigned nw, unsig
     __syncthreads();
 }
 
+// k-th largest (k >= 1) key among the keys a workgroup enumerates with visit(f)
+// (which must call f(key) for every candidate, the same set each time it is
+// invoked).  8-bit digits from the top; 16 interleaved histograms keep the LDS
+// atomics of neighbouring lanes apart.  Only the overflow path uses it.
+struct RadixScratch {
+    unsigned hist[16][257];
+    unsigned prefix, k;
+};
+
+template <class Visit>
+__device__ __forceinline__ unsigned block_kth_largest(RadixScratch& sc, unsigned k, Visit visit) {
+    unsigned prefix = 0, mask = 0;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        for (unsigned i = threadIdx.x; i < 16 * 257; i += kBlock) (&sc.hist[0][0])[i] = 0;
+        __syncthreads();
+        visit([&](unsigned key) {
+            if ((key & mask) == prefix) atomicAdd(&sc.hist[threadIdx.x & 15u][(key >> shift) & 255u], 1u);
+        });
+        __syncthreads();
+        {
+            unsigned t = threadIdx.x;  // kBlock == 256 bins: fold the 16 copies
+            unsigned c = 0;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) c += sc.hist[r][t];
+            __syncthreads();
+            sc.hist[0][t] = c;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            unsigned kk = k;
+            int d = 255;
+            for (; d > 0; --d) {
+                unsigned c = sc.hist[0][d];
+                if (kk <= c) break;
+                kk -= c;
+            }
+            sc.prefix = prefix | ((unsigned)d << shift);
+            sc.k = kk;
+        }
+        __syncthreads();
+        prefix = sc.prefix;
+        k = sc.k;
+        mask |= 0xffu << shift;
+        __syncthreads();
+    }
+    return prefix;
+}
+
 template <class SegSrc>
 __global__ __launch_bounds__(kBlock) void sparse_scan_kernel(SegSrc src, SparseWs ws) {
     __shared__ unsigned sh[2][kBlock];
     __shared__ RadixScratch sc;
     const Seg& s = src.at(blockIdx.x);
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const unsigned nw = s.ntiles * 4;
-    uint32_t* c = ws.counts + (unsigned long long)s.tile0 * 8;
+    const unsigned nw = s.ntiles;
+    uint32_t* c = ws.counts + (unsigned long long)s.tile0 * 2;
     unsigned thr = ws.thr[2 * s.id];
     unsigned quota = kNoQuota;
     unsigned tot_gt, tot_eq;
@@ -293,12 +379,12 @@ __global__ __launch_bounds__(kBlock) void sparse_scan_kernel(SegSrc src, SparseW
                 }
             }
         });
-        for (unsigned long long wt = wave; wt < nw; wt += 4) {
+        for (unsigned t = wave; t < nw; t += 4) {
             unsigned gt, eq;
-            count_wavetile(s, ws, wt, thr, lane, gt, eq);
+            count_tile(s, ws, t, thr, lane, gt, eq);
             if (lane == 0) {
-                c[2 * wt] = gt;
-                c[2 * wt + 1] = eq;
+                c[2 * t] = gt;
+                c[2 * t + 1] = eq;
             }
         }
         __syncthreads();
@@ -317,46 +403,59 @@ __global__ __launch_bounds__(kBlock) void sparse_scan_kernel(SegSrc src, SparseW
     }
 }
 
-// ---- 5. emit ----------------------------------------------------------------------
+// ---- 6. emit ----------------------------------------------------------------------
 
 template <class Src>
-__global__ __launch_bounds__(kBlock) void sparse_emit_kernel(Src src, SparseWs ws) {
-    unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+__global__ __launch_bounds__(kBlock) void sparse_emit_kernel(Src src, SparseWs ws, unsigned total_tiles) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned gt_idx = blockIdx.x * 4 + wave;
+    if (gt_idx >= total_tiles) return;
+    unsigned tile;
+    const Seg& s = src.get(tile, gt_idx);
     const long long n = (long long)s.n;
     const unsigned thr = ws.thr[2 * s.id], quota = ws.thr[2 * s.id + 1];
-    const unsigned long long wt = (unsigned long long)tile * 4 + wave;
-    const unsigned long long ci = ((unsigned long long)s.tile0 * 4 + wt) * 2;
+    const unsigned long long ci = (unsigned long long)(s.tile0 + tile) * 2;
     const unsigned G = ws.counts[ci], E = ws.counts[ci + 1];
-    unsigned pos = G + (E < quota ? E : quota);  // pairs written by earlier wavefront-tiles
+    unsigned pos = G + (E < quota ? E : quota);  // pairs written by earlier tiles
     unsigned eq_seen = E;
     int32_t* idx = reinterpret_cast<int32_t*>(s.pay + kHeaderBytes);
     float* val = reinterpret_cast<float*>(s.pay + kHeaderBytes + 4ull * s.cap);
-    const unsigned long long g0 = (unsigned long long)s.tile0 * 64 + wt * 16;
-    unsigned gm = lane < 16 ? ws.gmax[g0 + lane] : 0u;
+    unsigned gm = ws.gmax[(unsigned long long)(s.tile0 + tile) * 64 + lane];
     unsigned long long mask = __ballot(gm >= thr && gm > 0u);
+    const long long base = (long long)tile * kTile + lane;
     while (mask) {
-        unsigned gi = __ffsll((long long)mask) - 1;
-        mask &= mask - 1;
-        long long e = (long long)wt * kWaveTile + gi * 64 + lane;
-        float v = e < n ? s.s1[e] : 0.f;
-        unsigned key = key_of(v);
-        bool is_eq = key == thr && key > 0u;
-        unsigned long long m_eq = __ballot(is_eq);
-        bool sel = key > thr || (is_eq && eq_seen + popc_lt(m_eq, lane) < quota);
-        unsigned long long m_sel = __ballot(sel);
-        if (sel) {
-            unsigned p = pos + popc_lt(m_sel, lane);
-            if (p < s.cap) {
-                idx[p] = (int32_t)e;
-                val[p] = v;
-                s.s1[e] = 0.f;
-                if (s.s0) s.s0[e] = 0.f;
-            }
+        unsigned gi[4];
+        float v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            gi[k] = mask ? (unsigned)__ffsll((long long)mask) - 1 : 64u;
+            mask &= mask - 1;
         }
-        pos += __popcll(m_sel);
-        eq_seen += __popcll(m_eq);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            long long e = base + gi[k] * 64;
+            v[k] = (gi[k] < 64u && e < n) ? s.s1[e] : 0.f;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            long long e = base + gi[k] * 64;
+            unsigned key = key_of(v[k]);
+            bool is_eq = key == thr && key > 0u;
+            unsigned long long m_eq = __ballot(is_eq);
+            bool sel = key > thr || (is_eq && eq_seen + popc_lt(m_eq, lane) < quota);
+            unsigned long long m_sel = __ballot(sel);
+            if (sel) {
+                unsigned p = pos + popc_lt(m_sel, lane);
+                if (p < s.cap) {
+                    idx[p] = (int32_t)e;
+                    val[p] = v[k];
+                    s.s1[e] = 0.f;
+                    if (s.s0) s.s0[e] = 0.f;
+                }
+            }
+            pos += __popcll(m_sel);
+            eq_seen += __popcll(m_eq);
+        }
     }
 }
 
@@ -443,26 +542,33 @@ __global__ __launch_bounds__(kBlock) void merge_zero_fill_kernel(MSrc src) {
 // =============================================================================
 
 template <class Src, class SegSrcT>
-static hipError_t sparse_encode_src(const Src& src, const SegSrcT& ssrc, unsigned ntiles, unsigned nsegs,
-                                    bool dgc, const SparseWs& ws, int phase, hipStream_t st) {
+static hipError_t sparse_encode_src(const Src& src, const Src& ssrc_tiles, const SegSrcT& ssrc, unsigned ntiles,
+                                    unsigned nstiles, unsigned nsegs, bool dgc, const SparseWs& ws, int phase,
+                                    hipStream_t st) {
     auto on = [&](int p) { return phase < 0 || phase == p; };
+    const unsigned g4 = (ntiles + 3) / 4;
     if (on(0)) {
         if (dgc) hipLaunchKernelGGL((sparse_accum_kernel<Src, true>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
         else hipLaunchKernelGGL((sparse_accum_kernel<Src, false>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
     }
-    if (on(1)) hipLaunchKernelGGL((sparse_threshold_kernel<SegSrcT>), dim3(nsegs), dim3(kBlock), 0, st, ssrc, ws);
-    if (on(2)) hipLaunchKernelGGL((sparse_count_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
-    if (on(3)) hipLaunchKernelGGL((sparse_scan_kernel<SegSrcT>), dim3(nsegs), dim3(kBlock), 0, st, ssrc, ws);
-    if (on(4)) hipLaunchKernelGGL((sparse_emit_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
+    for (int pass = 0; pass < 3; ++pass)
+        if (on(1 + pass) && nstiles)
+            hipLaunchKernelGGL((sparse_select_kernel<Src>), dim3(nstiles), dim3(kBlock), 0, st, ssrc_tiles, ws, pass);
+    if (on(4)) hipLaunchKernelGGL((sparse_count_kernel<Src>), dim3(g4), dim3(kBlock), 0, st, src, ws, ntiles);
+    if (on(5)) hipLaunchKernelGGL((sparse_scan_kernel<SegSrcT>), dim3(nsegs), dim3(kBlock), 0, st, ssrc, ws);
+    if (on(6)) hipLaunchKernelGGL((sparse_emit_kernel<Src>), dim3(g4), dim3(kBlock), 0, st, src, ws, ntiles);
     return hipGetLastError();
 }
 
-// phase < 0 runs the whole sequence; 0..4 run one launch of it (accumulate,
-// threshold, count, scan, emit).
+// phase < 0 runs the whole sequence; 0..6 run one launch of it (accumulate,
+// three select passes, count, scan, emit).
 hipError_t launch_sparse_encode(const Launch& L, bool dgc, const SparseWs& ws, int phase, hipStream_t st) {
     if (L.ntiles == 0) return hipSuccess;
-    if (L.single) return sparse_encode_src(SingleSrc{L.seg}, SingleSegSrc{L.seg}, L.ntiles, 1, dgc, ws, phase, st);
-    return sparse_encode_src(BatchSrc{L.dsegs, L.dmap}, BatchSegSrc{L.dsegs}, L.ntiles, L.nsegs, dgc, ws, phase, st);
+    if (L.single)
+        return sparse_encode_src(SingleSrc{L.seg}, SingleSrc{L.seg}, SingleSegSrc{L.seg}, L.ntiles, L.seg.nsblk, 1, dgc,
+                                 ws, phase, st);
+    return sparse_encode_src(BatchSrc{L.dsegs, L.dmap}, BatchSrc{L.dsegs, L.dsmap}, BatchSegSrc{L.dsegs}, L.ntiles,
+                             L.nstiles, L.nsegs, dgc, ws, phase, st);
 }
 
 hipError_t launch_sparse_decode(const Launch& L, hipStream_t st) {

@@ -171,8 +171,8 @@ int hipress_batch_encode(hipress_batch *batch, void *stream);
 int hipress_batch_decode(hipress_batch *batch, void *stream);
 /* Measurement aid: enqueues only launch number `phase` of the encode sequence, so
  * that a caller can bracket one kernel with events.  onebit: 0 magnitude sum,
- * 1 scale, 2 quantise; tbq, terngrad: 0; dgc, graddrop: 0 accumulate, 1 threshold,
- * 2 count, 3 scan, 4 emit.  Running every phase in order equals
+ * 1 scale, 2 quantise; tbq, terngrad: 0; dgc, graddrop: 0 accumulate, 1-3 the
+ * three radix-select passes of the threshold, 4 count, 5 scan, 6 emit.  Running every phase in order equals
  * hipress_batch_encode.  No counterpart in the reference. */
 int hipress_batch_encode_phase(hipress_batch *batch, int32_t phase, void *stream);
 int hipress_batch_destroy(hipress_batch *batch);

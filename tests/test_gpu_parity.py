@@ -216,6 +216,25 @@ def test_graddrop_encode_decode(hp, n):
         np.testing.assert_array_equal(host(out), oracle.sparse_decode(want_pay, n))
 
 
+def test_sparse_threshold_many_sample_tiles(hp):
+    """24M elements: 240,000 sample keys = 59 sample tiles, so the per-tensor
+    histogram is merged from workgroups on every XCD."""
+    n = 24_000_000
+    g = np.random.default_rng(12).normal(0, 1e-3, n).astype(F)
+    for ratio, enc in ((0.001, "dgc"), (0.01, "graddrop")):
+        pay = payload(hp.sparse_payload_bytes(n, ratio))
+        acc = torch.zeros(n, device="cuda")
+        if enc == "dgc":
+            mom = torch.zeros(n, device="cuda")
+            hp.dgc_encode(dev(g), mom, acc, pay, 0.9, ratio)
+            want_pay, _, want_acc = oracle.dgc_encode(g, np.zeros(n, F), np.zeros(n, F), 0.9, ratio)
+        else:
+            hp.graddrop_encode(dev(g), acc, pay, ratio)
+            want_pay, want_acc = oracle.graddrop_encode(g, np.zeros(n, F), ratio)
+        check_sparse(host(pay), want_pay)
+        np.testing.assert_array_equal(host(acc), want_acc)
+
+
 def test_sparse_overflow_ties(hp):
     n = 10000
     g = np.full(n, 0.5, F)
