@@ -214,6 +214,7 @@ int build_decode_seg(int alg, const void* payload, int64_t payload_bytes, float*
         case HIPRESS_GRADDROP: {
             int64_t slots = (payload_bytes - HIPRESS_HEADER_BYTES) / 8;
             s->cap = (unsigned)(slots > 0xffffffffLL ? 0xffffffffLL : slots);
+            s->ncblk = (unsigned)(((int64_t)s->cap + 1023) / 1024);
             break;
         }
         default: return HIPRESS_ERR_PARAM;
@@ -304,7 +305,8 @@ struct hipress_batch {
     Seg* d_dec = nullptr;
     uint2* d_map = nullptr;
     uint2* d_smap = nullptr;  // sparse: sample tiles
-    unsigned ntiles = 0, nstiles = 0;
+    uint2* d_cmap = nullptr;  // sparse decode: payload-slot tiles
+    unsigned ntiles = 0, nstiles = 0, nctiles = 0;
     void* ws = nullptr;  // onebit: one float per tile; sparse: SparseWsLayout
     SparseWsLayout swl{};
 };
@@ -592,6 +594,7 @@ int hipress_batch_destroy(hipress_batch* b) {
     (void)hipFree(b->d_dec);
     (void)hipFree(b->d_map);
     (void)hipFree(b->d_smap);
+    (void)hipFree(b->d_cmap);
     (void)hipFree(b->ws);
     delete b;
     return HIPRESS_OK;
@@ -649,6 +652,13 @@ int hipress_batch_create(hipress_batch** out, int32_t alg, const hipress_tensor*
     } else if (enc_ok && alg == HIPRESS_ONEBIT) {
         if (hipMalloc(&b->ws, (size_t)round_up(4 * (int64_t)(b->ntiles ? b->ntiles : 1), 256)) != hipSuccess) return fail(HIPRESS_ERR_HIP);
     }
+    if (dec_ok && sparse) {
+        std::vector<uint2> cmap;
+        for (size_t i = 0; i < b->dec.size(); ++i)
+            for (unsigned j = 0; j < b->dec[i].ncblk; ++j) cmap.push_back(make_uint2((unsigned)i, j));
+        b->nctiles = (unsigned)cmap.size();
+        if ((rc = upload(cmap, &b->d_cmap))) return fail(rc);
+    }
     if ((rc = upload(b->enc, &b->d_enc))) return fail(rc);
     if ((rc = upload(b->dec, &b->d_dec))) return fail(rc);
     if ((rc = upload(map, &b->d_map))) return fail(rc);
@@ -663,8 +673,10 @@ static Launch batch_launch(const hipress_batch* b, bool encode) {
     L.dsegs = encode ? b->d_enc : b->d_dec;
     L.dmap = b->d_map;
     L.dsmap = b->d_smap;
+    L.dcmap = b->d_cmap;
     L.ntiles = b->ntiles;
     L.nstiles = b->nstiles;
+    L.nctiles = b->nctiles;
     L.nsegs = (unsigned)(encode ? b->enc.size() : b->dec.size());
     return L;
 }

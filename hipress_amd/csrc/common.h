@@ -46,6 +46,8 @@ struct Seg {
     unsigned long long ws0;  // sparse: element offset of this tensor's sample slice
     unsigned int id;         // index of this tensor in the launch's table
     unsigned int nsblk;      // sparse: workgroups the select passes spend on this tensor
+    unsigned int ncblk;      // sparse decode: workgroups of 1024 payload slots
+    unsigned int pad0;
     unsigned long long pay_bytes;  // size of the payload buffer (decode-side bounds checks)
 };
 
@@ -192,8 +194,10 @@ struct Launch {
     const Seg* dsegs;     // batch: device table
     const uint2* dmap;    // batch: device tile map
     const uint2* dsmap;   // batch, sparse: device map of sample tiles
+    const uint2* dcmap;   // batch, sparse decode: device map of payload-slot tiles
     unsigned ntiles;      // workgroups to launch
     unsigned nstiles;     // batch, sparse: sample tiles
+    unsigned nctiles;     // batch, sparse decode: payload-slot tiles
     unsigned nsegs;       // tensors in the table (1 for single)
 };
 

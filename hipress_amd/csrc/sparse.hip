@@ -149,6 +149,7 @@ __global__ __launch_bounds__(kBlock) void sparse_select_kernel(Src src, SparseWs
     uint32_t* gh = ws.hist + ((unsigned long long)s.id * 3 + pass) * kBins;
     const unsigned shift = digit_shift(pass), nb = digit_bins(pass), above = digit_mask_above(pass);
     const unsigned prefix = pass ? ctl[kCtlPrefix] : 0u;
+    const unsigned k = pass ? ctl[kCtlK] : s.ks;  // read before the barriers; the owner below rewrites it
     for (unsigned i = threadIdx.x; i < nb; i += kBlock) lh[i] = 0;
     __syncthreads();
     const unsigned long long lo = (unsigned long long)stile * kSampleTile;
@@ -179,64 +180,90 @@ __global__ __launch_bounds__(kBlock) void sparse_select_kernel(Src src, SparseWs
         lh[i] = __hip_atomic_load(&gh[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     const unsigned per = nb / kBlock;  // bins per thread, thread t owns the t-th chunk from the top
-    {
-        unsigned c = 0;
-        for (unsigned b = 0; b < per; ++b) c += lh[nb - 1 - (threadIdx.x * per + b)];
-        chunk[threadIdx.x] = c;
+    unsigned mine = 0;
+    for (unsigned b = 0; b < per; ++b) mine += lh[nb - 1 - (threadIdx.x * per + b)];
+    // exclusive prefix of the chunk sums, from the top: wavefront scan, then the
+    // four wavefront totals through LDS
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    unsigned incl = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        unsigned y = (unsigned)__shfl_up((int)incl, d, 64);
+        if ((int)lane >= d) incl += y;
     }
+    if (lane == 63) chunk[wave] = incl;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned k = pass ? ctl[kCtlK] : s.ks;
-        unsigned t = 0;
-        for (; t < kBlock - 1; ++t) {
-            if (k <= chunk[t]) break;
-            k -= chunk[t];
-        }
-        unsigned d = nb - 1 - t * per;
+    unsigned before = incl - mine;
+    for (unsigned w = 0; w < wave; ++w) before += chunk[w];
+    // exactly one thread owns the chunk that holds rank k (the last thread takes
+    // whatever is left if the counts fall short)
+    const bool owner = (k > before && k <= before + mine) || (threadIdx.x == kBlock - 1 && k > before + mine);
+    if (owner) {
+        unsigned kk = k - before;
+        unsigned d = nb - 1 - threadIdx.x * per;
         for (unsigned b = 0; b < per - 1; ++b, --d) {
             unsigned c = lh[d];
-            if (k <= c) break;
-            k -= c;
+            if (kk <= c) break;
+            kk -= c;
         }
         unsigned np = prefix | (d << shift);
         ctl[kCtlPrefix] = np;
-        ctl[kCtlK] = k;
+        ctl[kCtlK] = kk;
         if (pass == 2) ws.thr[2 * s.id] = np;
     }
 }
 
 // ---- 4. count ---------------------------------------------------------------------
 
+// The 16 lanes of a DPP row read one 64-element group as 16-byte vectors; a
+// wavefront therefore works on four flagged groups per load instruction.
+__device__ __forceinline__ f4 load_group4(const float* p, long long e, long long n, bool aligned) {
+    if (aligned && e + 3 < n) return *reinterpret_cast<const f4*>(p + e);
+    return ld4_guard(p, e, n);
+}
+
+// Takes the lowest set bit out of m: its index, or 64 when m is empty.
+__device__ __forceinline__ unsigned pop_bit(unsigned long long& m) {
+    unsigned i = m ? (unsigned)__ffsll((long long)m) - 1 : 64u;
+    m &= m - 1;
+    return i;
+}
+
+__device__ __forceinline__ unsigned pick_row(unsigned row, unsigned a, unsigned b, unsigned c, unsigned d) {
+    return row == 0 ? a : (row == 1 ? b : (row == 2 ? c : d));
+}
+
 // Counts, for tile `tile` (4096 elements) of tensor s, the keys above and equal
 // to thr; lane l looks at the maximum of 64-element group l and only groups
-// whose maximum reaches thr are read.  Wavefront-uniform result.
+// whose maximum reaches thr are read (eight at a time).  Wavefront-uniform result.
 __device__ __forceinline__ void count_tile(const Seg& s, const SparseWs& ws, unsigned tile, unsigned thr,
                                            unsigned lane, unsigned& gt, unsigned& eq) {
     const long long n = (long long)s.n;
+    const bool aligned = s.aligned != 0;
     unsigned gm = ws.gmax[(unsigned long long)(s.tile0 + tile) * 64 + lane];
     unsigned long long mask = __ballot(gm >= thr && gm > 0u);
-    const long long base = (long long)tile * kTile + lane;
-    gt = 0;
-    eq = 0;
+    const unsigned row = lane >> 4;
+    const long long base = (long long)tile * kTile + (lane & 15u) * 4;
+    unsigned cg = 0, ce = 0;
     while (mask) {
-        // up to four flagged groups per round, their loads in flight together
-        unsigned gi[4], key[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            gi[k] = mask ? (unsigned)__ffsll((long long)mask) - 1 : 64u;
-            mask &= mask - 1;
-        }
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            long long e = base + gi[k] * 64;
-            key[k] = (gi[k] < 64u && e < n) ? key_of(s.s1[e]) : 0u;
-        }
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            gt += __popcll(__ballot(key[k] > thr));
-            eq += __popcll(__ballot(key[k] == thr && key[k] > 0u));
-        }
+        unsigned a0 = pop_bit(mask), a1 = pop_bit(mask), a2 = pop_bit(mask), a3 = pop_bit(mask);
+        unsigned b0 = pop_bit(mask), b1 = pop_bit(mask), b2 = pop_bit(mask), b3 = pop_bit(mask);
+        unsigned ga = pick_row(row, a0, a1, a2, a3), gb = pick_row(row, b0, b1, b2, b3);
+        f4 va = {0.f, 0.f, 0.f, 0.f}, vb = {0.f, 0.f, 0.f, 0.f};
+        if (ga < 64u) va = load_group4(s.s1, base + ga * 64, n, aligned);
+        if (gb < 64u) vb = load_group4(s.s1, base + gb * 64, n, aligned);
+        unsigned k;
+        k = key_of(va.x); cg += k > thr; ce += (k == thr) & (k > 0u);
+        k = key_of(va.y); cg += k > thr; ce += (k == thr) & (k > 0u);
+        k = key_of(va.z); cg += k > thr; ce += (k == thr) & (k > 0u);
+        k = key_of(va.w); cg += k > thr; ce += (k == thr) & (k > 0u);
+        k = key_of(vb.x); cg += k > thr; ce += (k == thr) & (k > 0u);
+        k = key_of(vb.y); cg += k > thr; ce += (k == thr) & (k > 0u);
+        k = key_of(vb.z); cg += k > thr; ce += (k == thr) & (k > 0u);
+        k = key_of(vb.w); cg += k > thr; ce += (k == thr) & (k > 0u);
     }
+    gt = wave_sum_u(cg);
+    eq = wave_sum_u(ce);
 }
 
 // One wavefront per tile, four tiles per workgroup.
@@ -405,6 +432,15 @@ __global__ __launch_bounds__(kBlock) void sparse_scan_kernel(SegSrc src, SparseW
 
 // ---- 6. emit ----------------------------------------------------------------------
 
+// inclusive prefix sum over the 16 lanes of a DPP row
+__device__ __forceinline__ unsigned row_scan16(unsigned x) {
+    x += (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x111, 0xf, 0xf, true);  // row_shr:1
+    x += (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x112, 0xf, 0xf, true);  // row_shr:2
+    x += (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x114, 0xf, 0xf, true);  // row_shr:4
+    x += (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x118, 0xf, 0xf, true);  // row_shr:8
+    return x;
+}
+
 template <class Src>
 __global__ __launch_bounds__(kBlock) void sparse_emit_kernel(Src src, SparseWs ws, unsigned total_tiles) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
@@ -417,45 +453,98 @@ __global__ __launch_bounds__(kBlock) void sparse_emit_kernel(Src src, SparseWs w
     const unsigned long long ci = (unsigned long long)(s.tile0 + tile) * 2;
     const unsigned G = ws.counts[ci], E = ws.counts[ci + 1];
     unsigned pos = G + (E < quota ? E : quota);  // pairs written by earlier tiles
-    unsigned eq_seen = E;
     int32_t* idx = reinterpret_cast<int32_t*>(s.pay + kHeaderBytes);
     float* val = reinterpret_cast<float*>(s.pay + kHeaderBytes + 4ull * s.cap);
     unsigned gm = ws.gmax[(unsigned long long)(s.tile0 + tile) * 64 + lane];
     unsigned long long mask = __ballot(gm >= thr && gm > 0u);
-    const long long base = (long long)tile * kTile + lane;
-    while (mask) {
-        unsigned gi[4];
-        float v[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            gi[k] = mask ? (unsigned)__ffsll((long long)mask) - 1 : 64u;
-            mask &= mask - 1;
+    if (quota == kNoQuota) {
+        // Usual case: everything at or above the threshold is taken.  Row r of the
+        // wavefront reads the r-th flagged group of a round of four; positions come
+        // from a row prefix sum of the per-lane counts plus the totals of the rows
+        // before.  The next round's loads are issued before this round's stores
+        // (they touch different groups), so rounds overlap.
+        const unsigned row = lane >> 4;
+        const bool aligned = s.aligned != 0;
+        const long long base = (long long)tile * kTile + (lane & 15u) * 4;
+        const f4 zero4 = {0.f, 0.f, 0.f, 0.f};
+        unsigned gi;
+        f4 v = zero4;
+        {
+            unsigned g0 = pop_bit(mask), g1 = pop_bit(mask), g2 = pop_bit(mask), g3 = pop_bit(mask);
+            gi = pick_row(row, g0, g1, g2, g3);
+            if (gi < 64u) v = load_group4(s.s1, base + gi * 64, n, aligned);
         }
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            long long e = base + gi[k] * 64;
-            v[k] = (gi[k] < 64u && e < n) ? s.s1[e] : 0.f;
-        }
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            long long e = base + gi[k] * 64;
-            unsigned key = key_of(v[k]);
-            bool is_eq = key == thr && key > 0u;
-            unsigned long long m_eq = __ballot(is_eq);
-            bool sel = key > thr || (is_eq && eq_seen + popc_lt(m_eq, lane) < quota);
-            unsigned long long m_sel = __ballot(sel);
-            if (sel) {
-                unsigned p = pos + popc_lt(m_sel, lane);
-                if (p < s.cap) {
-                    idx[p] = (int32_t)e;
-                    val[p] = v[k];
-                    s.s1[e] = 0.f;
-                    if (s.s0) s.s0[e] = 0.f;
+        bool more = true;
+        while (more) {
+            more = mask != 0;
+            unsigned gi_next = 64u;
+            f4 v_next = zero4;
+            if (more) {
+                unsigned g0 = pop_bit(mask), g1 = pop_bit(mask), g2 = pop_bit(mask), g3 = pop_bit(mask);
+                gi_next = pick_row(row, g0, g1, g2, g3);
+                if (gi_next < 64u) v_next = load_group4(s.s1, base + gi_next * 64, n, aligned);
+            }
+            const long long e = base + gi * 64;
+            unsigned k0 = key_of(v.x), k1 = key_of(v.y), k2 = key_of(v.z), k3 = key_of(v.w);
+            unsigned s0 = (k0 >= thr) & (k0 > 0u), s1 = (k1 >= thr) & (k1 > 0u);
+            unsigned s2 = (k2 >= thr) & (k2 > 0u), s3 = (k3 >= thr) & (k3 > 0u);
+            unsigned c = s0 + s1 + s2 + s3;
+            unsigned incl = row_scan16(c);
+            unsigned t0 = (unsigned)__builtin_amdgcn_readlane((int)incl, 15);
+            unsigned t1 = (unsigned)__builtin_amdgcn_readlane((int)incl, 31);
+            unsigned t2 = (unsigned)__builtin_amdgcn_readlane((int)incl, 47);
+            unsigned t3 = (unsigned)__builtin_amdgcn_readlane((int)incl, 63);
+            unsigned p = pos + (incl - c) + (row > 0 ? t0 : 0u) + (row > 1 ? t1 : 0u) + (row > 2 ? t2 : 0u);
+            if (c && p + c <= s.cap) {  // the scan guarantees room; the test only guards the buffer
+                f4 keep = v;
+                if (s0) { idx[p] = (int32_t)e; val[p] = v.x; keep.x = 0.f; ++p; }
+                if (s1) { idx[p] = (int32_t)(e + 1); val[p] = v.y; keep.y = 0.f; ++p; }
+                if (s2) { idx[p] = (int32_t)(e + 2); val[p] = v.z; keep.z = 0.f; ++p; }
+                if (s3) { idx[p] = (int32_t)(e + 3); val[p] = v.w; keep.w = 0.f; ++p; }
+                if (aligned && e + 3 < n) {
+                    *reinterpret_cast<f4*>(s.s1 + e) = keep;
+                    if (s.s0) {
+                        f4 m = *reinterpret_cast<const f4*>(s.s0 + e);
+                        m.x = s0 ? 0.f : m.x; m.y = s1 ? 0.f : m.y; m.z = s2 ? 0.f : m.z; m.w = s3 ? 0.f : m.w;
+                        *reinterpret_cast<f4*>(s.s0 + e) = m;
+                    }
+                } else {
+                    if (s0) { s.s1[e] = 0.f; if (s.s0) s.s0[e] = 0.f; }
+                    if (s1) { s.s1[e + 1] = 0.f; if (s.s0) s.s0[e + 1] = 0.f; }
+                    if (s2) { s.s1[e + 2] = 0.f; if (s.s0) s.s0[e + 2] = 0.f; }
+                    if (s3) { s.s1[e + 3] = 0.f; if (s.s0) s.s0[e + 3] = 0.f; }
                 }
             }
-            pos += __popcll(m_sel);
-            eq_seen += __popcll(m_eq);
+            pos += t0 + t1 + t2 + t3;
+            gi = gi_next;
+            v = v_next;
         }
+        return;
+    }
+    // Overflow case: ties at the threshold are rationed in index order, one group
+    // of 64 at a time across the whole wavefront.
+    unsigned eq_seen = E;
+    const long long base = (long long)tile * kTile + lane;
+    while (mask) {
+        unsigned gi = pop_bit(mask);
+        long long e = base + gi * 64;
+        float v = e < n ? s.s1[e] : 0.f;
+        unsigned key = key_of(v);
+        bool is_eq = key == thr && key > 0u;
+        unsigned long long m_eq = __ballot(is_eq);
+        bool sel = key > thr || (is_eq && eq_seen + popc_lt(m_eq, lane) < quota);
+        unsigned long long m_sel = __ballot(sel);
+        if (sel) {
+            unsigned p = pos + popc_lt(m_sel, lane);
+            if (p < s.cap) {
+                idx[p] = (int32_t)e;
+                val[p] = v;
+                s.s1[e] = 0.f;
+                if (s.s0) s.s0[e] = 0.f;
+            }
+        }
+        pos += __popcll(m_sel);
+        eq_seen += __popcll(m_eq);
     }
 }
 
@@ -490,21 +579,24 @@ __device__ __forceinline__ unsigned sparse_header(const uint8_t* pay, unsigned s
     return nnz < cap ? nnz : cap;
 }
 
-// The slots of a tensor are dealt out evenly over that tensor's tiles.
+// One workgroup per 1024 slots of a tensor's payload; workgroups past nnz exit.
+constexpr int kSlotTile = 1024;
+
 template <class Src>
 __global__ __launch_bounds__(kBlock) void sparse_scatter_kernel(Src src) {
-    unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+    unsigned ct;
+    const Seg& s = src.get(ct, blockIdx.x);
     const int32_t* idx;
     const float* val;
     const unsigned nnz = sparse_header(s.pay, s.cap, idx, val);
-    const unsigned per = (s.cap + s.ntiles - 1) / s.ntiles;
-    const unsigned long long lo = (unsigned long long)tile * per;
-    unsigned long long hi = lo + per;
-    if (hi > nnz) hi = nnz;
-    for (unsigned long long j = lo + threadIdx.x; j < hi; j += kBlock) {
-        long long i = idx[j];
-        if (i >= 0 && i < (long long)s.n) s.out[i] = val[j];
+    const unsigned long long lo = (unsigned long long)ct * kSlotTile;
+#pragma unroll
+    for (int k = 0; k < kSlotTile / kBlock; ++k) {
+        unsigned long long j = lo + k * kBlock + threadIdx.x;
+        if (j < nnz) {
+            long long i = idx[j];
+            if (i >= 0 && i < (long long)s.n) s.out[i] = val[j];
+        }
     }
 }
 
@@ -576,11 +668,14 @@ hipError_t launch_sparse_decode(const Launch& L, hipStream_t st) {
     if (L.single) {
         SingleSrc src{L.seg};
         hipLaunchKernelGGL((zero_fill_kernel<SingleSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
-        hipLaunchKernelGGL((sparse_scatter_kernel<SingleSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
+        if (L.seg.ncblk)
+            hipLaunchKernelGGL((sparse_scatter_kernel<SingleSrc>), dim3(L.seg.ncblk), dim3(kBlock), 0, st, src);
     } else {
         BatchSrc src{L.dsegs, L.dmap};
         hipLaunchKernelGGL((zero_fill_kernel<BatchSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
-        hipLaunchKernelGGL((sparse_scatter_kernel<BatchSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
+        BatchSrc csrc{L.dsegs, L.dcmap};
+        if (L.nctiles)
+            hipLaunchKernelGGL((sparse_scatter_kernel<BatchSrc>), dim3(L.nctiles), dim3(kBlock), 0, st, csrc);
     }
     return hipGetLastError();
 }
