@@ -72,6 +72,10 @@ class SetWorkload:
                 elif self.alg == "onebit":
                     t["residual"] = torch.zeros(n, device=dev)
                     nb = hp.onebit_payload_bytes(n)
+                elif self.alg == "onebit_deferred":
+                    t["state"] = torch.zeros(n, device=dev)
+                    t["scale_state"] = torch.zeros(1, device=dev)
+                    nb = hp.onebit_payload_bytes(n)
                 elif self.alg == "terngrad":
                     nb = hp.terngrad_payload_bytes(n, self.params.get("bucket", 512))
                 elif self.alg == "dgc":
@@ -196,6 +200,8 @@ def make_workload(name):
     vgg, rn, bert = W.vgg19_sizes(), W.resnet50_sizes(), W.bert_large_sizes()
     if name == "onebit_vgg19":
         return SetWorkload(name, "onebit", vgg, "vgg", {}, 12.125, 4.125, 2, "onebit_quant_kernel", 12.125, nphases=3)
+    if name == "onebit_deferred_vgg19":
+        return SetWorkload(name, "onebit_deferred", vgg, "vgg", {}, 12.125, 4.125, 0, "onebit_deferred_kernel", 12.125, nphases=2)
     if name == "tbq_vgg19":
         return SetWorkload(name, "tbq", vgg, "vgg", {"threshold": 0.05}, 12.25, 4.25, 0, "tbq_encode_kernel", 12.25)
     if name == "terngrad_vgg19":
@@ -225,7 +231,7 @@ def make_workload(name):
 
 
 ALL_WORKLOADS = [
-    "onebit_vgg19", "tbq_vgg19", "terngrad_vgg19", "dgc_vgg19", "graddrop_vgg19", "tbq_262144", "tbq_262144_x512",
+    "onebit_vgg19", "onebit_deferred_vgg19", "tbq_vgg19", "terngrad_vgg19", "dgc_vgg19", "graddrop_vgg19", "tbq_262144", "tbq_262144_x512",
     "terngrad_resnet50", "dgc_bert_large", "graddrop_bert_large", "merge_tbq_vgg19", "merge_dgc_vgg19",
 ]
 

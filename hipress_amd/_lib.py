@@ -9,8 +9,9 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhipress_amd.so")
 
-ONEBIT, TBQ, TERNGRAD, DGC, GRADDROP = range(5)
-ALG_IDS = {"onebit": ONEBIT, "tbq": TBQ, "terngrad": TERNGRAD, "dgc": DGC, "graddrop": GRADDROP}
+ONEBIT, TBQ, TERNGRAD, DGC, GRADDROP, ONEBIT_DEFERRED = range(6)
+ALG_IDS = {"onebit": ONEBIT, "tbq": TBQ, "terngrad": TERNGRAD, "dgc": DGC, "graddrop": GRADDROP,
+           "onebit_deferred": ONEBIT_DEFERRED}
 MAX_PEERS = 16
 HEADER_BYTES = 16
 
@@ -56,6 +57,8 @@ SIGNATURES = {
     "hipress_tbq_decode": (ctypes.c_int, [_vp, _i64, _vp, _i64, _vp]),
     "hipress_onebit_encode": (ctypes.c_int, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "hipress_onebit_decode": (ctypes.c_int, [_vp, _i64, _vp, _i64, _vp]),
+    "hipress_onebit_encode_deferred": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
+    "hipress_onebit_residual": (ctypes.c_int, [_vp, _vp, _i64, _vp, _vp]),
     "hipress_terngrad_encode": (ctypes.c_int, [_vp, _vp, _i64, _vp, _i64, _i32, _vp]),
     "hipress_terngrad_decode": (ctypes.c_int, [_vp, _i64, _vp, _i64, _vp]),
     "hipress_dgc_encode": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp, _i64, _f32, _f64, _vp, _i64, _vp]),

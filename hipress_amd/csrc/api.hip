@@ -94,7 +94,8 @@ inline int hiperr(hipError_t e) { return e == hipSuccess ? HIPRESS_OK : HIPRESS_
 
 int payload_need(int alg, int64_t n, const hipress_params& pr, int64_t* need) {
     switch (alg) {
-        case HIPRESS_ONEBIT: *need = HIPRESS_HEADER_BYTES + words_bytes(n, 1); return HIPRESS_OK;
+        case HIPRESS_ONEBIT:
+        case HIPRESS_ONEBIT_DEFERRED: *need = HIPRESS_HEADER_BYTES + words_bytes(n, 1); return HIPRESS_OK;
         case HIPRESS_TBQ: *need = HIPRESS_HEADER_BYTES + words_bytes(n, 2); return HIPRESS_OK;
         case HIPRESS_TERNGRAD:
             if (pr.bucket < 1) return HIPRESS_ERR_PARAM;
@@ -111,7 +112,8 @@ int payload_need(int alg, int64_t n, const hipress_params& pr, int64_t* need) {
 
 int check_params(int alg, const hipress_params& pr) {
     switch (alg) {
-        case HIPRESS_ONEBIT: return HIPRESS_OK;
+        case HIPRESS_ONEBIT:
+        case HIPRESS_ONEBIT_DEFERRED: return HIPRESS_OK;
         case HIPRESS_TBQ: return (pr.threshold >= 0.f && std::isfinite(pr.threshold)) ? HIPRESS_OK : HIPRESS_ERR_PARAM;
         case HIPRESS_TERNGRAD: return pr.bucket >= 1 ? HIPRESS_OK : HIPRESS_ERR_PARAM;
         case HIPRESS_DGC:
@@ -133,12 +135,13 @@ int build_encode_seg(int alg, const hipress_tensor& t, const hipress_params& pr,
     int64_t need;
     if ((rc = payload_need(alg, t.n, pr, &need))) return rc;
     if (t.payload_bytes < need) return HIPRESS_ERR_SIZE;
-    const bool need_s0 = alg == HIPRESS_ONEBIT || alg == HIPRESS_TBQ || alg == HIPRESS_DGC || alg == HIPRESS_GRADDROP;
-    const bool need_s1 = alg == HIPRESS_DGC;
+    const bool need_s0 = alg != HIPRESS_TERNGRAD;
+    const bool need_s1 = alg == HIPRESS_DGC || alg == HIPRESS_ONEBIT_DEFERRED;
     const bool need_u = alg == HIPRESS_TERNGRAD;
     if (t.n > 0) {
         if (!t.grad || (need_s0 && !t.state0) || (need_s1 && !t.state1) || (need_u && !t.uniform)) return HIPRESS_ERR_NULL;
     }
+    if (alg == HIPRESS_ONEBIT_DEFERRED && !t.state1) return HIPRESS_ERR_NULL;  // the scale word is always read
     if (mis(t.grad, 4) || mis(t.state0, 4) || mis(t.state1, 4) || mis(t.uniform, 4)) return HIPRESS_ERR_ALIGN;
     s->g = t.grad;
     s->pay = static_cast<uint8_t*>(t.payload);
@@ -147,8 +150,10 @@ int build_encode_seg(int alg, const hipress_tensor& t, const hipress_params& pr,
     s->aligned = al16(t.grad);
     switch (alg) {
         case HIPRESS_ONEBIT:
+        case HIPRESS_ONEBIT_DEFERRED:
         case HIPRESS_TBQ:
             s->s0 = t.state0;
+            s->s1 = alg == HIPRESS_ONEBIT_DEFERRED ? t.state1 : nullptr;
             s->aligned = s->aligned && al16(t.state0);
             s->f0 = pr.threshold;
             s->words_off = HIPRESS_HEADER_BYTES;
@@ -201,6 +206,7 @@ int build_decode_seg(int alg, const void* payload, int64_t payload_bytes, float*
     s->words_off = HIPRESS_HEADER_BYTES;
     switch (alg) {
         case HIPRESS_ONEBIT:
+        case HIPRESS_ONEBIT_DEFERRED:
             if (payload_bytes < HIPRESS_HEADER_BYTES + words_bytes(n, 1)) return HIPRESS_ERR_SIZE;
             break;
         case HIPRESS_TBQ:
@@ -416,6 +422,33 @@ int hipress_onebit_decode(const void* payload, int64_t payload_bytes, float* out
     return hiperr(launch_onebit_decode(single_launch(s), static_cast<hipStream_t>(stream)));
 }
 
+int hipress_onebit_encode_deferred(const float* grad, float* state, float* scale_state, int64_t n, void* payload,
+                                   int64_t payload_bytes, void* workspace, int64_t workspace_bytes, void* stream) {
+    hipress_tensor t{grad, state, scale_state, nullptr, payload, nullptr, n, payload_bytes};
+    hipress_params pr{};
+    Seg s;
+    int rc = build_encode_seg(HIPRESS_ONEBIT_DEFERRED, t, pr, &s);
+    if (rc) return rc;
+    if (!workspace || workspace_bytes < hipress_onebit_workspace_bytes(n)) return HIPRESS_ERR_WORKSPACE;
+    if (mis(workspace, 16)) return HIPRESS_ERR_ALIGN;
+    return hiperr(launch_onebit_encode_deferred(single_launch(s), static_cast<float*>(workspace), -1,
+                                                static_cast<hipStream_t>(stream)));
+}
+
+int hipress_onebit_residual(const float* state, const float* scale_state, int64_t n, float* residual, void* stream) {
+    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (!scale_state || (n > 0 && (!state || !residual))) return HIPRESS_ERR_NULL;
+    if (mis(state, 4) || mis(scale_state, 4) || mis(residual, 4)) return HIPRESS_ERR_ALIGN;
+    Seg s;
+    std::memset(&s, 0, sizeof s);
+    s.s0 = const_cast<float*>(state);
+    s.s1 = const_cast<float*>(scale_state);
+    s.out = residual;
+    s.n = (unsigned long long)n;
+    s.ntiles = tiles_of(n);
+    return hiperr(launch_onebit_materialize(single_launch(s), static_cast<hipStream_t>(stream)));
+}
+
 // ---- TernGrad ----------------------------------------------------------------------
 
 int hipress_terngrad_encode(const float* grad, const float* uniform, int64_t n, void* payload,
@@ -605,7 +638,7 @@ int hipress_batch_create(hipress_batch** out, int32_t alg, const hipress_tensor*
     if (!out || !params || (count > 0 && !tensors)) return HIPRESS_ERR_NULL;
     *out = nullptr;
     if (count < 0) return HIPRESS_ERR_SIZE;
-    if (alg < HIPRESS_ONEBIT || alg > HIPRESS_GRADDROP) return HIPRESS_ERR_PARAM;
+    if (alg < HIPRESS_ONEBIT || alg > HIPRESS_ONEBIT_DEFERRED) return HIPRESS_ERR_PARAM;
     int rc = check_params(alg, *params);
     if (rc) return rc;
     hipress_batch* b = new (std::nothrow) hipress_batch;
@@ -649,7 +682,7 @@ int hipress_batch_create(hipress_batch** out, int32_t alg, const hipress_tensor*
         b->swl = sparse_ws_layout(total_ns, b->ntiles, count);
         if (b->swl.bytes && hipMalloc(&b->ws, (size_t)b->swl.bytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
         if ((rc = upload(smap, &b->d_smap))) return fail(rc);
-    } else if (enc_ok && alg == HIPRESS_ONEBIT) {
+    } else if (enc_ok && (alg == HIPRESS_ONEBIT || alg == HIPRESS_ONEBIT_DEFERRED)) {
         if (hipMalloc(&b->ws, (size_t)round_up(4 * (int64_t)(b->ntiles ? b->ntiles : 1), 256)) != hipSuccess) return fail(HIPRESS_ERR_HIP);
     }
     if (dec_ok && sparse) {
@@ -691,6 +724,9 @@ static int batch_encode_impl(hipress_batch* b, int phase, void* stream) {
         case HIPRESS_ONEBIT:
             if (phase > 2) return HIPRESS_ERR_PARAM;
             return hiperr(launch_onebit_encode(L, static_cast<float*>(b->ws), phase, st));
+        case HIPRESS_ONEBIT_DEFERRED:
+            if (phase > 1) return HIPRESS_ERR_PARAM;
+            return hiperr(launch_onebit_encode_deferred(L, static_cast<float*>(b->ws), phase, st));
         case HIPRESS_TBQ:
             if (phase > 0) return HIPRESS_ERR_PARAM;
             return hiperr(launch_tbq_encode(L, st));
@@ -719,7 +755,8 @@ int hipress_batch_decode(hipress_batch* b, void* stream) {
     hipStream_t st = static_cast<hipStream_t>(stream);
     Launch L = batch_launch(b, false);
     switch (b->alg) {
-        case HIPRESS_ONEBIT: return hiperr(launch_onebit_decode(L, st));
+        case HIPRESS_ONEBIT:
+        case HIPRESS_ONEBIT_DEFERRED: return hiperr(launch_onebit_decode(L, st));
         case HIPRESS_TBQ: return hiperr(launch_tbq_decode(L, st));
         case HIPRESS_TERNGRAD: return hiperr(launch_terngrad_decode(L, st));
         case HIPRESS_DGC:

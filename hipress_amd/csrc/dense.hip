@@ -176,27 +176,46 @@ __global__ __launch_bounds__(kBlock) void onebit_abs_kernel(Src src, float* part
     if (threadIdx.x == 0) partial[s.tile0 + tile] = (wsum[0] + wsum[1]) + (wsum[2] + wsum[3]);
 }
 
-// Pass 2: one workgroup per tensor adds that tensor's partials in double, in a
-// fixed order, and writes the header {scale, n, 0, 0}.
+// Pass 2: one workgroup of 1024 threads per tensor adds that tensor's partials in
+// double, in a fixed order, and writes the header {scale, n, 0, 0} (and the
+// scale-state word of the deferred variant).
+constexpr int kScaleBlock = 1024;
+
+__device__ __forceinline__ double wave_sum_d(double x) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) x += __shfl_xor(x, m, 64);
+    return x;
+}
+
 template <class Src>
-__global__ __launch_bounds__(kBlock) void onebit_scale_kernel(Src src, const float* partial) {
-    __shared__ double red[kBlock];
+__global__ __launch_bounds__(kScaleBlock) void onebit_scale_kernel(Src src, const float* partial) {
+    __shared__ double red[kScaleBlock / 64];
     const Seg& s = src.at(blockIdx.x);
-    double a = 0.0;
-    for (unsigned t = threadIdx.x; t < s.ntiles; t += kBlock) a += (double)partial[s.tile0 + t];
-    red[threadIdx.x] = a;
-    __syncthreads();
-    for (int w = kBlock / 2; w >= 1; w >>= 1) {
-        if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
-        __syncthreads();
+    const float* p = partial + s.tile0;
+    const unsigned nt = s.ntiles;
+    double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
+    unsigned t = threadIdx.x;
+    for (; t + 3 * kScaleBlock < nt; t += 4 * kScaleBlock) {
+        float x0 = p[t], x1 = p[t + kScaleBlock], x2 = p[t + 2 * kScaleBlock], x3 = p[t + 3 * kScaleBlock];
+        a0 += (double)x0;
+        a1 += (double)x1;
+        a2 += (double)x2;
+        a3 += (double)x3;
     }
+    for (; t < nt; t += kScaleBlock) a0 += (double)p[t];
+    double a = wave_sum_d((a0 + a1) + (a2 + a3));
+    if ((threadIdx.x & 63u) == 0) red[threadIdx.x >> 6] = a;
+    __syncthreads();
     if (threadIdx.x == 0) {
-        float sc = s.n ? (float)(red[0] / (double)s.n) : 0.f;
+        double tot = 0.0;
+        for (int w = 0; w < kScaleBlock / 64; ++w) tot += red[w];
+        float sc = s.n ? (float)(tot / (double)s.n) : 0.f;
         uint32_t* h = reinterpret_cast<uint32_t*>(s.pay);
         h[0] = __float_as_uint(sc);
         h[1] = (uint32_t)s.n;
         h[2] = 0;
         h[3] = 0;
+        if (s.s1) *s.s1 = sc;
     }
 }
 
@@ -244,6 +263,94 @@ __global__ __launch_bounds__(kBlock) void onebit_quant_kernel(Src src) {
     const Seg& s = src.get(tile, gridDim.x - 1 - blockIdx.x);
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) onebit_quant_tile<true>(s, tile);
     else onebit_quant_tile<false>(s, tile);
+}
+
+// ---- deferred residual ----------------------------------------------------------
+// The two-pass encode above reads gradient and residual twice because the scale
+// must be known before r' = v - d can be written.  The deferred variant keeps
+// the state buffer one step behind: it stores v (the value before the scale was
+// subtracted) together with that step's scale in a one-word side buffer, and the
+// NEXT call forms r = v_prev - d(v_prev, s_prev) on the fly before adding the new
+// gradient - the same two roundings in the same order, so every bit matches the
+// two-pass operator.  One pass per step: read g and state, write state and bits.
+template <bool FAST>
+__device__ __forceinline__ float onebit_deferred_tile(const Seg& s, unsigned tile, float sp) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    uint32_t* words = reinterpret_cast<uint32_t*>(s.pay + kHeaderBytes);
+    f4 g[4], v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        g[j] = load4<FAST>(s.g, e, n);
+        v[j] = load4<FAST>(s.s0, e, n);
+    }
+    unsigned myword = 0;
+    float a = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        f4 r;  // residual the two-pass operator would have stored last step
+        r.x = v[j].x - (v[j].x >= 0.f ? sp : -sp);
+        r.y = v[j].y - (v[j].y >= 0.f ? sp : -sp);
+        r.z = v[j].z - (v[j].z >= 0.f ? sp : -sp);
+        r.w = v[j].w - (v[j].w >= 0.f ? sp : -sp);
+        f4 nv = r + g[j];
+        unsigned nib = (nv.x >= 0.f) | ((nv.y >= 0.f) << 1) | ((nv.z >= 0.f) << 2) | ((nv.w >= 0.f) << 3);
+        if (!FAST) {
+            unsigned vm = valid4(e, n);
+            nib &= vm;
+            nv.x = (vm & 1u) ? nv.x : 0.f;
+            nv.y = (vm & 2u) ? nv.y : 0.f;
+            nv.z = (vm & 4u) ? nv.z : 0.f;
+            nv.w = (vm & 8u) ? nv.w : 0.f;
+        }
+        a += abs4sum(nv);
+        store4<FAST>(s.s0, e, n, nv);
+        unsigned w = oct_pack4(nib, lane);
+        myword = ((lane & 7u) == (unsigned)j) ? w : myword;
+    }
+    long long widx = (base >> 5) + (lane & 7u) * 8 + (lane >> 3);
+    if ((lane & 7u) < 4u && (FAST || widx < (long long)((n + 31) >> 5))) words[widx] = myword;
+    return a;
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void onebit_deferred_kernel(Src src, float* partial) {
+    __shared__ float wsum[4];
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    const float sp = *s.s1;  // last step's scale (0 before the first step)
+    float a;
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) a = onebit_deferred_tile<true>(s, tile, sp);
+    else a = onebit_deferred_tile<false>(s, tile, sp);
+    a = wave_sum(a);
+    if ((threadIdx.x & 63u) == 0) wsum[threadIdx.x >> 6] = a;
+    __syncthreads();
+    if (threadIdx.x == 0) partial[s.tile0 + tile] = (wsum[0] + wsum[1]) + (wsum[2] + wsum[3]);
+}
+
+// out = v - d(v, scale): the residual the two-pass operator holds after the same steps.
+template <class Src>
+__global__ __launch_bounds__(kBlock) void onebit_materialize_kernel(Src src) {
+    unsigned tile;
+    const Seg& s = src.get(tile, blockIdx.x);
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    const float sp = *s.s1;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        f4 v = ld4_guard(s.s0, e, n);
+        f4 r;
+        r.x = v.x - (v.x >= 0.f ? sp : -sp);
+        r.y = v.y - (v.y >= 0.f ? sp : -sp);
+        r.z = v.z - (v.z >= 0.f ? sp : -sp);
+        r.w = v.w - (v.w >= 0.f ? sp : -sp);
+        st4_guard(s.out, e, n, r);
+    }
 }
 
 template <bool FAST>
@@ -516,10 +623,10 @@ static hipError_t onebit_quant(const Launch& L, hipStream_t st) { HP_LAUNCH(oneb
 static hipError_t onebit_scale(const Launch& L, const float* partial, hipStream_t st) {
     if (L.single) {
         SingleSegSrc src{L.seg};
-        hipLaunchKernelGGL((onebit_scale_kernel<SingleSegSrc>), dim3(1), dim3(kBlock), 0, st, src, partial);
+        hipLaunchKernelGGL((onebit_scale_kernel<SingleSegSrc>), dim3(1), dim3(kScaleBlock), 0, st, src, partial);
     } else {
         BatchSegSrc src{L.dsegs};
-        hipLaunchKernelGGL((onebit_scale_kernel<BatchSegSrc>), dim3(L.nsegs), dim3(kBlock), 0, st, src, partial);
+        hipLaunchKernelGGL((onebit_scale_kernel<BatchSegSrc>), dim3(L.nsegs), dim3(kScaleBlock), 0, st, src, partial);
     }
     return hipGetLastError();
 }
@@ -539,6 +646,24 @@ hipError_t launch_onebit_encode(const Launch& L, float* partial, int phase, hipS
     }
     return hipSuccess;
 }
+
+static hipError_t onebit_deferred(const Launch& L, float* partial, hipStream_t st) {
+    HP_LAUNCH(onebit_deferred_kernel, L, st, partial);
+}
+
+// phase < 0: both launches; 0: the fused pass; 1: the scale.
+hipError_t launch_onebit_encode_deferred(const Launch& L, float* partial, int phase, hipStream_t st) {
+    hipError_t e;
+    if (L.ntiles && (phase < 0 || phase == 0)) {
+        if ((e = onebit_deferred(L, partial, st)) != hipSuccess) return e;
+    }
+    if (phase < 0 || phase == 1) {
+        if ((e = onebit_scale(L, partial, st)) != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+hipError_t launch_onebit_materialize(const Launch& L, hipStream_t st) { HP_LAUNCH(onebit_materialize_kernel, L, st); }
 
 template <class Src>
 static hipError_t terngrad_encode_src(const Src& src, unsigned ntiles, unsigned bucket, hipStream_t st) {

@@ -8,6 +8,8 @@ hipError_t launch_tbq_encode(const Launch& L, hipStream_t st);
 hipError_t launch_tbq_decode(const Launch& L, hipStream_t st);
 hipError_t launch_onebit_encode(const Launch& L, float* partial, int phase, hipStream_t st);
 hipError_t launch_onebit_decode(const Launch& L, hipStream_t st);
+hipError_t launch_onebit_encode_deferred(const Launch& L, float* partial, int phase, hipStream_t st);
+hipError_t launch_onebit_materialize(const Launch& L, hipStream_t st);
 hipError_t launch_terngrad_encode(const Launch& L, unsigned bucket, hipStream_t st);
 hipError_t launch_terngrad_decode(const Launch& L, hipStream_t st);
 

@@ -26,7 +26,7 @@ from ._lib import ALG_IDS, MAX_PEERS, MergeChunk, Params, Tensor, check, size
 __all__ = [
     "onebit_payload_bytes", "tbq_payload_bytes", "terngrad_payload_bytes", "sparse_capacity",
     "sparse_payload_bytes", "dgc_payload_bytes", "graddrop_payload_bytes",
-    "onebit_encode", "onebit_decode", "tbq_encode", "tbq_decode", "terngrad_encode", "terngrad_decode",
+    "onebit_encode", "onebit_decode", "onebit_encode_deferred", "onebit_residual", "tbq_encode", "tbq_decode", "terngrad_encode", "terngrad_decode",
     "dgc_encode", "dgc_decode", "graddrop_encode", "graddrop_decode",
     "onebit_decode_merge", "tbq_decode_merge", "terngrad_decode_merge", "dgc_decode_merge",
     "graddrop_decode_merge", "Batch", "MergeBatch", "ALIASES",
@@ -142,6 +142,33 @@ def onebit_encode(gradient, residual, compressed):
         ws = _workspace(gradient, need)
         check(L.hipress_onebit_encode(_p(gradient), _p(residual), n, _p(compressed), compressed.numel(),
                                       _p(ws), ws.numel(), _stream(gradient)), "onebit_encode")
+
+
+def onebit_encode_deferred(gradient, state, scale_state, compressed):
+    """onebit_encode in one pass per step: `state` holds v = residual + gradient of the
+    previous step (initially the residual) and `scale_state` (1 float, initially 0) its
+    scale; the payloads equal onebit_encode's.  Use onebit_residual to read the residual."""
+    _f32(gradient, "gradient"); _f32(state, "state", gradient); _f32(scale_state, "scale_state", gradient)
+    _u8(compressed, "compressed", gradient)
+    _same_numel(gradient, state, "gradient", "state")
+    if scale_state.numel() != 1:
+        raise ValueError("scale_state must hold exactly one float")
+    L = _lib.lib()
+    n = gradient.numel()
+    with torch.cuda.device(gradient.device):
+        ws = _workspace(gradient, size(L.hipress_onebit_workspace_bytes(n), "onebit_workspace_bytes"))
+        check(L.hipress_onebit_encode_deferred(_p(gradient), _p(state), _p(scale_state), n, _p(compressed),
+                                               compressed.numel(), _p(ws), ws.numel(), _stream(gradient)),
+              "onebit_encode_deferred")
+
+
+def onebit_residual(state, scale_state, residual):
+    """residual = the error-feedback residual onebit_encode would hold after the same steps."""
+    _f32(state, "state"); _f32(scale_state, "scale_state", state); _f32(residual, "residual", state)
+    _same_numel(state, residual, "state", "residual")
+    with torch.cuda.device(state.device):
+        check(_lib.lib().hipress_onebit_residual(_p(state), _p(scale_state), state.numel(), _p(residual),
+                                                 _stream(state)), "onebit_residual")
 
 
 def onebit_decode(compressed, gradient):
@@ -295,6 +322,8 @@ class Batch:
             g = t.get("gradient")
             if alg in ("onebit", "tbq"):
                 s0, s1 = t.get("residual"), None
+            elif alg == "onebit_deferred":
+                s0, s1 = t.get("state"), t.get("scale_state")
             elif alg == "dgc":
                 s0, s1 = t.get("momentum"), t.get("accumulator")
             elif alg == "graddrop":

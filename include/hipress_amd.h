@@ -65,7 +65,8 @@ enum hipress_alg {
     HIPRESS_TBQ = 1,
     HIPRESS_TERNGRAD = 2,
     HIPRESS_DGC = 3,
-    HIPRESS_GRADDROP = 4
+    HIPRESS_GRADDROP = 4,
+    HIPRESS_ONEBIT_DEFERRED = 5 /* batches only: state0 = state, state1 = one-word scale state */
 };
 
 int hipress_version(void);
@@ -97,6 +98,20 @@ int hipress_onebit_encode(const float *grad, float *residual, int64_t n, void *p
                           void *stream);
 int hipress_onebit_decode(const void *payload, int64_t payload_bytes, float *out, int64_t n,
                           void *stream);
+
+/* onebit with a deferred residual: one pass per step instead of two.  `state`
+ * holds v = r + g of the LAST step (initially the residual itself) and
+ * `scale_state` (one float, initially 0) that step's scale; each call first forms
+ * the residual r = v - (v >= 0 ? s : -s) on the fly, exactly as the two-pass
+ * operator would have stored it, then proceeds as hipress_onebit_encode.  Payloads
+ * are identical to hipress_onebit_encode's; hipress_onebit_residual writes the
+ * residual that operator would hold into `residual`.  No counterpart in the
+ * reference: an extension for callers that do not read the residual between steps. */
+int hipress_onebit_encode_deferred(const float *grad, float *state, float *scale_state, int64_t n,
+                                   void *payload, int64_t payload_bytes, void *workspace,
+                                   int64_t workspace_bytes, void *stream);
+int hipress_onebit_residual(const float *state, const float *scale_state, int64_t n,
+                            float *residual, void *stream);
 
 /* ---- TernGrad: stochastic ternarisation, per-bucket max-abs scale ---------- */
 /* Replaces TernGradEncode_body / TernGradDecode_body for "terngrad"

@@ -130,6 +130,34 @@ def test_onebit_scale_is_deterministic(hp):
     assert len(set(scales)) == 1
 
 
+@pytest.mark.parametrize("n", [1, 33, 4097, 1000003])
+def test_onebit_deferred_matches_two_pass(hp, n):
+    """The one-pass variant must produce the payloads of onebit_encode and, on
+    request, the residual it would hold - bit for bit, over several steps."""
+    rng = np.random.default_rng(500 + n)
+    r0 = rng.normal(0, 1e-3, n).astype(F)
+    state, sstate = dev(r0), torch.zeros(1, device="cuda")
+    r_two = dev(r0)
+    r_ref = r0
+    for step in range(4):
+        g = rng.normal(0, 1e-3, n).astype(F)
+        pay_d = payload(hp.onebit_payload_bytes(n))
+        pay_t = payload(hp.onebit_payload_bytes(n))
+        hp.onebit_encode_deferred(dev(g), state, sstate, pay_d)
+        hp.onebit_encode(dev(g), r_two, pay_t)
+        got = host(pay_d)
+        np.testing.assert_array_equal(got, host(pay_t), err_msg=f"payload step {step}")
+        res = torch.empty(n, device="cuda")
+        hp.onebit_residual(state, sstate, res)
+        np.testing.assert_array_equal(host(res), host(r_two), err_msg=f"residual step {step}")
+        # and against the oracle, given the GPU's scale
+        s_gpu = got[:4].view(F)[0]
+        assert host(sstate)[0] == s_gpu
+        want_pay, r_ref = oracle.onebit_encode(g, r_ref, scale=s_gpu)
+        np.testing.assert_array_equal(got, want_pay)
+        np.testing.assert_array_equal(host(res), r_ref)
+
+
 def test_onebit_zero_tensor(hp):
     n = 5000
     pay = payload(hp.onebit_payload_bytes(n))
@@ -339,6 +367,34 @@ def test_sparse_decode_merge(hp, n):
 # ---------------------------------------------------------------- batched launches
 def mixed_sizes():
     return [1728, 64, 36864, 64, 73728, 128, 4097, 1, 262144, 512, 1000003, 1000]
+
+
+def test_batch_onebit_deferred(hp):
+    rng = np.random.default_rng(43)
+    tensors, refs = [], []
+    for n in mixed_sizes():
+        r0 = rng.normal(0, 1e-3, n).astype(F)
+        tensors.append({"gradient": torch.zeros(n, device="cuda"), "state": dev(r0), "scale_state": torch.zeros(1, device="cuda"),
+                        "compressed": payload(hp.onebit_payload_bytes(n)), "out": torch.empty(n, device="cuda")})
+        refs.append(r0)
+    b = hp.Batch("onebit_deferred", tensors)
+    for step in range(3):
+        gs = [rng.normal(0, 1e-3, t["gradient"].numel()).astype(F) for t in tensors]
+        for t, g in zip(tensors, gs):
+            t["gradient"].copy_(dev(g))
+        b.encode()
+        b.decode()
+        for i, (t, g) in enumerate(zip(tensors, gs)):
+            n = g.size
+            got = host(t["compressed"])
+            s = got[:4].view(F)[0]
+            want, refs[i] = oracle.onebit_encode(g, refs[i], scale=s)
+            np.testing.assert_array_equal(got, want)
+            res = torch.empty(n, device="cuda")
+            hp.onebit_residual(t["state"], t["scale_state"], res)
+            np.testing.assert_array_equal(host(res), refs[i])
+            np.testing.assert_array_equal(host(t["out"]), oracle.onebit_decode(want, n))
+    b.close()
 
 
 @pytest.mark.parametrize("alg", ["tbq", "onebit", "terngrad", "dgc", "graddrop"])
