@@ -23,8 +23,12 @@ import time
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs (see profiles/), keyed by workload; None = not measured.
-MEASURED_TRAFFIC = {}
+# WRITE_SIZE runs (summaries under profiles/), keyed by workload; absent = not
+# measured.  (FETCH_SIZE KiB * 2.0 + WRITE_SIZE KiB * 1.0) * 1024, the factors
+# being what the same counters read for a plain 1 GiB copy.
+MEASURED_TRAFFIC = {
+    "onebit_vgg19": int((563473.8 * 2.0 + 579850.1) * 1024),  # onebit_quant_kernel
+}
 
 
 def _events(n):
@@ -332,6 +336,9 @@ def main():
     ap.add_argument("--no-others", action="store_true", help="measure only --workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--others-steps", type=int, default=10)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a plain 1 GiB device-to-device copy (a kernel of known traffic: 1 GiB read, "
+                         "1 GiB written) so that rocprofv3 FETCH_SIZE / WRITE_SIZE can be scaled against it")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.stderr.write("bench.py: this build measures one GPU's share of the path; run with --gpus 1 "
@@ -343,6 +350,16 @@ def main():
         sys.stderr.write("bench.py needs a GPU\n")
         sys.exit(2)
     import hipress_amd  # noqa: F401  (raises if libhipress_amd.so is missing)
+
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "torch copy_ of 2**28 fp32", "bytes_read": 4 << 28, "bytes_written": 4 << 28,
+                          "launches": args.steps}))
+        return
 
     main_res = measure(args.workload, args.steps, args.warmup)
     others = []
