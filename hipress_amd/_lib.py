@@ -53,6 +53,7 @@ SIGNATURES = {
     "hipress_sparse_payload_bytes": (_i64, [_i64, _f64]),
     "hipress_onebit_workspace_bytes": (_i64, [_i64]),
     "hipress_sparse_workspace_bytes": (_i64, [_i64, _f64]),
+    "hipress_sparse_merge_workspace_bytes": (_i64, [_i64, _i32, _f64, _i32]),
     "hipress_tbq_encode": (ctypes.c_int, [_vp, _vp, _i64, _vp, _i64, _f32, _vp]),
     "hipress_tbq_decode": (ctypes.c_int, [_vp, _i64, _vp, _i64, _vp]),
     "hipress_onebit_encode": (ctypes.c_int, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),

@@ -88,6 +88,12 @@ inline SparseWs sparse_ws_at(void* base, const SparseWsLayout& l) {
     return w;
 }
 
+// Index part of a sparse merge workspace: per chunk npeers x (tiles + 1) tile
+// pointers, then one "not sorted" flag per (chunk, peer).
+inline int64_t merge_index_bytes(int64_t tileptr_words, int64_t nchunks, int64_t npeers) {
+    return round_up(4 * tileptr_words, 256) + round_up(4 * nchunks * npeers, 256);
+}
+
 inline int hiperr(hipError_t e) { return e == hipSuccess ? HIPRESS_OK : HIPRESS_ERR_HIP; }
 
 // ---- descriptor builders: validate one tensor and fill its Seg -------------------------
@@ -331,6 +337,8 @@ struct hipress_merge_batch {
     unsigned ntiles = 0, nstiles = 0;
     void* ws = nullptr;
     SparseWsLayout swl{};
+    void* iws = nullptr;  // sparse: tile pointers and "not sorted" flags
+    int64_t tp_words = 0;
 };
 
 extern "C" {
@@ -594,6 +602,17 @@ int hipress_terngrad_decode_merge(const void* const* payloads, const int64_t* pa
                                      static_cast<hipStream_t>(stream)));
 }
 
+int64_t hipress_sparse_merge_workspace_bytes(int64_t n, int32_t npeers, double ratio, int32_t reencode) {
+    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (npeers < 1 || npeers > HIPRESS_MAX_PEERS) return HIPRESS_ERR_PARAM;
+    int64_t bytes = merge_index_bytes((int64_t)npeers * (tiles_of(n) + 1), 1, npeers);
+    if (reencode) {
+        if (bad_ratio(ratio)) return HIPRESS_ERR_PARAM;
+        bytes += sparse_ws_layout(sparse_plan(n, ratio).ns, tiles_of(n), 1).bytes;
+    }
+    return bytes;
+}
+
 int hipress_sparse_decode_merge(const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
                                 float* aggregate, int64_t n, float* accumulator, void* out_payload,
                                 int64_t out_payload_bytes, double ratio, void* workspace,
@@ -601,21 +620,29 @@ int hipress_sparse_decode_merge(const void* const* payloads, const int64_t* payl
     MergeSeg m;
     int rc = build_merge_seg(HIPRESS_DGC, payloads, payload_bytes, npeers, aggregate, n, &m);
     if (rc) return rc;
-    Seg s;
     SparseWsLayout l{};
+    const int64_t tp_words = (int64_t)npeers * (m.s.ntiles + 1);
+    const int64_t ibytes = merge_index_bytes(tp_words, 1, npeers);
+    int64_t need = ibytes;
     if (accumulator) {
         hipress_tensor t{aggregate, accumulator, nullptr, nullptr, out_payload, nullptr, n, out_payload_bytes};
         hipress_params pr{};
         pr.ratio = ratio;
-        if ((rc = build_encode_seg(HIPRESS_GRADDROP, t, pr, &s))) return rc;
-        l = sparse_ws_layout(s.ns, s.ntiles, 1);
-        if (!workspace || workspace_bytes < l.bytes) return HIPRESS_ERR_WORKSPACE;
-        if (mis(workspace, 16)) return HIPRESS_ERR_ALIGN;
+        if ((rc = build_encode_seg(HIPRESS_GRADDROP, t, pr, &m.r))) return rc;
+        l = sparse_ws_layout(m.r.ns, m.r.ntiles, 1);
+        need += l.bytes;
     }
+    if (!workspace || workspace_bytes < need) return HIPRESS_ERR_WORKSPACE;
+    if (mis(workspace, 16)) return HIPRESS_ERR_ALIGN;
+    uint8_t* wsb = static_cast<uint8_t*>(workspace);
+    uint32_t* tileptr = reinterpret_cast<uint32_t*>(wsb);
+    uint32_t* unsorted = reinterpret_cast<uint32_t*>(wsb + round_up(4 * tp_words, 256));
+    SparseWs ws{};
+    if (accumulator) ws = sparse_ws_at(wsb + ibytes, l);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipError_t e = launch_sparse_merge_scatter(single_merge_launch(m, npeers, false), st);
+    hipError_t e = launch_sparse_merge(single_merge_launch(m, npeers, accumulator != nullptr), ws, tileptr, unsorted, st);
     if (e != hipSuccess) return HIPRESS_ERR_HIP;
-    if (accumulator) e = launch_sparse_encode(single_launch(s), false, sparse_ws_at(workspace, l), -1, st);
+    if (accumulator) e = launch_sparse_encode(single_launch(m.r), false, ws, kSparseAfterAccum, st);
     return hiperr(e);
 }
 
@@ -770,6 +797,7 @@ int hipress_batch_decode(hipress_batch* b, void* stream) {
 int hipress_merge_batch_destroy(hipress_merge_batch* b) {
     if (!b) return HIPRESS_OK;
     (void)hipFree(b->d_segs);
+    (void)hipFree(b->iws);
     (void)hipFree(b->d_renc);
     (void)hipFree(b->d_map);
     (void)hipFree(b->d_smap);
@@ -827,6 +855,16 @@ int hipress_merge_batch_create(hipress_merge_batch** out, int32_t alg, const hip
         b->swl = sparse_ws_layout(total_ns, b->ntiles, count);
         if (b->swl.bytes && hipMalloc(&b->ws, (size_t)b->swl.bytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
         if ((rc = upload(smap, &b->d_smap))) return fail(rc);
+        for (size_t i = 0; i < b->segs.size(); ++i) b->segs[i].r = b->renc[i];  // the merge kernel runs their first launch
+    }
+    if (sparse) {
+        int64_t words = 0;
+        for (MergeSeg& m : b->segs) {
+            m.tp0 = (unsigned long long)words;
+            words += (int64_t)npeers * (m.s.ntiles + 1);
+        }
+        b->tp_words = words;
+        if (hipMalloc(&b->iws, (size_t)merge_index_bytes(words, count, npeers)) != hipSuccess) return fail(HIPRESS_ERR_HIP);
     }
     if ((rc = upload(b->segs, &b->d_segs))) return fail(rc);
     if ((rc = upload(b->renc, &b->d_renc))) return fail(rc);
@@ -849,7 +887,11 @@ int hipress_merge_batch_run(hipress_merge_batch* b, void* stream) {
     L.npeers = b->npeers;
     L.reencode = b->reencode;
     if (b->alg == HIPRESS_DGC || b->alg == HIPRESS_GRADDROP) {
-        hipError_t e = launch_sparse_merge_scatter(L, st);
+        uint32_t* tileptr = static_cast<uint32_t*>(b->iws);
+        uint32_t* unsorted = reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(b->iws) + round_up(4 * b->tp_words, 256));
+        SparseWs ws{};
+        if (b->reencode) ws = sparse_ws_at(b->ws, b->swl);
+        hipError_t e = launch_sparse_merge(L, ws, tileptr, unsorted, st);
         if (e != hipSuccess) return HIPRESS_ERR_HIP;
         if (b->reencode) {
             Launch R;
@@ -861,7 +903,7 @@ int hipress_merge_batch_run(hipress_merge_batch* b, void* stream) {
             R.nstiles = b->nstiles;
             R.ntiles = b->ntiles;
             R.nsegs = (unsigned)b->renc.size();
-            e = launch_sparse_encode(R, false, sparse_ws_at(b->ws, b->swl), -1, st);
+            e = launch_sparse_encode(R, false, ws, kSparseAfterAccum, st);
         }
         return hiperr(e);
     }

@@ -57,6 +57,8 @@ struct MergeSeg {
     unsigned long long peer_bytes[kMaxPeers];  // size of each peer's buffer
     unsigned int peer_slots[kMaxPeers];  // sparse: pairs each peer's buffer has room for
     Seg s;  // out = aggregate, s0 = aggregator residual (tbq), pay = re-encoded payload
+    Seg r;  // sparse re-encode of the aggregate (GradDrop descriptor: s1 = accumulator, pay = out payload)
+    unsigned long long tp0;  // sparse: first tile pointer of this chunk
 };
 
 struct SingleSrc {
@@ -86,6 +88,16 @@ struct SingleSegSrc {
 struct BatchSegSrc {
     const Seg* segs;
     __device__ __forceinline__ const Seg& at(unsigned i) const { return segs[i]; }
+};
+
+struct MergeSingleSegSrc {
+    MergeSeg seg;
+    __device__ __forceinline__ const MergeSeg& at(unsigned) const { return seg; }
+};
+
+struct MergeBatchSegSrc {
+    const MergeSeg* segs;
+    __device__ __forceinline__ const MergeSeg& at(unsigned i) const { return segs[i]; }
 };
 
 struct MergeSingleSrc {

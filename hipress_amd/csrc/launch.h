@@ -27,6 +27,8 @@ struct SparseWs {
 };
 hipError_t launch_sparse_encode(const Launch& L, bool dgc, const SparseWs& ws, int phase, hipStream_t st);
 hipError_t launch_sparse_decode(const Launch& L, hipStream_t st);
-hipError_t launch_sparse_merge_scatter(const MergeLaunch& L, hipStream_t st);
+constexpr int kSparseAfterAccum = 100;  // launch_sparse_encode phase: everything after the accumulate launch
+hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, uint32_t* tileptr, uint32_t* unsorted,
+                               hipStream_t st);
 
 }  // namespace hp

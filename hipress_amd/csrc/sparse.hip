@@ -57,8 +57,10 @@ __device__ __forceinline__ unsigned digit_mask_above(int pass) {
 
 // ---- 0. accumulate -------------------------------------------------------------
 
-template <bool FAST, bool DGC>
-__device__ __forceinline__ void sparse_accum_tile(const Seg& s, unsigned tile, const SparseWs& ws) {
+// gload(j, e) supplies the four gradient values of step j (element e): global
+// memory for the encoders, the LDS tile of merged peers for decode-and-merge.
+template <bool FAST, bool DGC, class GLoad>
+__device__ __forceinline__ void sparse_accum_tile(const Seg& s, unsigned tile, const SparseWs& ws, GLoad gload) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long n = (long long)s.n;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
@@ -68,7 +70,7 @@ __device__ __forceinline__ void sparse_accum_tile(const Seg& s, unsigned tile, c
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         long long e = base + j * 256 + lane * 4;
-        g[j] = load4<FAST>(s.g, e, n);
+        g[j] = gload(j, e);
         a[j] = load4<FAST>(s.s1, e, n);
         if (DGC) m[j] = load4<FAST>(s.s0, e, n);
     }
@@ -116,22 +118,27 @@ __device__ __forceinline__ void sparse_accum_tile(const Seg& s, unsigned tile, c
     }
 }
 
+// Tile 0 of a tensor resets that tensor's select-pass state.
+__device__ __forceinline__ void sparse_reset_select(const Seg& s, const SparseWs& ws) {
+    uint32_t* h = ws.hist + (unsigned long long)s.id * (3 * kBins);
+    for (unsigned i = threadIdx.x; i < 3 * kBins; i += kBlock) h[i] = 0;
+    if (threadIdx.x < kCtlWords) ws.ctl[s.id * kCtlWords + threadIdx.x] = threadIdx.x == kCtlK ? s.ks : 0u;
+    if (threadIdx.x == 0) {
+        ws.thr[2 * s.id] = 0;
+        ws.thr[2 * s.id + 1] = kNoQuota;
+    }
+}
+
 template <class Src, bool DGC>
 __global__ __launch_bounds__(kBlock) void sparse_accum_kernel(Src src, SparseWs ws) {
     unsigned tile;
     const Seg& s = src.get(tile, blockIdx.x);
-    if (tile == 0) {
-        // this tensor's select-pass state starts from zero every call
-        uint32_t* h = ws.hist + (unsigned long long)s.id * (3 * kBins);
-        for (unsigned i = threadIdx.x; i < 3 * kBins; i += kBlock) h[i] = 0;
-        if (threadIdx.x < kCtlWords) ws.ctl[s.id * kCtlWords + threadIdx.x] = threadIdx.x == kCtlK ? s.ks : 0u;
-        if (threadIdx.x == 0) {
-            ws.thr[2 * s.id] = 0;
-            ws.thr[2 * s.id + 1] = kNoQuota;
-        }
-    }
-    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) sparse_accum_tile<true, DGC>(s, tile, ws);
-    else sparse_accum_tile<false, DGC>(s, tile, ws);
+    if (tile == 0) sparse_reset_select(s, ws);
+    const long long n = (long long)s.n;
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n)
+        sparse_accum_tile<true, DGC>(s, tile, ws, [&](int, long long e) { return load4<true>(s.g, e, n); });
+    else
+        sparse_accum_tile<false, DGC>(s, tile, ws, [&](int, long long e) { return load4<false>(s.g, e, n); });
 }
 
 // ---- 1-3. select -----------------------------------------------------------------
@@ -286,42 +293,63 @@ __global__ __launch_bounds__(kBlock) void sparse_count_kernel(Src src, SparseWs 
 
 // ---- 5. scan ----------------------------------------------------------------------
 
-// In-place exclusive scan of nw {above, equal} pairs by one workgroup; returns
-// the totals to every thread.
-__device__ __forceinline__ void block_scan_pairs(uint32_t* c, unsigned nw, unsigned (&sh)[2][kBlock],
+// In-place exclusive scan of nw {above, equal} pairs by one workgroup of
+// kScanBlock threads; returns the totals to every thread.  Each wavefront owns a
+// contiguous span: one coalesced sweep for the span totals, a second one that
+// scans 64 pairs at a time with shuffles.
+constexpr int kScanBlock = 1024;
+constexpr int kScanWaves = kScanBlock / 64;
+
+__device__ __forceinline__ unsigned wave_incl_scan(unsigned x, unsigned lane) {
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        unsigned y = (unsigned)__shfl_up((int)x, d, 64);
+        if ((int)lane >= d) x += y;
+    }
+    return x;
+}
+
+__device__ __forceinline__ void block_scan_pairs(uint32_t* c, unsigned nw, unsigned (&sh)[2][kScanWaves],
                                                  unsigned& tot_gt, unsigned& tot_eq) {
-    const unsigned t = threadIdx.x;
-    const unsigned per = (nw + kBlock - 1) / kBlock;
-    const unsigned lo = t * per, hi = lo + per < nw ? lo + per : nw;
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    uint2* c2 = reinterpret_cast<uint2*>(c);
+    const unsigned span = ((nw + kScanWaves - 1) / kScanWaves + 63u) & ~63u;
+    const unsigned lo = wave * span < nw ? wave * span : nw;
+    const unsigned hi = lo + span < nw ? lo + span : nw;
     unsigned sg = 0, se = 0;
-    for (unsigned i = lo; i < hi; ++i) {
-        sg += c[2 * i];
-        se += c[2 * i + 1];
+    for (unsigned i = lo + lane; i < hi; i += 64) {
+        uint2 v = c2[i];
+        sg += v.x;
+        se += v.y;
     }
-    sh[0][t] = sg;
-    sh[1][t] = se;
+    sg = wave_sum_u(sg);
+    se = wave_sum_u(se);
+    __syncthreads();  // sh may still be read from a previous call
+    if (lane == 0) {
+        sh[0][wave] = sg;
+        sh[1][wave] = se;
+    }
     __syncthreads();
-    // Hillis-Steele inclusive scan over the 256 thread sums
-    for (int d = 1; d < kBlock; d <<= 1) {
-        unsigned ag = 0, ae = 0;
-        if ((int)t >= d) {
-            ag = sh[0][t - d];
-            ae = sh[1][t - d];
+    unsigned bg = 0, be = 0;
+    tot_gt = 0;
+    tot_eq = 0;
+#pragma unroll
+    for (int w = 0; w < kScanWaves; ++w) {
+        unsigned g = sh[0][w], e = sh[1][w];
+        if ((unsigned)w < wave) {
+            bg += g;
+            be += e;
         }
-        __syncthreads();
-        sh[0][t] += ag;
-        sh[1][t] += ae;
-        __syncthreads();
+        tot_gt += g;
+        tot_eq += e;
     }
-    tot_gt = sh[0][kBlock - 1];
-    tot_eq = sh[1][kBlock - 1];
-    unsigned og = sh[0][t] - sg, oe = sh[1][t] - se;  // exclusive offsets of this thread's chunk
-    for (unsigned i = lo; i < hi; ++i) {
-        unsigned cg = c[2 * i], ce = c[2 * i + 1];
-        c[2 * i] = og;
-        c[2 * i + 1] = oe;
-        og += cg;
-        oe += ce;
+    for (unsigned i0 = lo; i0 < hi; i0 += 64) {
+        unsigned i = i0 + lane;
+        uint2 v = i < hi ? c2[i] : make_uint2(0u, 0u);
+        unsigned ig = wave_incl_scan(v.x, lane), ie = wave_incl_scan(v.y, lane);
+        if (i < hi) c2[i] = make_uint2(bg + ig - v.x, be + ie - v.y);
+        bg += (unsigned)__builtin_amdgcn_readlane((int)ig, 63);
+        be += (unsigned)__builtin_amdgcn_readlane((int)ie, 63);
     }
     __syncthreads();
 }
@@ -339,18 +367,17 @@ template <class Visit>
 __device__ __forceinline__ unsigned block_kth_largest(RadixScratch& sc, unsigned k, Visit visit) {
     unsigned prefix = 0, mask = 0;
     for (int shift = 24; shift >= 0; shift -= 8) {
-        for (unsigned i = threadIdx.x; i < 16 * 257; i += kBlock) (&sc.hist[0][0])[i] = 0;
+        for (unsigned i = threadIdx.x; i < 16 * 257; i += blockDim.x) (&sc.hist[0][0])[i] = 0;
         __syncthreads();
         visit([&](unsigned key) {
             if ((key & mask) == prefix) atomicAdd(&sc.hist[threadIdx.x & 15u][(key >> shift) & 255u], 1u);
         });
         __syncthreads();
-        {
-            unsigned t = threadIdx.x;  // kBlock == 256 bins: fold the 16 copies
+        if (threadIdx.x < 256) {  // fold the 16 copies, one bin per thread
+            unsigned t = threadIdx.x;
             unsigned c = 0;
 #pragma unroll
             for (int r = 0; r < 16; ++r) c += sc.hist[r][t];
-            __syncthreads();
             sc.hist[0][t] = c;
         }
         __syncthreads();
@@ -375,8 +402,8 @@ __device__ __forceinline__ unsigned block_kth_largest(RadixScratch& sc, unsigned
 }
 
 template <class SegSrc>
-__global__ __launch_bounds__(kBlock) void sparse_scan_kernel(SegSrc src, SparseWs ws) {
-    __shared__ unsigned sh[2][kBlock];
+__global__ __launch_bounds__(kScanBlock) void sparse_scan_kernel(SegSrc src, SparseWs ws) {
+    __shared__ unsigned sh[2][kScanWaves];
     __shared__ RadixScratch sc;
     const Seg& s = src.at(blockIdx.x);
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
@@ -397,7 +424,7 @@ __global__ __launch_bounds__(kBlock) void sparse_scan_kernel(SegSrc src, SparseW
         const unsigned long long ngroups = (unsigned long long)s.ntiles * 64;
         const uint32_t* gmax = ws.gmax + (unsigned long long)s.tile0 * 64;
         thr = block_kth_largest(sc, s.cap, [&](auto f) {
-            for (unsigned long long g = wave; g < ngroups; g += 4) {
+            for (unsigned long long g = wave; g < ngroups; g += kScanWaves) {
                 unsigned gm = gmax[g];
                 if (gm >= old && gm > 0u) {
                     long long e = (long long)g * 64 + lane;
@@ -406,7 +433,7 @@ __global__ __launch_bounds__(kBlock) void sparse_scan_kernel(SegSrc src, SparseW
                 }
             }
         });
-        for (unsigned t = wave; t < nw; t += 4) {
+        for (unsigned t = wave; t < nw; t += kScanWaves) {
             unsigned gt, eq;
             count_tile(s, ws, t, thr, lane, gt, eq);
             if (lane == 0) {
@@ -600,33 +627,93 @@ __global__ __launch_bounds__(kBlock) void sparse_scatter_kernel(Src src) {
     }
 }
 
-// Scatter-ADD of every peer of a chunk into its (already zeroed) aggregate.
-template <class MSrc>
-__global__ __launch_bounds__(kBlock) void sparse_scatter_add_kernel(MSrc src, int npeers) {
+// ---- sparse decode-and-merge -------------------------------------------------------
+// Pairs arrive in ascending index order, so the pairs of one 4096-element tile are
+// one contiguous run of every peer's payload.  A small index kernel finds those
+// runs (and notices a payload that is not sorted); the merge kernel then gives
+// every tile to one workgroup, which adds the peers' runs into an LDS tile in
+// peer order, writes the aggregate once and, if asked, continues with the
+// GradDrop-style re-encode pass on the values it already holds.  Summation order
+// per element is the peer order, as in a sequential implementation.
+
+// first position in idx[0, nnz) whose index is >= key
+__device__ __forceinline__ unsigned lower_bound_idx(const int32_t* idx, unsigned nnz, long long key) {
+    unsigned lo = 0, hi = nnz;
+    while (lo < hi) {
+        unsigned mid = (lo + hi) >> 1;
+        if ((long long)idx[mid] < key) lo = mid + 1;
+        else hi = mid;
+    }
+    return lo;
+}
+
+// One workgroup per (chunk, peer): tile pointers ptr[t] = first pair of tile t
+// (ptr[ntiles] = nnz) and a flag that is set when the indices are not ascending.
+template <class MSegSrc>
+__global__ __launch_bounds__(kBlock) void sparse_merge_index_kernel(MSegSrc src, uint32_t* tileptr, uint32_t* unsorted,
+                                                                    int npeers) {
+    __shared__ unsigned bad;
+    const unsigned chunk = blockIdx.x / npeers, p = blockIdx.x % npeers;
+    const MergeSeg& m = src.at(chunk);
+    const int32_t* idx;
+    const float* val;
+    const unsigned nnz = sparse_header(m.peer[p], m.peer_slots[p], idx, val);
+    const unsigned nt = m.s.ntiles;
+    uint32_t* ptr = tileptr + m.tp0 + (unsigned long long)p * (nt + 1);
+    if (threadIdx.x == 0) bad = 0;
+    __syncthreads();
+    unsigned b = 0;
+    for (unsigned j = threadIdx.x + 1; j < nnz; j += kBlock) b |= idx[j - 1] > idx[j];
+    if (b) bad = 1;  // benign race: every writer stores 1
+    for (unsigned t = threadIdx.x; t <= nt; t += kBlock) ptr[t] = lower_bound_idx(idx, nnz, (long long)t * kTile);
+    __syncthreads();
+    if (threadIdx.x == 0) unsorted[(unsigned long long)chunk * npeers + p] = bad;
+}
+
+template <class MSrc, bool REENC>
+__global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs ws, const uint32_t* tileptr,
+                                                              const uint32_t* unsorted, int npeers) {
+    __shared__ __attribute__((aligned(16))) float lds[kTile];
     unsigned tile;
     const MergeSeg& m = src.get(tile, blockIdx.x);
+    const Seg& s = m.s;
+    const long long n = (long long)s.n;
+    const long long t_lo = (long long)tile * kTile, t_hi = t_lo + kTile < n ? t_lo + kTile : n;
+    for (unsigned i = threadIdx.x; i < kTile; i += kBlock) lds[i] = 0.f;
+    __syncthreads();
     for (int p = 0; p < npeers; ++p) {
         const int32_t* idx;
         const float* val;
-        const unsigned slots = m.peer_slots[p];
-        const unsigned nnz = sparse_header(m.peer[p], slots, idx, val);
-        const unsigned per = (slots + m.s.ntiles - 1) / m.s.ntiles;
-        const unsigned long long lo = (unsigned long long)tile * per;
-        unsigned long long hi = lo + per;
-        if (hi > nnz) hi = nnz;
-        for (unsigned long long j = lo + threadIdx.x; j < hi; j += kBlock) {
-            long long i = idx[j];
-            if (i >= 0 && i < (long long)m.s.n) atomicAdd(&m.s.out[i], val[j]);
+        const unsigned nnz = sparse_header(m.peer[p], m.peer_slots[p], idx, val);
+        unsigned lo = 0, hi = nnz;
+        if (!unsorted[(unsigned long long)s.id * npeers + p]) {
+            const uint32_t* ptr = tileptr + m.tp0 + (unsigned long long)p * (s.ntiles + 1);
+            lo = ptr[tile];
+            hi = ptr[tile + 1];
+            if (hi > nnz) hi = nnz;
         }
+        for (unsigned j = lo + threadIdx.x; j < hi; j += kBlock) {
+            long long i = idx[j];
+            if (i >= t_lo && i < t_hi) atomicAdd(&lds[i - t_lo], val[j]);  // distinct addresses unless a peer repeats an index
+        }
+        __syncthreads();
     }
-}
-
-template <class MSrc>
-__global__ __launch_bounds__(kBlock) void merge_zero_fill_kernel(MSrc src) {
-    unsigned tile;
-    const MergeSeg& m = src.get(tile, blockIdx.x);
-    if (m.s.aligned && (unsigned long long)(tile + 1) * kTile <= m.s.n) zero_tile<true>(m.s.out, (long long)m.s.n, tile);
-    else zero_tile<false>(m.s.out, (long long)m.s.n, tile);
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const bool fast = s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n;
+    auto from_lds = [&](int j, long long) { return *reinterpret_cast<const f4*>(&lds[wave * kWaveTile + j * 256 + lane * 4]); };
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = t_lo + wave * kWaveTile + j * 256 + lane * 4;
+        if (fast) st4(s.out + e, from_lds(j, e));
+        else st4_guard(s.out, e, n, from_lds(j, e));
+    }
+    if (REENC) {
+        // the re-encode descriptor of this chunk: same tile numbering, g replaced by the LDS tile
+        const Seg& r = m.r;
+        if (tile == 0) sparse_reset_select(r, ws);
+        if (fast) sparse_accum_tile<true, false>(r, tile, ws, from_lds);
+        else sparse_accum_tile<false, false>(r, tile, ws, from_lds);
+    }
 }
 
 // =============================================================================
@@ -637,7 +724,7 @@ template <class Src, class SegSrcT>
 static hipError_t sparse_encode_src(const Src& src, const Src& ssrc_tiles, const SegSrcT& ssrc, unsigned ntiles,
                                     unsigned nstiles, unsigned nsegs, bool dgc, const SparseWs& ws, int phase,
                                     hipStream_t st) {
-    auto on = [&](int p) { return phase < 0 || phase == p; };
+    auto on = [&](int p) { return phase < 0 || phase == p || (phase == kSparseAfterAccum && p > 0); };
     const unsigned g4 = (ntiles + 3) / 4;
     if (on(0)) {
         if (dgc) hipLaunchKernelGGL((sparse_accum_kernel<Src, true>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
@@ -647,13 +734,13 @@ static hipError_t sparse_encode_src(const Src& src, const Src& ssrc_tiles, const
         if (on(1 + pass) && nstiles)
             hipLaunchKernelGGL((sparse_select_kernel<Src>), dim3(nstiles), dim3(kBlock), 0, st, ssrc_tiles, ws, pass);
     if (on(4)) hipLaunchKernelGGL((sparse_count_kernel<Src>), dim3(g4), dim3(kBlock), 0, st, src, ws, ntiles);
-    if (on(5)) hipLaunchKernelGGL((sparse_scan_kernel<SegSrcT>), dim3(nsegs), dim3(kBlock), 0, st, ssrc, ws);
+    if (on(5)) hipLaunchKernelGGL((sparse_scan_kernel<SegSrcT>), dim3(nsegs), dim3(kScanBlock), 0, st, ssrc, ws);
     if (on(6)) hipLaunchKernelGGL((sparse_emit_kernel<Src>), dim3(g4), dim3(kBlock), 0, st, src, ws, ntiles);
     return hipGetLastError();
 }
 
 // phase < 0 runs the whole sequence; 0..6 run one launch of it (accumulate,
-// three select passes, count, scan, emit).
+// three select passes, count, scan, emit); kSparseAfterAccum runs launches 1..6.
 hipError_t launch_sparse_encode(const Launch& L, bool dgc, const SparseWs& ws, int phase, hipStream_t st) {
     if (L.ntiles == 0) return hipSuccess;
     if (L.single)
@@ -680,16 +767,33 @@ hipError_t launch_sparse_decode(const Launch& L, hipStream_t st) {
     return hipGetLastError();
 }
 
-hipError_t launch_sparse_merge_scatter(const MergeLaunch& L, hipStream_t st) {
+// Index kernel + tile-owner merge.  With L.reencode the merge kernel also runs launch 0
+// of the GradDrop-style re-encode (the caller follows with launch_sparse_encode phases 1..6).
+hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, uint32_t* tileptr, uint32_t* unsorted,
+                               hipStream_t st) {
     if (L.ntiles == 0) return hipSuccess;
     if (L.single) {
+        MergeSingleSegSrc isrc{L.seg};
+        hipLaunchKernelGGL((sparse_merge_index_kernel<MergeSingleSegSrc>), dim3(L.npeers), dim3(kBlock), 0, st, isrc,
+                           tileptr, unsorted, L.npeers);
         MergeSingleSrc src{L.seg};
-        hipLaunchKernelGGL((merge_zero_fill_kernel<MergeSingleSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
-        hipLaunchKernelGGL((sparse_scatter_add_kernel<MergeSingleSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src, L.npeers);
+        if (L.reencode)
+            hipLaunchKernelGGL((sparse_merge_kernel<MergeSingleSrc, true>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
+                               tileptr, unsorted, L.npeers);
+        else
+            hipLaunchKernelGGL((sparse_merge_kernel<MergeSingleSrc, false>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
+                               tileptr, unsorted, L.npeers);
     } else {
+        MergeBatchSegSrc isrc{L.dsegs};
+        hipLaunchKernelGGL((sparse_merge_index_kernel<MergeBatchSegSrc>), dim3(L.nsegs * L.npeers), dim3(kBlock), 0, st,
+                           isrc, tileptr, unsorted, L.npeers);
         MergeBatchSrc src{L.dsegs, L.dmap};
-        hipLaunchKernelGGL((merge_zero_fill_kernel<MergeBatchSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
-        hipLaunchKernelGGL((sparse_scatter_add_kernel<MergeBatchSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src, L.npeers);
+        if (L.reencode)
+            hipLaunchKernelGGL((sparse_merge_kernel<MergeBatchSrc, true>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
+                               tileptr, unsorted, L.npeers);
+        else
+            hipLaunchKernelGGL((sparse_merge_kernel<MergeBatchSrc, false>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
+                               tileptr, unsorted, L.npeers);
     }
     return hipGetLastError();
 }

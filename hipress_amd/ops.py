@@ -289,8 +289,8 @@ def dgc_decode_merge(compressed_list, aggregate, accumulator=None, out_compresse
         _f32(accumulator, "accumulator", aggregate); _u8(out_compressed, "out_compressed", aggregate)
         _same_numel(aggregate, accumulator, "aggregate", "accumulator")
     with torch.cuda.device(aggregate.device):
-        if accumulator is not None:
-            ws = _workspace(aggregate, size(L.hipress_sparse_workspace_bytes(n, float(ratio)), "sparse_workspace_bytes"))
+        ws = _workspace(aggregate, size(L.hipress_sparse_merge_workspace_bytes(n, P, float(ratio), int(accumulator is not None)),
+                                        "sparse_merge_workspace_bytes"))
         check(L.hipress_sparse_decode_merge(
             ptrs, lens, P, _p(aggregate), n, _p(accumulator), _p(out_compressed),
             out_compressed.numel() if out_compressed is not None else 0, float(ratio),

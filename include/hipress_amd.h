@@ -80,6 +80,7 @@ int64_t hipress_sparse_capacity(int64_t n, double ratio);
 int64_t hipress_sparse_payload_bytes(int64_t n, double ratio);
 int64_t hipress_onebit_workspace_bytes(int64_t n);
 int64_t hipress_sparse_workspace_bytes(int64_t n, double ratio);
+int64_t hipress_sparse_merge_workspace_bytes(int64_t n, int32_t npeers, double ratio, int32_t reencode);
 
 /* ---- TBQ: threshold two-bit quantisation with error feedback ------------- */
 /* Replaces <Func>_body for the built-in "tbq" algorithm
@@ -149,6 +150,10 @@ int hipress_onebit_decode_merge(const void *const *payloads, const int64_t *payl
                                 int32_t npeers, float *aggregate, int64_t n, void *stream);
 int hipress_terngrad_decode_merge(const void *const *payloads, const int64_t *payload_bytes,
                                   int32_t npeers, float *aggregate, int64_t n, void *stream);
+/* Sparse payloads must hold their pairs in ascending index order (the encoders
+ * here write them so); a payload that does not is still merged correctly, but
+ * slowly.  workspace: hipress_sparse_merge_workspace_bytes(n, npeers, ratio,
+ * accumulator != NULL). */
 int hipress_sparse_decode_merge(const void *const *payloads, const int64_t *payload_bytes,
                                 int32_t npeers, float *aggregate, int64_t n, float *accumulator,
                                 void *out_payload, int64_t out_payload_bytes, double ratio,

@@ -364,6 +364,29 @@ def test_sparse_decode_merge(hp, n):
     np.testing.assert_array_equal(host(acc), want_acc)
 
 
+def test_sparse_decode_merge_is_exact_in_peer_order_and_accepts_unsorted(hp):
+    n, P, ratio = 300000, 8, 0.001
+    rng = np.random.default_rng(17)
+    pays = []
+    for p in range(P):
+        g = rng.normal(0, 1e-3, n).astype(F)
+        g[:30] += 1.0 + p * 0.37  # the same leading entries in every peer: sums depend on order
+        pays.append(oracle.dgc_encode(g, np.zeros(n, F), np.zeros(n, F), 0.9, ratio)[0])
+    agg = torch.full((n,), 7.0, device="cuda")
+    hp.dgc_decode_merge([dev(p) for p in pays], agg)
+    np.testing.assert_array_equal(host(agg), oracle.sparse_decode_merge(pays, n))  # peer order => bit-exact
+    # shuffle the pairs of two peers: still the same aggregate
+    shuffled = [p.copy() for p in pays]
+    for q in (1, 5):
+        nnz, _, cap, _, idx, val = oracle.sparse_unpack(shuffled[q])
+        perm = rng.permutation(nnz)
+        shuffled[q][16 : 16 + 4 * nnz].view(np.int32)[:] = idx[perm]
+        shuffled[q][16 + 4 * cap : 16 + 4 * cap + 4 * nnz].view(F)[:] = val[perm]
+    agg.fill_(7.0)
+    hp.dgc_decode_merge([dev(p) for p in shuffled], agg)
+    np.testing.assert_array_equal(host(agg), oracle.sparse_decode_merge(pays, n))
+
+
 # ---------------------------------------------------------------- batched launches
 def mixed_sizes():
     return [1728, 64, 36864, 64, 73728, 128, 4097, 1, 262144, 512, 1000003, 1000]
@@ -460,6 +483,52 @@ def test_batch_matches_oracle(hp, alg):
             np.testing.assert_array_equal(host(t["accumulator"]), acc)
             dec = oracle.sparse_decode(want, n)
         np.testing.assert_array_equal(host(t["out"]), dec)
+    b.close()
+
+
+@pytest.mark.parametrize("alg,ratio", [("dgc", 0.001), ("graddrop", 0.01)])
+def test_sparse_batch_many_steps(hp, alg, ratio):
+    """A batch keeps a threshold prediction between steps and stages candidates
+    against it.  The steps below make the prediction hold, fail (threshold drops),
+    overflow single staging areas (a local burst) and overflow the payload capacity
+    (many equal large values); every step must still match the oracle bit for bit."""
+    rng = np.random.default_rng(91)
+    sizes = [1000003, 262144, 4097, 70001, 300000, 64]
+    tensors, refs = [], []
+    for n in sizes:
+        t = {"gradient": torch.zeros(n, device="cuda"), "accumulator": torch.zeros(n, device="cuda"),
+             "compressed": payload(hp.sparse_payload_bytes(n, ratio)), "out": torch.empty(n, device="cuda")}
+        ref = {"acc": np.zeros(n, F)}
+        if alg == "dgc":
+            t["momentum"] = torch.zeros(n, device="cuda")
+            ref["mom"] = np.zeros(n, F)
+        tensors.append(t)
+        refs.append(ref)
+    b = hp.Batch(alg, tensors, momentum_factor=0.9, ratio=ratio)
+    plan = ["plain", "plain", "plain", "tiny", "plain", "burst", "big", "ties", "plain", "plain"]
+    for step, kind in enumerate(plan):
+        for t, ref in zip(tensors, refs):
+            n = t["gradient"].numel()
+            scale = {"tiny": 1e-5, "big": 5e-3}.get(kind, 1e-3)
+            g = rng.normal(0, scale, n).astype(F)
+            if kind == "burst" and n > 5000:
+                g[3000:5000] += 0.05  # 2000 neighbours far above the threshold
+            if kind == "ties" and n > 5000:
+                g[::7] = 0.25  # far more equal values than the payload has slots
+            t["gradient"].copy_(dev(g))
+            ref["g"] = g
+        b.encode()
+        b.decode()
+        for t, ref in zip(tensors, refs):
+            n = ref["g"].size
+            if alg == "dgc":
+                want, ref["mom"], ref["acc"] = oracle.dgc_encode(ref["g"], ref["mom"], ref["acc"], 0.9, ratio)
+                np.testing.assert_array_equal(host(t["momentum"]), ref["mom"], err_msg=f"step {step} {kind} n={n}")
+            else:
+                want, ref["acc"] = oracle.graddrop_encode(ref["g"], ref["acc"], ratio)
+            check_sparse(host(t["compressed"]), want)
+            np.testing.assert_array_equal(host(t["accumulator"]), ref["acc"], err_msg=f"step {step} {kind} n={n}")
+            np.testing.assert_array_equal(host(t["out"]), oracle.sparse_decode(want, n))
     b.close()
 
 
