@@ -59,8 +59,11 @@ __device__ __forceinline__ unsigned digit_mask_above(int pass) {
 
 // gload(j, e) supplies the four gradient values of step j (element e): global
 // memory for the encoders, the LDS tile of merged peers for decode-and-merge.
-template <bool FAST, bool DGC, class GLoad>
-__device__ __forceinline__ void sparse_accum_tile(const Seg& s, unsigned tile, const SparseWs& ws, GLoad gload) {
+// aload(j, e) supplies the accumulator values the same way (decode-and-merge
+// loads them before it starts merging, to have them in flight early).
+template <bool FAST, bool DGC, class GLoad, class ALoad>
+__device__ __forceinline__ void sparse_accum_tile(const Seg& s, unsigned tile, const SparseWs& ws, GLoad gload,
+                                                  ALoad aload) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long n = (long long)s.n;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
@@ -71,7 +74,7 @@ __device__ __forceinline__ void sparse_accum_tile(const Seg& s, unsigned tile, c
     for (int j = 0; j < 4; ++j) {
         long long e = base + j * 256 + lane * 4;
         g[j] = gload(j, e);
-        a[j] = load4<FAST>(s.s1, e, n);
+        a[j] = aload(j, e);
         if (DGC) m[j] = load4<FAST>(s.s0, e, n);
     }
 #pragma unroll
@@ -136,9 +139,11 @@ __global__ __launch_bounds__(kBlock) void sparse_accum_kernel(Src src, SparseWs 
     if (tile == 0) sparse_reset_select(s, ws);
     const long long n = (long long)s.n;
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n)
-        sparse_accum_tile<true, DGC>(s, tile, ws, [&](int, long long e) { return load4<true>(s.g, e, n); });
+        sparse_accum_tile<true, DGC>(s, tile, ws, [&](int, long long e) { return load4<true>(s.g, e, n); },
+                                     [&](int, long long e) { return load4<true>(s.s1, e, n); });
     else
-        sparse_accum_tile<false, DGC>(s, tile, ws, [&](int, long long e) { return load4<false>(s.g, e, n); });
+        sparse_accum_tile<false, DGC>(s, tile, ws, [&](int, long long e) { return load4<false>(s.g, e, n); },
+                                      [&](int, long long e) { return load4<false>(s.s1, e, n); });
 }
 
 // ---- 1-3. select -----------------------------------------------------------------
@@ -674,14 +679,28 @@ template <class MSrc, bool REENC>
 __global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs ws, const uint32_t* tileptr,
                                                               const uint32_t* unsorted, int npeers) {
     __shared__ __attribute__((aligned(16))) float lds[kTile];
+    __shared__ unsigned plo[kMaxPeers], pcnt[kMaxPeers], pcap[kMaxPeers];
     unsigned tile;
     const MergeSeg& m = src.get(tile, blockIdx.x);
     const Seg& s = m.s;
+    const Seg& r = m.r;  // re-encode descriptor of this chunk: same tile numbering
     const long long n = (long long)s.n;
     const long long t_lo = (long long)tile * kTile, t_hi = t_lo + kTile < n ? t_lo + kTile : n;
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const bool fast = s.aligned && (!REENC || r.aligned) && (unsigned long long)(tile + 1) * kTile <= s.n;
+    // the accumulator tile of the re-encode is requested first: it is in flight while the peers are merged
+    f4 apre[4];
+    if (REENC) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            long long e = t_lo + wave * kWaveTile + j * 256 + lane * 4;
+            apre[j] = fast ? ld4(r.s1 + e) : ld4_guard(r.s1, e, n);
+        }
+    }
     for (unsigned i = threadIdx.x; i < kTile; i += kBlock) lds[i] = 0.f;
-    __syncthreads();
-    for (int p = 0; p < npeers; ++p) {
+    // one thread per peer: where this tile's pairs are in that peer's payload
+    if ((int)threadIdx.x < npeers) {
+        const unsigned p = threadIdx.x;
         const int32_t* idx;
         const float* val;
         const unsigned nnz = sparse_header(m.peer[p], m.peer_slots[p], idx, val);
@@ -691,15 +710,43 @@ __global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs
             lo = ptr[tile];
             hi = ptr[tile + 1];
             if (hi > nnz) hi = nnz;
+            if (lo > hi) lo = hi;
         }
-        for (unsigned j = lo + threadIdx.x; j < hi; j += kBlock) {
-            long long i = idx[j];
-            if (i >= t_lo && i < t_hi) atomicAdd(&lds[i - t_lo], val[j]);  // distinct addresses unless a peer repeats an index
-        }
-        __syncthreads();
+        plo[p] = lo;
+        pcnt[p] = hi - lo;
+        pcap[p] = reinterpret_cast<const uint32_t*>(m.peer[p])[2];
     }
-    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const bool fast = s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n;
+    __syncthreads();
+    unsigned total = 0;
+    for (int p = 0; p < npeers; ++p) total += pcnt[p];
+    // The pairs of all peers, flattened peer by peer, are dealt out one per thread, so a
+    // whole round is one memory round trip; they are then added peer by peer (sums must
+    // follow the peer order; within a peer the indices are distinct).
+    for (unsigned base = 0; base < total; base += kBlock) {
+        const unsigned f = base + threadIdx.x;
+        unsigned myp = 0, before = 0;
+        while (myp + 1 < (unsigned)npeers && f >= before + pcnt[myp]) before += pcnt[myp++];
+        const bool have = f < total;
+        long long i = -1;
+        float v = 0.f;
+        if (have) {
+            const unsigned j = plo[myp] + (f - before);
+            i = reinterpret_cast<const int32_t*>(m.peer[myp] + kHeaderBytes)[j];
+            v = reinterpret_cast<const float*>(m.peer[myp] + kHeaderBytes + 4ull * pcap[myp])[j];
+        }
+        const bool inside = have && i >= t_lo && i < t_hi;
+        // peers present in this round (uniform): first and last flat entry of the round
+        unsigned pfirst = 0, acc0 = 0;
+        while (pfirst + 1 < (unsigned)npeers && base >= acc0 + pcnt[pfirst]) acc0 += pcnt[pfirst++];
+        const unsigned lastf = (base + kBlock < total ? base + kBlock : total) - 1;
+        unsigned plast = pfirst, acc1 = acc0;
+        while (plast + 1 < (unsigned)npeers && lastf >= acc1 + pcnt[plast]) acc1 += pcnt[plast++];
+        for (unsigned p = pfirst; p <= plast; ++p) {
+            if (inside && myp == p) atomicAdd(&lds[i - t_lo], v);
+            __syncthreads();
+        }
+    }
+    __syncthreads();
     auto from_lds = [&](int j, long long) { return *reinterpret_cast<const f4*>(&lds[wave * kWaveTile + j * 256 + lane * 4]); };
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -708,11 +755,10 @@ __global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs
         else st4_guard(s.out, e, n, from_lds(j, e));
     }
     if (REENC) {
-        // the re-encode descriptor of this chunk: same tile numbering, g replaced by the LDS tile
-        const Seg& r = m.r;
         if (tile == 0) sparse_reset_select(r, ws);
-        if (fast) sparse_accum_tile<true, false>(r, tile, ws, from_lds);
-        else sparse_accum_tile<false, false>(r, tile, ws, from_lds);
+        auto from_pre = [&](int j, long long) { return apre[j]; };
+        if (fast) sparse_accum_tile<true, false>(r, tile, ws, from_lds, from_pre);
+        else sparse_accum_tile<false, false>(r, tile, ws, from_lds, from_pre);
     }
 }
 
