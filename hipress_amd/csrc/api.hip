@@ -15,8 +15,6 @@ using namespace hp;
 
 namespace {
 
-constexpr int64_t kSampleFrom = 262144;  // tensors at least this large are sampled at stride 100
-constexpr int64_t kSampleStride = 100;
 constexpr int64_t kSampleTile = 4096;    // sample keys per workgroup of the select passes
 
 inline bool mis(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }

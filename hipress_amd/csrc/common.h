@@ -21,6 +21,8 @@ constexpr int kWaveTile = 1024;   // elements per wavefront per tile
 constexpr int kTile = 4096;       // elements per workgroup
 constexpr int kHeaderBytes = 16;
 constexpr int kMaxPeers = 16;
+constexpr int kSampleStride = 100;      // sparse: every 100th element of a large tensor is a sample
+constexpr long long kSampleFrom = 262144;  // sparse: tensors at least this large are sampled
 
 // One tensor (or one chunk) as the kernels see it.  Batched launches index a
 // device-resident array of these through a tile map; single-tensor launches

@@ -110,7 +110,7 @@ __device__ __forceinline__ void sparse_accum_tile(const Seg& s, unsigned tile, c
             if (e + 2 < n) sample[e + 2] = k2;
             if (e + 3 < n) sample[e + 3] = k3;
         } else {  // sample positions are q*S + S/2; at most one falls into [e, e+4)
-            const unsigned long long S = s.sstride, h = S / 2;
+            constexpr unsigned long long S = kSampleStride, h = S / 2;  // a constant: division by multiply
             unsigned long long q = ((unsigned long long)e + (S - 1 - h)) / S;  // first q with q*S+h >= e
             unsigned long long p = q * S + h;
             if (p < (unsigned long long)e + 4 && q < s.ns) {

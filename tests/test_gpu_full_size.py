@@ -1,0 +1,203 @@
+"""GPU parity at the sizes the benchmark configurations name: whole gradient sets
+through the batched C ABI, compared with the CPU oracle where the oracle finishes
+in seconds and through size-independent properties everywhere.  Also checks that
+a captured HIP graph of encode+decode replays to the eager results."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+F = np.float32
+
+
+@pytest.fixture(scope="module")
+def hp():
+    import hipress_amd
+
+    assert torch.cuda.is_available()
+    hipress_amd._lib.lib()
+    return hipress_amd
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def test_onebit_vgg19_full_set(hp):
+    """configs[1]: onebit over the 38 VGG19 tensors, 143,667,240 elements."""
+    from hipress_amd import workloads as W
+
+    sizes = W.vgg19_sizes()
+    grads = W.normal_set(sizes, torch.device("cuda:0"), 0, log_sigma_range=(-4.0, -2.0))
+    ts = [{"gradient": g, "residual": torch.zeros_like(g), "out": torch.empty_like(g),
+           "compressed": torch.full((hp.onebit_payload_bytes(g.numel()),), 0xAB, dtype=torch.uint8, device="cuda")}
+          for g in grads]
+    b = hp.Batch("onebit", ts)
+    b.encode()
+    b.decode()
+    for t, n in zip(ts, sizes):
+        g = host(t["gradient"])
+        got = host(t["compressed"])
+        s = got[:4].view(F)[0]
+        s_ref = oracle.onebit_scale(g, np.zeros(n, F))
+        assert abs(float(s) - float(s_ref)) <= 1e-5 * float(s_ref), (n, s, s_ref)
+        want, r = oracle.onebit_encode(g, np.zeros(n, F), scale=s)
+        np.testing.assert_array_equal(got, want, err_msg=f"payload n={n}")
+        res = host(t["residual"])
+        np.testing.assert_array_equal(res, r, err_msg=f"residual n={n}")
+        out = host(t["out"])
+        # properties that hold at any size
+        assert set(np.unique(out)).issubset({s, -s})
+        np.testing.assert_array_equal((res + out).astype(F), ((g - out) + out).astype(F))  # r' = v - d with v = g here
+    b.close()
+
+
+def test_terngrad_resnet50_full_set(hp):
+    """configs[2]: bucket 512, heavy-tailed gradients, explicit uniform tensor."""
+    from hipress_amd import workloads as W
+
+    sizes = W.resnet50_sizes()
+    dev = torch.device("cuda:0")
+    grads, unis = W.heavy_tailed_set(sizes, dev, 0), W.uniform_set(sizes, dev, 1000)
+    ts = [{"gradient": g, "uniform": u, "out": torch.empty_like(g),
+           "compressed": torch.full((hp.terngrad_payload_bytes(g.numel(), 512),), 0xAB, dtype=torch.uint8, device="cuda")}
+          for g, u in zip(grads, unis)]
+    b = hp.Batch("terngrad", ts, bucket=512)
+    b.encode()
+    b.decode()
+    for t, n in zip(ts, sizes):
+        g, u = host(t["gradient"]), host(t["uniform"])
+        assert u.max() < 1.0
+        want = oracle.terngrad_encode(g, u, 512)
+        np.testing.assert_array_equal(host(t["compressed"]), want, err_msg=f"n={n}")
+        out = host(t["out"])
+        np.testing.assert_array_equal(out, oracle.terngrad_decode(want, n))
+        # kept elements carry their bucket's scale with the gradient's sign
+        nz = out != 0
+        assert (np.sign(out[nz]) == np.sign(g[nz])).all()
+    b.close()
+
+
+def test_dgc_bert_large_full_set_properties(hp):
+    """configs[3]: DGC 0.1 % with momentum over the 391 BERT-large tensors (335,141,888
+    elements), two steps.  Oracle comparison on the largest and a few other tensors;
+    for all of them the identities that hold at any size."""
+    from hipress_amd import workloads as W
+
+    sizes = W.bert_large_sizes()
+    dev = torch.device("cuda:0")
+    ratio, m = 0.001, 0.9
+    grads = W.normal_set(sizes, dev, 0, sigma=1e-3)
+    ts = [{"gradient": g, "momentum": torch.zeros_like(g), "accumulator": torch.zeros_like(g), "out": torch.empty_like(g),
+           "compressed": torch.zeros(hp.dgc_payload_bytes(g.numel(), ratio), dtype=torch.uint8, device="cuda")}
+          for g in grads]
+    b = hp.Batch("dgc", ts, momentum_factor=m, ratio=ratio)
+    check = {0, 1, 2, 5, 9, 21, len(sizes) - 2}  # word embedding (31M), position embedding, small vectors, 1M/4M matrices
+    ref = {i: (np.zeros(sizes[i], F), np.zeros(sizes[i], F)) for i in check}
+    total_nnz = 0
+    for step in range(2):
+        b.encode()
+        b.decode()
+        total_nnz = 0
+        for i, (t, n) in enumerate(zip(ts, sizes)):
+            pay = host(t["compressed"])
+            nnz, n_hdr, cap, thr, idx, val = oracle.sparse_unpack(pay)
+            total_nnz += nnz
+            assert n_hdr == n and nnz <= cap
+            assert (np.diff(idx) > 0).all(), f"indices not ascending, tensor {i}"
+            assert (np.abs(val) >= thr).all() and (val != 0).all()
+            if i in check:
+                g = host(t["gradient"])
+                want, mom, acc = oracle.dgc_encode(g, ref[i][0], ref[i][1], m, ratio)
+                ref[i] = (mom, acc)
+                w = oracle.sparse_unpack(want)
+                assert (nnz, cap) == (w[0], w[2]) and thr.view(np.uint32) == w[3].view(np.uint32)
+                np.testing.assert_array_equal(idx, w[4])
+                np.testing.assert_array_equal(val, w[5])
+                got_acc, got_mom = host(t["accumulator"]), host(t["momentum"])
+                np.testing.assert_array_equal(got_acc, acc)
+                np.testing.assert_array_equal(got_mom, mom)
+                out = host(t["out"])
+                np.testing.assert_array_equal(out, oracle.sparse_decode(want, n))
+                # sent + kept: selected places are zero in the accumulator and momentum, and nowhere else changed
+                assert not got_acc[idx].any() and not got_mom[idx].any()
+                assert np.count_nonzero(out) == nnz
+        density = total_nnz / sum(sizes)
+        assert 0.0008 < density < 0.0015, density
+    b.close()
+
+
+def test_merge_vgg19_chunks_tbq(hp):
+    """configs[4], TBQ half: 8 peers x 168 chunks of at most 4 MB, decode-and-merge with the
+    fused re-encode; oracle comparison on a sample of chunks, identities on all."""
+    from hipress_amd import workloads as W
+
+    sizes = W.chunk_sizes(W.vgg19_sizes())
+    assert len(sizes) == 168
+    dev = torch.device("cuda:0")
+    tau, P = 0.05, 8
+    chunks = [{"compressed": [torch.zeros(hp.tbq_payload_bytes(n), dtype=torch.uint8, device=dev) for _ in range(P)],
+               "aggregate": torch.empty(n, device=dev), "state": torch.zeros(n, device=dev),
+               "out_compressed": torch.zeros(hp.tbq_payload_bytes(n), dtype=torch.uint8, device=dev)} for n in sizes]
+    for p in range(P):
+        grads = W.normal_set(sizes, dev, p + 1, sigma=0.02)
+        enc = hp.Batch("tbq", [{"gradient": g, "residual": torch.zeros_like(g), "compressed": c["compressed"][p]}
+                               for g, c in zip(grads, chunks)], threshold=tau)
+        enc.encode()
+        torch.cuda.synchronize()
+        enc.close()
+    mb = hp.MergeBatch("tbq", chunks, threshold=tau)
+    mb.run()
+    for i, (c, n) in enumerate(zip(chunks, sizes)):
+        agg = host(c["aggregate"])
+        # every aggregate value is an integer multiple of tau between -8 tau and 8 tau
+        k = np.rint(agg / F(tau))
+        assert np.abs(k).max() <= P
+        np.testing.assert_allclose(agg, k * np.float64(tau), rtol=1e-5, atol=0)
+        if i % 24 == 0 or n < 4096:
+            pays = [host(p) for p in c["compressed"]]
+            want_agg, want_out, want_r = oracle.tbq_decode_merge(pays, n, np.zeros(n, F), tau)
+            np.testing.assert_array_equal(agg, want_agg)
+            np.testing.assert_array_equal(host(c["out_compressed"]), want_out)
+            np.testing.assert_array_equal(host(c["state"]), want_r)
+    mb.close()
+
+
+def test_hip_graph_replay_matches_eager(hp):
+    """encode + decode enqueue only kernels (no allocation, no host synchronisation),
+    so they can be captured in a HIP graph; every replay must equal the eager result."""
+    n = 262144
+    g = torch.randn(n, device="cuda", generator=torch.Generator(device="cuda").manual_seed(0)) * 0.02
+    r = torch.zeros(n, device="cuda")
+    pay = torch.zeros(hp.tbq_payload_bytes(n), dtype=torch.uint8, device="cuda")
+    out = torch.empty(n, device="cuda")
+    # eager reference over three steps (the residual carries)
+    eager = []
+    for _ in range(3):
+        hp.tbq_encode(g, r, pay, 0.05)
+        hp.tbq_decode(pay, out)
+        eager.append((host(pay).copy(), host(r).copy(), host(out).copy()))
+    r.zero_()
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        hp.tbq_encode(g, r, pay, 0.05)  # warm-up on the capture stream
+        hp.tbq_decode(pay, out)
+        stream.synchronize()
+        r.zero_()
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            hp.tbq_encode(g, r, pay, 0.05)
+            hp.tbq_decode(pay, out)
+    for step in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        _ = (out * 2).sum().item()  # unrelated eager work between replays
+        np.testing.assert_array_equal(host(pay), eager[step][0], err_msg=f"payload, replay {step}")
+        np.testing.assert_array_equal(host(r), eager[step][1], err_msg=f"residual, replay {step}")
+        np.testing.assert_array_equal(host(out), eager[step][2], err_msg=f"decode, replay {step}")
