@@ -27,7 +27,18 @@ HBM_PEAK_GBS = 8000.0
 # measured.  (FETCH_SIZE KiB * 2.0 + WRITE_SIZE KiB * 1.0) * 1024, the factors
 # being what the same counters read for a plain 1 GiB copy.
 MEASURED_TRAFFIC = {
-    "onebit_vgg19": int((563473.8 * 2.0 + 579850.1) * 1024),  # onebit_quant_kernel
+    "onebit_vgg19": 1747756544,           # onebit_quant_kernel
+    "onebit_deferred_vgg19": 1748901068,  # onebit_deferred_kernel
+    "tbq_vgg19": 1765703884,              # tbq_encode_kernel
+    "terngrad_vgg19": 1193269862,         # terngrad_encode_kernel
+    "dgc_vgg19": 2896060825,              # sparse_accum_kernel
+    "graddrop_vgg19": 1746493952,         # sparse_accum_kernel
+    "tbq_262144_x512": 1650108825,        # tbq_encode_kernel
+    "terngrad_resnet50": 212457881,       # terngrad_encode_kernel
+    "dgc_bert_large": 6761927884,         # sparse_accum_kernel
+    "graddrop_bert_large": 4080578662,    # sparse_accum_kernel
+    "merge_tbq_vgg19": 2090648268,        # dense_merge_kernel
+    "merge_dgc_vgg19": 1828696576,        # sparse_merge_kernel
 }
 
 
@@ -41,7 +52,8 @@ class SetWorkload:
     """encode+decode of one compressor over a list of tensor sizes through a Batch."""
 
     def __init__(self, name, alg, sizes, data, params, enc_bytes, dec_bytes, dominant_phase, dominant_kernel,
-                 dominant_bytes, rotate=1, nphases=1):
+                 dominant_bytes, rotate=1, nphases=1, graph=False):
+        self.graph = graph  # replay encode+decode from a captured HIP graph (one launch per step)
         self.name, self.alg, self.sizes, self.data, self.params = name, alg, sizes, data, params
         self.enc_bytes, self.dec_bytes = enc_bytes, dec_bytes  # algorithmic bytes per element
         self.dominant_phase, self.dominant_kernel, self.dominant_bytes = dominant_phase, dominant_kernel, dominant_bytes
@@ -97,8 +109,24 @@ class SetWorkload:
             self.tensors.append(ts)
             self.batches.append(hp.Batch(self.alg, ts, **self.params))
         self.k = 0
+        self.captured = None
+        if self.graph:
+            side = torch.cuda.Stream()
+            b = self.batches[0]
+            with torch.cuda.stream(side):
+                b.encode()
+                b.decode()
+                side.synchronize()
+                self.captured = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(self.captured, stream=side):
+                    b.encode()
+                    b.decode()
+            torch.cuda.synchronize()
 
     def step(self, ev=None):
+        if self.captured is not None:
+            self.captured.replay()
+            return
         b = self.batches[self.k % self.rotate]
         self.k += 1
         if ev is None:
@@ -123,6 +151,7 @@ class SetWorkload:
         return nnz / self.elements
 
     def close(self):
+        self.captured = None
         for b in self.batches:
             b.close()
         self.batches, self.tensors = [], []
@@ -176,13 +205,19 @@ class MergeWorkload:
             self.dominant_kernel, self.dominant_bytes = "dense_merge_kernel", self.enc_bytes
         else:
             self.enc_bytes, self.dec_bytes = 12.0, 0.0  # + 8*(P*rho + rho'), added after the run
-            self.dominant_kernel, self.dominant_bytes = "sparse_accum_kernel", 12.0
+            self.dominant_kernel, self.dominant_bytes = "sparse_merge_kernel", 12.0
 
     def step(self, ev=None):
         if ev is not None and self.alg == "tbq":
             ev[0].record()
             self.mb.run()
             ev[1].record()
+        elif ev is not None:
+            self.mb.run_phase(0)
+            ev[0].record()
+            self.mb.run_phase(1)
+            ev[1].record()
+            self.mb.run_phase(2)
         else:
             self.mb.run()
 
@@ -217,6 +252,9 @@ def make_workload(name):
         return SetWorkload(name, "graddrop", vgg, "vgg", {"ratio": 0.01}, 12.0, 4.0, 0, "sparse_accum_kernel", 12.0, nphases=7)
     if name == "tbq_262144":
         return SetWorkload(name, "tbq", [262144], "n0.02", {"threshold": 0.05}, 12.25, 4.25, 0, "tbq_encode_kernel", 12.25)
+    if name == "tbq_262144_graph":
+        return SetWorkload(name, "tbq", [262144], "n0.02", {"threshold": 0.05}, 12.25, 4.25, 0, "tbq_encode_kernel", 12.25,
+                           graph=True)
     if name == "tbq_262144_x512":
         return SetWorkload(name, "tbq", [262144] * 512, "n0.02", {"threshold": 0.05}, 12.25, 4.25, 0, "tbq_encode_kernel", 12.25)
     if name == "terngrad_resnet50":
@@ -332,7 +370,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="onebit_vgg19", choices=ALL_WORKLOADS)
+    ap.add_argument("--workload", default="onebit_vgg19", choices=ALL_WORKLOADS + ["tbq_262144_graph"])
     ap.add_argument("--no-others", action="store_true", help="measure only --workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--others-steps", type=int, default=10)

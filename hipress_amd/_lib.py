@@ -76,6 +76,7 @@ SIGNATURES = {
     "hipress_batch_destroy": (ctypes.c_int, [_vp]),
     "hipress_merge_batch_create": (ctypes.c_int, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(MergeChunk), _i32, _i32, ctypes.POINTER(Params)]),
     "hipress_merge_batch_run": (ctypes.c_int, [_vp, _vp]),
+    "hipress_merge_batch_run_phase": (ctypes.c_int, [_vp, _i32, _vp]),
     "hipress_merge_batch_destroy": (ctypes.c_int, [_vp]),
 }
 

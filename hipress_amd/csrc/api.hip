@@ -638,7 +638,7 @@ int hipress_sparse_decode_merge(const void* const* payloads, const int64_t* payl
     SparseWs ws{};
     if (accumulator) ws = sparse_ws_at(wsb + ibytes, l);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipError_t e = launch_sparse_merge(single_merge_launch(m, npeers, accumulator != nullptr), ws, tileptr, unsorted, st);
+    hipError_t e = launch_sparse_merge(single_merge_launch(m, npeers, accumulator != nullptr), ws, tileptr, unsorted, -1, st);
     if (e != hipSuccess) return HIPRESS_ERR_HIP;
     if (accumulator) e = launch_sparse_encode(single_launch(m.r), false, ws, kSparseAfterAccum, st);
     return hiperr(e);
@@ -871,7 +871,9 @@ int hipress_merge_batch_create(hipress_merge_batch** out, int32_t alg, const hip
     return HIPRESS_OK;
 }
 
-int hipress_merge_batch_run(hipress_merge_batch* b, void* stream) {
+// phase < 0: everything.  Sparse: 0 index, 1 merge (+ accumulate of the re-encode),
+// 2 the remaining re-encode launches.  Dense: 0.
+static int merge_batch_run_impl(hipress_merge_batch* b, int phase, void* stream) {
     if (!b) return HIPRESS_ERR_NULL;
     if (b->segs.empty()) return HIPRESS_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -885,13 +887,15 @@ int hipress_merge_batch_run(hipress_merge_batch* b, void* stream) {
     L.npeers = b->npeers;
     L.reencode = b->reencode;
     if (b->alg == HIPRESS_DGC || b->alg == HIPRESS_GRADDROP) {
+        if (phase > 2) return HIPRESS_ERR_PARAM;
         uint32_t* tileptr = static_cast<uint32_t*>(b->iws);
         uint32_t* unsorted = reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(b->iws) + round_up(4 * b->tp_words, 256));
         SparseWs ws{};
         if (b->reencode) ws = sparse_ws_at(b->ws, b->swl);
-        hipError_t e = launch_sparse_merge(L, ws, tileptr, unsorted, st);
+        hipError_t e = hipSuccess;
+        if (phase < 0 || phase < 2) e = launch_sparse_merge(L, ws, tileptr, unsorted, phase, st);
         if (e != hipSuccess) return HIPRESS_ERR_HIP;
-        if (b->reencode) {
+        if (b->reencode && (phase < 0 || phase == 2)) {
             Launch R;
             std::memset(&R, 0, sizeof R);
             R.single = false;
@@ -905,7 +909,15 @@ int hipress_merge_batch_run(hipress_merge_batch* b, void* stream) {
         }
         return hiperr(e);
     }
+    if (phase > 0) return HIPRESS_ERR_PARAM;
     return hiperr(launch_dense_merge(L, b->alg, st));
+}
+
+int hipress_merge_batch_run(hipress_merge_batch* b, void* stream) { return merge_batch_run_impl(b, -1, stream); }
+
+int hipress_merge_batch_run_phase(hipress_merge_batch* b, int32_t phase, void* stream) {
+    if (phase < 0) return HIPRESS_ERR_PARAM;
+    return merge_batch_run_impl(b, phase, stream);
 }
 
 }  // extern "C"

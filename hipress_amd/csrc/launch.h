@@ -29,6 +29,6 @@ hipError_t launch_sparse_encode(const Launch& L, bool dgc, const SparseWs& ws, i
 hipError_t launch_sparse_decode(const Launch& L, hipStream_t st);
 constexpr int kSparseAfterAccum = 100;  // launch_sparse_encode phase: everything after the accumulate launch
 hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, uint32_t* tileptr, uint32_t* unsorted,
-                               hipStream_t st);
+                               int phase, hipStream_t st);
 
 }  // namespace hp

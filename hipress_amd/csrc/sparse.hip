@@ -813,31 +813,35 @@ hipError_t launch_sparse_decode(const Launch& L, hipStream_t st) {
     return hipGetLastError();
 }
 
-// Index kernel + tile-owner merge.  With L.reencode the merge kernel also runs launch 0
-// of the GradDrop-style re-encode (the caller follows with launch_sparse_encode phases 1..6).
+// Index kernel (phase 0) + tile-owner merge (phase 1); phase < 0 runs both.  With
+// L.reencode the merge kernel also runs launch 0 of the GradDrop-style re-encode
+// (the caller follows with launch_sparse_encode, kSparseAfterAccum).
 hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, uint32_t* tileptr, uint32_t* unsorted,
-                               hipStream_t st) {
+                               int phase, hipStream_t st) {
     if (L.ntiles == 0) return hipSuccess;
+    const bool index = phase < 0 || phase == 0, merge = phase < 0 || phase == 1;
     if (L.single) {
         MergeSingleSegSrc isrc{L.seg};
-        hipLaunchKernelGGL((sparse_merge_index_kernel<MergeSingleSegSrc>), dim3(L.npeers), dim3(kBlock), 0, st, isrc,
-                           tileptr, unsorted, L.npeers);
+        if (index)
+            hipLaunchKernelGGL((sparse_merge_index_kernel<MergeSingleSegSrc>), dim3(L.npeers), dim3(kBlock), 0, st, isrc,
+                               tileptr, unsorted, L.npeers);
         MergeSingleSrc src{L.seg};
-        if (L.reencode)
+        if (merge && L.reencode)
             hipLaunchKernelGGL((sparse_merge_kernel<MergeSingleSrc, true>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
                                tileptr, unsorted, L.npeers);
-        else
+        else if (merge)
             hipLaunchKernelGGL((sparse_merge_kernel<MergeSingleSrc, false>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
                                tileptr, unsorted, L.npeers);
     } else {
         MergeBatchSegSrc isrc{L.dsegs};
-        hipLaunchKernelGGL((sparse_merge_index_kernel<MergeBatchSegSrc>), dim3(L.nsegs * L.npeers), dim3(kBlock), 0, st,
-                           isrc, tileptr, unsorted, L.npeers);
+        if (index)
+            hipLaunchKernelGGL((sparse_merge_index_kernel<MergeBatchSegSrc>), dim3(L.nsegs * L.npeers), dim3(kBlock), 0,
+                               st, isrc, tileptr, unsorted, L.npeers);
         MergeBatchSrc src{L.dsegs, L.dmap};
-        if (L.reencode)
+        if (merge && L.reencode)
             hipLaunchKernelGGL((sparse_merge_kernel<MergeBatchSrc, true>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
                                tileptr, unsorted, L.npeers);
-        else
+        else if (merge)
             hipLaunchKernelGGL((sparse_merge_kernel<MergeBatchSrc, false>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
                                tileptr, unsorted, L.npeers);
     }

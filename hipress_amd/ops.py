@@ -406,6 +406,12 @@ class MergeBatch:
         with torch.cuda.device(self.device):
             check(_lib.lib().hipress_merge_batch_run(self._h, torch.cuda.current_stream(self.device).cuda_stream), "merge_batch_run")
 
+    def run_phase(self, phase):
+        """One part of the launch sequence (measurement aid)."""
+        with torch.cuda.device(self.device):
+            check(_lib.lib().hipress_merge_batch_run_phase(self._h, int(phase), torch.cuda.current_stream(self.device).cuda_stream),
+                  "merge_batch_run_phase")
+
     def close(self):
         if getattr(self, "_h", None):
             _lib.lib().hipress_merge_batch_destroy(self._h)

@@ -214,6 +214,11 @@ int hipress_merge_batch_create(hipress_merge_batch **out, int32_t alg,
                                const hipress_merge_chunk *chunks, int32_t count, int32_t npeers,
                                const hipress_params *params);
 int hipress_merge_batch_run(hipress_merge_batch *batch, void *stream);
+/* Measurement aid, like hipress_batch_encode_phase.  dgc / graddrop: 0 tile index of
+ * the peers' payloads, 1 merge (with the first launch of the re-encode fused in),
+ * 2 the remaining launches of the re-encode; onebit, tbq, terngrad: 0.  No
+ * counterpart in the reference. */
+int hipress_merge_batch_run_phase(hipress_merge_batch *batch, int32_t phase, void *stream);
 int hipress_merge_batch_destroy(hipress_merge_batch *batch);
 
 #ifdef __cplusplus
