@@ -80,7 +80,7 @@ __device__ __forceinline__ void tbq_encode_tile(const Seg& s, unsigned tile) {
 template <class Src>
 __global__ __launch_bounds__(kBlock) void tbq_encode_kernel(Src src) {
     unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, blockIdx.x);
     if (tile == 0 && threadIdx.x == 0) {
         uint32_t* h = reinterpret_cast<uint32_t*>(s.pay);
         h[0] = __float_as_uint(s.f0);
@@ -130,7 +130,7 @@ __device__ __forceinline__ void tbq_decode_tile(const Seg& s, unsigned tile) {
 template <class Src>
 __global__ __launch_bounds__(kBlock) void tbq_decode_kernel(Src src) {
     unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, blockIdx.x);
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) tbq_decode_tile<true>(s, tile);
     else tbq_decode_tile<false>(s, tile);
 }
@@ -166,7 +166,7 @@ template <class Src>
 __global__ __launch_bounds__(kBlock) void onebit_abs_kernel(Src src, float* partial) {
     __shared__ float wsum[4];
     unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, blockIdx.x);
     float a;
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) a = onebit_abs_tile<true>(s, tile);
     else a = onebit_abs_tile<false>(s, tile);
@@ -190,7 +190,7 @@ __device__ __forceinline__ double wave_sum_d(double x) {
 template <class Src>
 __global__ __launch_bounds__(kScaleBlock) void onebit_scale_kernel(Src src, const float* partial) {
     __shared__ double red[kScaleBlock / 64];
-    const Seg& s = src.at(blockIdx.x);
+    const Seg s = src.at(blockIdx.x);
     const float* p = partial + s.tile0;
     const unsigned nt = s.ntiles;
     double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
@@ -260,7 +260,7 @@ __device__ __forceinline__ void onebit_quant_tile(const Seg& s, unsigned tile) {
 template <class Src>
 __global__ __launch_bounds__(kBlock) void onebit_quant_kernel(Src src) {
     unsigned tile;
-    const Seg& s = src.get(tile, gridDim.x - 1 - blockIdx.x);
+    const Seg s = src.get(tile, gridDim.x - 1 - blockIdx.x);
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) onebit_quant_tile<true>(s, tile);
     else onebit_quant_tile<false>(s, tile);
 }
@@ -320,7 +320,7 @@ template <class Src>
 __global__ __launch_bounds__(kBlock) void onebit_deferred_kernel(Src src, float* partial) {
     __shared__ float wsum[4];
     unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, blockIdx.x);
     const float sp = *s.s1;  // last step's scale (0 before the first step)
     float a;
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) a = onebit_deferred_tile<true>(s, tile, sp);
@@ -335,7 +335,7 @@ __global__ __launch_bounds__(kBlock) void onebit_deferred_kernel(Src src, float*
 template <class Src>
 __global__ __launch_bounds__(kBlock) void onebit_materialize_kernel(Src src) {
     unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, blockIdx.x);
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long n = (long long)s.n;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
@@ -382,7 +382,7 @@ __device__ __forceinline__ void onebit_decode_tile(const Seg& s, unsigned tile) 
 template <class Src>
 __global__ __launch_bounds__(kBlock) void onebit_decode_kernel(Src src) {
     unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, blockIdx.x);
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) onebit_decode_tile<true>(s, tile);
     else onebit_decode_tile<false>(s, tile);
 }
@@ -459,7 +459,7 @@ __device__ __forceinline__ void terngrad_zero_scale_pad(const Seg& s, unsigned t
 template <class Src, int BPW>
 __global__ __launch_bounds__(kBlock) void terngrad_encode_kernel(Src src) {
     unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, blockIdx.x);
     if (tile == 0 && threadIdx.x == 0) {
         uint32_t* h = reinterpret_cast<uint32_t*>(s.pay);
         h[0] = (uint32_t)s.n;
@@ -477,7 +477,7 @@ template <class Src>
 __global__ __launch_bounds__(kBlock) void terngrad_scale_generic_kernel(Src src) {
     // grid: tiles of the tensor; each workgroup walks the buckets that START in its tile
     unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, blockIdx.x);
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long n = (long long)s.n, B = s.bucket;
     const long long lo = (long long)tile * kTile, hi = lo + kTile < n ? lo + kTile : n;
@@ -504,7 +504,7 @@ __global__ __launch_bounds__(kBlock) void terngrad_scale_generic_kernel(Src src)
 template <class Src>
 __global__ __launch_bounds__(kBlock) void terngrad_quant_generic_kernel(Src src) {
     unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, blockIdx.x);
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long n = (long long)s.n, B = s.bucket;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
@@ -581,7 +581,7 @@ __device__ __forceinline__ const uint32_t* terngrad_words(const uint8_t* pay, un
 template <class Src>
 __global__ __launch_bounds__(kBlock) void terngrad_decode_kernel(Src src) {
     unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, blockIdx.x);
     long long B;
     const uint32_t* words = terngrad_words(s.pay, s.pay_bytes, s.n, B);
     const bool fast = s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n;

@@ -30,7 +30,7 @@ __device__ __forceinline__ unsigned tbq_q(float v, float tau, float& keep) {
 template <bool FAST, int ALG, bool REENC>
 __device__ __forceinline__ void merge_tile(const MergeSeg& m, unsigned tile, int npeers) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const Seg& s = m.s;
+    const Seg s = m.s;
     const long long n = (long long)s.n;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
     f4 agg[4];

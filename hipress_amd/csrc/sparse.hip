@@ -135,7 +135,7 @@ __device__ __forceinline__ void sparse_reset_select(const Seg& s, const SparseWs
 template <class Src, bool DGC>
 __global__ __launch_bounds__(kBlock) void sparse_accum_kernel(Src src, SparseWs ws) {
     unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, blockIdx.x);
     if (tile == 0) sparse_reset_select(s, ws);
     const long long n = (long long)s.n;
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n)
@@ -155,7 +155,7 @@ __global__ __launch_bounds__(kBlock) void sparse_select_kernel(Src src, SparseWs
     __shared__ unsigned chunk[kBlock];
     __shared__ unsigned is_last;
     unsigned stile;
-    const Seg& s = src.get(stile, blockIdx.x);
+    const Seg s = src.get(stile, blockIdx.x);
     const uint32_t* keys = ws.sample + s.ws0;
     uint32_t* ctl = ws.ctl + s.id * kCtlWords;
     uint32_t* gh = ws.hist + ((unsigned long long)s.id * 3 + pass) * kBins;
@@ -285,7 +285,7 @@ __global__ __launch_bounds__(kBlock) void sparse_count_kernel(Src src, SparseWs 
     const unsigned gt_idx = blockIdx.x * 4 + wave;
     if (gt_idx >= total_tiles) return;
     unsigned tile;
-    const Seg& s = src.get(tile, gt_idx);
+    const Seg s = src.get(tile, gt_idx);
     const unsigned thr = ws.thr[2 * s.id];
     unsigned gt, eq;
     count_tile(s, ws, tile, thr, lane, gt, eq);
@@ -410,7 +410,7 @@ template <class SegSrc>
 __global__ __launch_bounds__(kScanBlock) void sparse_scan_kernel(SegSrc src, SparseWs ws) {
     __shared__ unsigned sh[2][kScanWaves];
     __shared__ RadixScratch sc;
-    const Seg& s = src.at(blockIdx.x);
+    const Seg s = src.at(blockIdx.x);
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const unsigned nw = s.ntiles;
     uint32_t* c = ws.counts + (unsigned long long)s.tile0 * 2;
@@ -479,7 +479,7 @@ __global__ __launch_bounds__(kBlock) void sparse_emit_kernel(Src src, SparseWs w
     const unsigned gt_idx = blockIdx.x * 4 + wave;
     if (gt_idx >= total_tiles) return;
     unsigned tile;
-    const Seg& s = src.get(tile, gt_idx);
+    const Seg s = src.get(tile, gt_idx);
     const long long n = (long long)s.n;
     const unsigned thr = ws.thr[2 * s.id], quota = ws.thr[2 * s.id + 1];
     const unsigned long long ci = (unsigned long long)(s.tile0 + tile) * 2;
@@ -594,7 +594,7 @@ __device__ __forceinline__ void zero_tile(float* out, long long n, unsigned tile
 template <class Src>
 __global__ __launch_bounds__(kBlock) void zero_fill_kernel(Src src) {
     unsigned tile;
-    const Seg& s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, blockIdx.x);
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) zero_tile<true>(s.out, (long long)s.n, tile);
     else zero_tile<false>(s.out, (long long)s.n, tile);
 }
@@ -617,7 +617,7 @@ constexpr int kSlotTile = 1024;
 template <class Src>
 __global__ __launch_bounds__(kBlock) void sparse_scatter_kernel(Src src) {
     unsigned ct;
-    const Seg& s = src.get(ct, blockIdx.x);
+    const Seg s = src.get(ct, blockIdx.x);
     const int32_t* idx;
     const float* val;
     const unsigned nnz = sparse_header(s.pay, s.cap, idx, val);
@@ -682,8 +682,8 @@ __global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs
     __shared__ unsigned plo[kMaxPeers], pcnt[kMaxPeers], pcap[kMaxPeers];
     unsigned tile;
     const MergeSeg& m = src.get(tile, blockIdx.x);
-    const Seg& s = m.s;
-    const Seg& r = m.r;  // re-encode descriptor of this chunk: same tile numbering
+    const Seg s = m.s;
+    const Seg r = m.r;  // re-encode descriptor of this chunk: same tile numbering
     const long long n = (long long)s.n;
     const long long t_lo = (long long)tile * kTile, t_hi = t_lo + kTile < n ? t_lo + kTile : n;
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
