@@ -9,7 +9,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libhipress_amd.so")
-SOURCES = ["api.hip", "dense.hip", "sparse.hip", "merge.hip"]
+SOURCES = ["api.hip", "dense.hip", "sparse.hip", "merge.hip", "compll.hip"]
 FLAGS = [
     "--offload-arch=gfx950",
     "-O3",

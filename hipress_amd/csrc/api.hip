@@ -479,6 +479,56 @@ int hipress_terngrad_decode(const void* payload, int64_t payload_bytes, float* o
     return hiperr(launch_terngrad_decode(single_launch(s), static_cast<hipStream_t>(stream)));
 }
 
+// ---- the in-tree CompLL operator -------------------------------------------------------
+
+int64_t hipress_compll_payload_bytes(int64_t n, int32_t bitwidth) {
+    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (bitwidth != 1 && bitwidth != 2 && bitwidth != 4 && bitwidth != 8) return HIPRESS_ERR_PARAM;
+    return 10 + (n * bitwidth + 7) / 8;
+}
+
+int64_t hipress_compll_workspace_bytes(int64_t n) {
+    return bad_n(n) ? HIPRESS_ERR_SIZE : round_up(8 * (int64_t)tiles_of(n), 256);
+}
+
+int hipress_compll_encode(const float* grad, const float* uniform, int64_t n, void* compressed,
+                          int64_t compressed_bytes, int32_t bitwidth, void* workspace, int64_t workspace_bytes,
+                          void* stream) {
+    int64_t need = hipress_compll_payload_bytes(n, bitwidth);
+    if (need < 0) return (int)need;
+    if (!compressed || (n > 0 && (!grad || !uniform))) return HIPRESS_ERR_NULL;
+    if (mis(grad, 4) || mis(uniform, 4)) return HIPRESS_ERR_ALIGN;
+    if (compressed_bytes < need) return HIPRESS_ERR_SIZE;
+    if (!workspace || workspace_bytes < hipress_compll_workspace_bytes(n)) return HIPRESS_ERR_WORKSPACE;
+    if (mis(workspace, 16)) return HIPRESS_ERR_ALIGN;
+    Seg s;
+    std::memset(&s, 0, sizeof s);
+    s.g = grad;
+    s.u = uniform;
+    s.pay = static_cast<uint8_t*>(compressed);
+    s.n = (unsigned long long)n;
+    s.ntiles = tiles_of(n);
+    s.aligned = al16(grad) && al16(uniform);
+    s.bucket = (unsigned)bitwidth;
+    return hiperr(launch_compll_encode(single_launch(s), bitwidth, static_cast<float*>(workspace),
+                                       static_cast<hipStream_t>(stream)));
+}
+
+int hipress_compll_decode(const void* compressed, int64_t compressed_bytes, float* out, int64_t n, void* stream) {
+    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (!compressed || (n > 0 && !out)) return HIPRESS_ERR_NULL;
+    if (mis(out, 4)) return HIPRESS_ERR_ALIGN;
+    if (compressed_bytes < 10) return HIPRESS_ERR_SIZE;
+    Seg s;
+    std::memset(&s, 0, sizeof s);
+    s.pay = const_cast<uint8_t*>(static_cast<const uint8_t*>(compressed));
+    s.pay_bytes = (unsigned long long)compressed_bytes;
+    s.out = out;
+    s.n = (unsigned long long)n;
+    s.ntiles = tiles_of(n);
+    return hiperr(launch_compll_decode(single_launch(s), static_cast<hipStream_t>(stream)));
+}
+
 // ---- DGC / GradDrop ------------------------------------------------------------------
 
 static int sparse_encode_single(int alg, const hipress_tensor& t, const hipress_params& pr, void* workspace,

@@ -1,0 +1,205 @@
+// The in-tree CompLL operator (min/max b-bit stochastic quantiser, 10-byte header)
+// for gfx950, as its DSL source states it
+// (/root/reference/src/CompLL/GCGen/pse/TernGradEncode.pse:22-33,
+//  /root/reference/src/CompLL/GCGen/pse/TernGradDecode.pse:1-14):
+//   encode: max/min reduction, gap = (max-min)/(2^b-1), code_i = floor((g_i-min)/gap + u_i),
+//           payload [b:u8][tail:u8][min:f32][max:f32] then codes, code i at bit
+//           (i mod 8/b)*b of byte floor(i*b/8) - the placement the decoder reads
+//           (TernGradDecode_body.h:44);
+//   decode: count = (8*csz - 80)/b - tail elements, out_i = code_i*gap + min
+//           (TernGradDecode_body.h:65-72).
+// Three launches for encode (per-tile min/max, per-tensor header, quantise), one
+// for decode; same tile / wavefront / lane decomposition as the other operators.
+#include "common.h"
+#include "launch.h"
+
+namespace hp {
+
+constexpr float kMaxInit = -99999.0f, kMinInit = 99999.0f;  // the DSL's reduce() initial values
+
+__device__ __forceinline__ float load_f32_bytes(const uint8_t* p) {
+    return __uint_as_float((unsigned)p[0] | ((unsigned)p[1] << 8) | ((unsigned)p[2] << 16) | ((unsigned)p[3] << 24));
+}
+__device__ __forceinline__ void store_f32_bytes(uint8_t* p, float x) {
+    unsigned u = __float_as_uint(x);
+    p[0] = (uint8_t)u;
+    p[1] = (uint8_t)(u >> 8);
+    p[2] = (uint8_t)(u >> 16);
+    p[3] = (uint8_t)(u >> 24);
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void compll_minmax_kernel(Src src, float* partial) {
+    __shared__ float wmx[4], wmn[4];
+    unsigned tile;
+    const Seg s = src.get(tile, blockIdx.x);
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    const bool fast = s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n;
+    float mx = kMaxInit, mn = kMinInit;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        f4 v = fast ? ld4(s.g + e) : ld4_guard(s.g, e, n);
+        unsigned ok = fast ? 0xfu : valid4(e, n);
+        if (ok & 1u) { mx = v.x > mx ? v.x : mx; mn = v.x < mn ? v.x : mn; }
+        if (ok & 2u) { mx = v.y > mx ? v.y : mx; mn = v.y < mn ? v.y : mn; }
+        if (ok & 4u) { mx = v.z > mx ? v.z : mx; mn = v.z < mn ? v.z : mn; }
+        if (ok & 8u) { mx = v.w > mx ? v.w : mx; mn = v.w < mn ? v.w : mn; }
+    }
+    mx = wave_max(mx);
+    mn = -wave_max(-mn);
+    if (lane == 0) {
+        wmx[wave] = mx;
+        wmn[wave] = mn;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        partial[2 * (s.tile0 + tile)] = fmaxf(fmaxf(wmx[0], wmx[1]), fmaxf(wmx[2], wmx[3]));
+        partial[2 * (s.tile0 + tile) + 1] = fminf(fminf(wmn[0], wmn[1]), fminf(wmn[2], wmn[3]));
+    }
+}
+
+template <class SegSrc>
+__global__ __launch_bounds__(kBlock) void compll_header_kernel(SegSrc src, const float* partial) {
+    __shared__ float smx[kBlock], smn[kBlock];
+    const Seg s = src.at(blockIdx.x);
+    float mx = kMaxInit, mn = kMinInit;
+    for (unsigned t = threadIdx.x; t < s.ntiles; t += kBlock) {
+        mx = fmaxf(mx, partial[2 * (s.tile0 + t)]);
+        mn = fminf(mn, partial[2 * (s.tile0 + t) + 1]);
+    }
+    smx[threadIdx.x] = mx;
+    smn[threadIdx.x] = mn;
+    __syncthreads();
+    for (int w = kBlock / 2; w >= 1; w >>= 1) {
+        if ((int)threadIdx.x < w) {
+            smx[threadIdx.x] = fmaxf(smx[threadIdx.x], smx[threadIdx.x + w]);
+            smn[threadIdx.x] = fminf(smn[threadIdx.x], smn[threadIdx.x + w]);
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const unsigned b = s.bucket;  // bit width
+        s.pay[0] = (uint8_t)b;
+        s.pay[1] = (uint8_t)(s.n % (1ull << b));  // the DSL's tail = size % (1 << bitwidth)
+        store_f32_bytes(s.pay + 2, smn[0]);
+        store_f32_bytes(s.pay + 6, smx[0]);
+    }
+}
+
+__device__ __forceinline__ unsigned compll_code(float g, float u, float mn, float gap, float top) {
+    if (!(gap > 0.f)) return 0u;
+    float f = floorf((g - mn) / gap + u);
+    return f <= 0.f ? 0u : (f >= top ? (unsigned)top : (unsigned)f);
+}
+
+template <class Src, int B>
+__global__ __launch_bounds__(kBlock) void compll_quant_kernel(Src src) {
+    unsigned tile;
+    const Seg s = src.get(tile, blockIdx.x);
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    const bool fast = s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n;
+    const float mn = load_f32_bytes(s.pay + 2), mx = load_f32_bytes(s.pay + 6);
+    constexpr float top = (float)((1 << B) - 1);
+    const float gap = (mx - mn) / top;
+    uint8_t* Q = s.pay + 10;
+    const long long nbytes = (n * B + 7) / 8;
+    f4 g[4], u[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        g[j] = fast ? ld4(s.g + e) : ld4_guard(s.g, e, n);
+        u[j] = fast ? ld4(s.u + e) : ld4_guard(s.u, e, n);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        unsigned ok = fast ? 0xfu : valid4(e, n);
+        unsigned c0 = (ok & 1u) ? compll_code(g[j].x, u[j].x, mn, gap, top) : 0u;
+        unsigned c1 = (ok & 2u) ? compll_code(g[j].y, u[j].y, mn, gap, top) : 0u;
+        unsigned c2 = (ok & 4u) ? compll_code(g[j].z, u[j].z, mn, gap, top) : 0u;
+        unsigned c3 = (ok & 8u) ? compll_code(g[j].w, u[j].w, mn, gap, top) : 0u;
+        if (B == 8) {
+            if (ok & 1u) Q[e] = (uint8_t)c0;
+            if (ok & 2u) Q[e + 1] = (uint8_t)c1;
+            if (ok & 4u) Q[e + 2] = (uint8_t)c2;
+            if (ok & 8u) Q[e + 3] = (uint8_t)c3;
+        } else if (B == 4) {
+            if (ok & 1u) Q[e / 2] = (uint8_t)(c0 | (c1 << 4));
+            if (ok & 4u) Q[e / 2 + 1] = (uint8_t)(c2 | (c3 << 4));
+        } else if (B == 2) {
+            if (ok & 1u) Q[e / 4] = (uint8_t)(c0 | (c1 << 2) | (c2 << 4) | (c3 << 6));
+        } else {  // B == 1: two neighbouring lanes share a byte
+            unsigned nib = c0 | (c1 << 1) | (c2 << 2) | (c3 << 3);
+            unsigned other = (unsigned)__builtin_amdgcn_update_dpp(0, (int)nib, 0xB1, 0xf, 0xf, false);  // quad_perm [1,0,3,2]
+            if ((lane & 1u) == 0 && e / 8 < nbytes && (ok & 1u)) Q[e / 8] = (uint8_t)(nib | (other << 4));
+        }
+    }
+}
+
+// Decode follows the reference literally: the element count comes from the payload
+// length and the tail byte; at most n (the caller's buffer) elements are written.
+template <class Src>
+__global__ __launch_bounds__(kBlock) void compll_decode_kernel(Src src) {
+    unsigned tile;
+    const Seg s = src.get(tile, blockIdx.x);
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned b = s.pay[0], tail = s.pay[1];
+    if (b != 1 && b != 2 && b != 4 && b != 8) return;
+    const float mn = load_f32_bytes(s.pay + 2), mx = load_f32_bytes(s.pay + 6);
+    const float gap = (mx - mn) / (float)((1u << b) - 1u);
+    long long count = (8 * (long long)s.pay_bytes - 80) / (long long)b - (long long)tail;
+    if (count > (long long)s.n) count = (long long)s.n;
+    const uint8_t* Q = s.pay + 10;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    const unsigned per = 8 / b, mask = (1u << b) - 1u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            long long i = e + k;
+            if (i < count) {
+                unsigned code = (Q[i * b / 8] >> ((unsigned)(i % per) * b)) & mask;
+                s.out[i] = __fadd_rn(__fmul_rn((float)code, gap), mn);
+            }
+        }
+    }
+}
+
+template <class Src, class SegSrcT>
+static hipError_t compll_encode_src(const Src& src, const SegSrcT& ssrc, unsigned ntiles, unsigned nsegs, int b,
+                                    float* partial, hipStream_t st) {
+    hipLaunchKernelGGL((compll_minmax_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src, partial);
+    hipLaunchKernelGGL((compll_header_kernel<SegSrcT>), dim3(nsegs), dim3(kBlock), 0, st, ssrc, partial);
+    if (b == 1) hipLaunchKernelGGL((compll_quant_kernel<Src, 1>), dim3(ntiles), dim3(kBlock), 0, st, src);
+    else if (b == 2) hipLaunchKernelGGL((compll_quant_kernel<Src, 2>), dim3(ntiles), dim3(kBlock), 0, st, src);
+    else if (b == 4) hipLaunchKernelGGL((compll_quant_kernel<Src, 4>), dim3(ntiles), dim3(kBlock), 0, st, src);
+    else hipLaunchKernelGGL((compll_quant_kernel<Src, 8>), dim3(ntiles), dim3(kBlock), 0, st, src);
+    return hipGetLastError();
+}
+
+// partial: two floats per tile
+hipError_t launch_compll_encode(const Launch& L, int bitwidth, float* partial, hipStream_t st) {
+    if (L.ntiles == 0) return hipSuccess;
+    if (L.single) return compll_encode_src(SingleSrc{L.seg}, SingleSegSrc{L.seg}, L.ntiles, 1, bitwidth, partial, st);
+    return compll_encode_src(BatchSrc{L.dsegs, L.dmap}, BatchSegSrc{L.dsegs}, L.ntiles, L.nsegs, bitwidth, partial, st);
+}
+
+hipError_t launch_compll_decode(const Launch& L, hipStream_t st) {
+    if (L.ntiles == 0) return hipSuccess;
+    if (L.single) {
+        SingleSrc src{L.seg};
+        hipLaunchKernelGGL((compll_decode_kernel<SingleSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
+    } else {
+        BatchSrc src{L.dsegs, L.dmap};
+        hipLaunchKernelGGL((compll_decode_kernel<BatchSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace hp

@@ -13,6 +13,10 @@ hipError_t launch_onebit_materialize(const Launch& L, hipStream_t st);
 hipError_t launch_terngrad_encode(const Launch& L, unsigned bucket, hipStream_t st);
 hipError_t launch_terngrad_decode(const Launch& L, hipStream_t st);
 
+// The in-tree CompLL operator (10-byte header, b-bit min/max quantiser).
+hipError_t launch_compll_encode(const Launch& L, int bitwidth, float* partial, hipStream_t st);
+hipError_t launch_compll_decode(const Launch& L, hipStream_t st);
+
 // Dense decode-and-merge; alg is a hipress_alg value (onebit, tbq, terngrad).
 hipError_t launch_dense_merge(const MergeLaunch& L, int alg, hipStream_t st);
 

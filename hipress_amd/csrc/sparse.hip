@@ -247,32 +247,47 @@ __device__ __forceinline__ unsigned pick_row(unsigned row, unsigned a, unsigned 
 
 // Counts, for tile `tile` (4096 elements) of tensor s, the keys above and equal
 // to thr; lane l looks at the maximum of 64-element group l and only groups
-// whose maximum reaches thr are read (eight at a time).  Wavefront-uniform result.
+// whose maximum reaches thr are read, eight per round, the next round's loads in
+// flight while this round is counted.  Wavefront-uniform result.
 __device__ __forceinline__ void count_tile(const Seg& s, const SparseWs& ws, unsigned tile, unsigned thr,
                                            unsigned lane, unsigned& gt, unsigned& eq) {
     const long long n = (long long)s.n;
     const bool aligned = s.aligned != 0;
+    const float* acc = s.s1;
     unsigned gm = ws.gmax[(unsigned long long)(s.tile0 + tile) * 64 + lane];
     unsigned long long mask = __ballot(gm >= thr && gm > 0u);
     const unsigned row = lane >> 4;
     const long long base = (long long)tile * kTile + (lane & 15u) * 4;
+    const f4 zero4 = {0.f, 0.f, 0.f, 0.f};
     unsigned cg = 0, ce = 0;
-    while (mask) {
+    auto fetch = [&](f4& va, f4& vb) {
         unsigned a0 = pop_bit(mask), a1 = pop_bit(mask), a2 = pop_bit(mask), a3 = pop_bit(mask);
         unsigned b0 = pop_bit(mask), b1 = pop_bit(mask), b2 = pop_bit(mask), b3 = pop_bit(mask);
         unsigned ga = pick_row(row, a0, a1, a2, a3), gb = pick_row(row, b0, b1, b2, b3);
-        f4 va = {0.f, 0.f, 0.f, 0.f}, vb = {0.f, 0.f, 0.f, 0.f};
-        if (ga < 64u) va = load_group4(s.s1, base + ga * 64, n, aligned);
-        if (gb < 64u) vb = load_group4(s.s1, base + gb * 64, n, aligned);
+        va = zero4;
+        vb = zero4;
+        if (ga < 64u) va = load_group4(acc, base + ga * 64, n, aligned);
+        if (gb < 64u) vb = load_group4(acc, base + gb * 64, n, aligned);
+    };
+    auto tally = [&](f4 v) {
         unsigned k;
-        k = key_of(va.x); cg += k > thr; ce += (k == thr) & (k > 0u);
-        k = key_of(va.y); cg += k > thr; ce += (k == thr) & (k > 0u);
-        k = key_of(va.z); cg += k > thr; ce += (k == thr) & (k > 0u);
-        k = key_of(va.w); cg += k > thr; ce += (k == thr) & (k > 0u);
-        k = key_of(vb.x); cg += k > thr; ce += (k == thr) & (k > 0u);
-        k = key_of(vb.y); cg += k > thr; ce += (k == thr) & (k > 0u);
-        k = key_of(vb.z); cg += k > thr; ce += (k == thr) & (k > 0u);
-        k = key_of(vb.w); cg += k > thr; ce += (k == thr) & (k > 0u);
+        k = key_of(v.x); cg += k > thr; ce += (k == thr) & (k > 0u);
+        k = key_of(v.y); cg += k > thr; ce += (k == thr) & (k > 0u);
+        k = key_of(v.z); cg += k > thr; ce += (k == thr) & (k > 0u);
+        k = key_of(v.w); cg += k > thr; ce += (k == thr) & (k > 0u);
+    };
+    f4 va, vb;
+    bool have = mask != 0;
+    if (have) fetch(va, vb);
+    while (have) {
+        f4 na = zero4, nb = zero4;
+        const bool more = mask != 0;
+        if (more) fetch(na, nb);
+        tally(va);
+        tally(vb);
+        va = na;
+        vb = nb;
+        have = more;
     }
     gt = wave_sum_u(cg);
     eq = wave_sum_u(ce);

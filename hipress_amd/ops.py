@@ -28,6 +28,7 @@ __all__ = [
     "sparse_payload_bytes", "dgc_payload_bytes", "graddrop_payload_bytes",
     "onebit_encode", "onebit_decode", "onebit_encode_deferred", "onebit_residual", "tbq_encode", "tbq_decode", "terngrad_encode", "terngrad_decode",
     "dgc_encode", "dgc_decode", "graddrop_encode", "graddrop_decode",
+    "compll_payload_bytes", "compll_terngrad_encode", "compll_terngrad_decode",
     "onebit_decode_merge", "tbq_decode_merge", "terngrad_decode_merge", "dgc_decode_merge",
     "graddrop_decode_merge", "Batch", "MergeBatch", "ALIASES",
 ]
@@ -193,6 +194,32 @@ def terngrad_decode(compressed, gradient):
     with torch.cuda.device(gradient.device):
         check(_lib.lib().hipress_terngrad_decode(_p(compressed), compressed.numel(), _p(gradient), gradient.numel(),
                                                  _stream(gradient)), "terngrad_decode")
+
+
+# ---------------------------------------------------------------- the in-tree CompLL operator
+def compll_payload_bytes(n, bitwidth=2):
+    return size(_lib.lib().hipress_compll_payload_bytes(n, int(bitwidth)), "compll_payload_bytes")
+
+
+def compll_terngrad_encode(gradient, uniform, compressed, bitwidth=2):
+    """The operator CompLL generates from pse/TernGradEncode.pse: min/max `bitwidth`-bit
+    stochastic quantiser with the 10-byte header; `uniform` replaces random<float>(0,1)."""
+    _f32(gradient, "gradient"); _f32(uniform, "uniform", gradient); _u8(compressed, "compressed", gradient)
+    _same_numel(gradient, uniform, "gradient", "uniform")
+    L = _lib.lib()
+    n = gradient.numel()
+    with torch.cuda.device(gradient.device):
+        ws = _workspace(gradient, size(L.hipress_compll_workspace_bytes(n), "compll_workspace_bytes"))
+        check(L.hipress_compll_encode(_p(gradient), _p(uniform), n, _p(compressed), compressed.numel(), int(bitwidth),
+                                      _p(ws), ws.numel(), _stream(gradient)), "compll_encode")
+
+
+def compll_terngrad_decode(compressed, gradient):
+    """Decode of that format; the element count comes from the payload length and its tail byte."""
+    _u8(compressed, "compressed"); _f32(gradient, "gradient", compressed)
+    with torch.cuda.device(gradient.device):
+        check(_lib.lib().hipress_compll_decode(_p(compressed), compressed.numel(), _p(gradient), gradient.numel(),
+                                               _stream(gradient)), "compll_decode")
 
 
 # ---------------------------------------------------------------- DGC / GradDrop
@@ -445,6 +472,8 @@ _SCHEMAS = {
     "dgc_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
     "graddrop_encode": "(Tensor gradient, Tensor(a!) accumulator, Tensor(b!) compressed, float ratio=0.01) -> ()",
     "graddrop_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
+    "compll_terngrad_encode": "(Tensor gradient, Tensor uniform, Tensor(a!) compressed, int bitwidth=2) -> ()",
+    "compll_terngrad_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
     "onebit_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate) -> ()",
     "terngrad_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate) -> ()",
     "tbq_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate, Tensor(b!)? residual=None, "

@@ -124,6 +124,24 @@ int hipress_terngrad_encode(const float *grad, const float *uniform, int64_t n, 
 int hipress_terngrad_decode(const void *payload, int64_t payload_bytes, float *out, int64_t n,
                             void *stream);
 
+/* ---- the in-tree CompLL operator, in its own wire format ---------------------- */
+/* Replaces TernGradEncode_body / TernGradDecode_body as generated in the tree
+ * (/root/reference/src/CompLL/GCGen/output/TernGradEncode/TernGradEncode_body.h:99-126,
+ *  /root/reference/src/CompLL/GCGen/output/TernGradDecode/TernGradDecode_body.h:48-74),
+ * with the semantics of their DSL sources (pse/TernGradEncode.pse:22-33): payload
+ * [bitwidth:u8][tail:u8][min:f32][max:f32] then b-bit codes, code i at bit
+ * (i mod 8/b)*b of byte floor(i*b/8); bitwidth in {1,2,4,8}; no alignment is
+ * required of `compressed`.  The rounding noise is an explicit uniform[0,1)
+ * tensor.  Decode writes (8*compressed_bytes - 80)/b - tail elements, as the
+ * reference does, but never more than n. */
+int64_t hipress_compll_payload_bytes(int64_t n, int32_t bitwidth);
+int64_t hipress_compll_workspace_bytes(int64_t n);
+int hipress_compll_encode(const float *grad, const float *uniform, int64_t n, void *compressed,
+                          int64_t compressed_bytes, int32_t bitwidth, void *workspace,
+                          int64_t workspace_bytes, void *stream);
+int hipress_compll_decode(const void *compressed, int64_t compressed_bytes, float *out, int64_t n,
+                          void *stream);
+
 /* ---- DGC / GradDrop: sampled-threshold sparsification ---------------------- */
 /* Replace <Func>_body for "dgc" and "graddrop" (/root/reference/README.md:9,162).
  * ratio is the kept fraction (DGC 0.001; GradDrop drop ratio 0.99 = 0.01). */

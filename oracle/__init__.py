@@ -70,6 +70,9 @@ def lib():
             "hpo_terngrad_decode_merge": (None, [_ptr, ctypes.c_int, _ptr, _i64]),
             "hpo_sparse_decode_merge": (None, [_ptr, ctypes.c_int, _ptr, _i64, _ptr, _ptr, _f64]),
             "hpo_compll_decode": (_i64, [_ptr, _i64, _ptr, _i64]),
+            "hpo_compll_payload_bytes": (_i64, [_i64, ctypes.c_int]),
+            "hpo_compll_encode": (_i64, [_ptr, _ptr, _i64, _ptr, ctypes.c_int]),
+            "hpo_lcg_uniform": (None, [ctypes.c_uint32, _f32, _f32, _ptr, _i64]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(L, name)
@@ -283,3 +286,20 @@ def compll_decode(compressed, out_cap):
     out = np.zeros(out_cap, dtype=np.float32)
     cnt = lib().hpo_compll_decode(_p(compressed), compressed.size, _p(out), out_cap)
     return out[:cnt]
+
+
+def compll_payload_bytes(n, b):
+    return int(lib().hpo_compll_payload_bytes(n, b))
+
+
+def compll_encode(g, u, b):
+    g, u = _f32c(g), _f32c(u)
+    pay = _payload(compll_payload_bytes(g.size, b))
+    lib().hpo_compll_encode(_p(g), _p(u), g.size, _p(pay), b)
+    return pay
+
+
+def lcg_uniform(seed, n, lo=0.0, hi=1.0):
+    out = np.empty(n, dtype=np.float32)
+    lib().hpo_lcg_uniform(seed, lo, hi, _p(out), n)
+    return out

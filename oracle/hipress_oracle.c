@@ -35,8 +35,11 @@
  * reference's numbers every function here except the bit-placement helpers is
  * "parity unpinned".  They are pinned instead by hand-worked known answers,
  * closed forms, invariants and brute force in tests/test_oracle_*.py.
- * hpo_get_code/hpo_put_code and hpo_compll_decode are pinned against the
- * reference text (TernGradDecode_body.h:44,65-72).
+ * hpo_get_code/hpo_put_code, hpo_compll_decode and hpo_lcg_uniform are pinned
+ * against the reference text (TernGradDecode_body.h:44,65-72;
+ * naive_random.hpp:40-68); hpo_compll_encode follows the DSL source of the
+ * in-tree operator and is pinned by its header layout, grid-point round trips
+ * through hpo_compll_decode and a float64 closed form.
  *
  * Build: gcc -O2 -ffp-contract=off -fno-fast-math (see oracle/Makefile).  All
  * arithmetic is IEEE binary32 round-to-nearest with no contraction.
@@ -518,4 +521,63 @@ int64_t hpo_compll_decode(const uint8_t *compressed, int64_t csz, float *out, in
         out[i] = (float)code * gap + mn;
     }
     return count < 0 ? 0 : count;
+}
+
+/* Encode of the in-tree CompLL operator as its DSL source states it
+ * (/root/reference/src/CompLL/GCGen/pse/TernGradEncode.pse:22-33), not as the
+ * generator mis-translated it (the generated functor walks output bytes as if
+ * they were element indices and shifts codes in from the wrong end,
+ * TernGradEncode_body.h:48-59):
+ *   max = reduce(g, -99999, greater), min = reduce(g, 99999, smaller) in float;
+ *   gap = (max - min) / ((1<<b) - 1);  tail = n % (1<<b) kept as uint8;
+ *   code_i = floor((g_i - min) / gap + u_i), u_i an explicit uniform[0,1) draw in
+ *   place of random<float>(0,1), limited to [0, 2^b - 1]; gap == 0 gives code 0;
+ *   code i is stored where the decoder reads it: bit (i mod 8/b)*b of byte
+ *   floor(i*b/8) after the 10-byte header [b][tail][min][max]
+ *   (TernGradEncode_body.h:114,120-123; TernGradDecode_body.h:44).
+ * b must divide 8.  Returns the payload length 10 + ceil(n*b/8). */
+int64_t hpo_compll_payload_bytes(int64_t n, int b) { return 10 + (n * b + 7) / 8; }
+
+int64_t hpo_compll_encode(const float *g, const float *u, int64_t n, uint8_t *compressed, int b)
+{
+    float mx = -99999.0f, mn = 99999.0f, gap;
+    int64_t nbytes = (n * b + 7) / 8;
+    uint8_t *Q = compressed + 10;
+    uint8_t tail = (uint8_t)(n % (1 << b));
+    uint32_t top = (1u << b) - 1u;
+    for (int64_t i = 0; i < n; ++i) {
+        if (g[i] > mx) mx = g[i];
+        if (g[i] < mn) mn = g[i];
+    }
+    gap = (mx - mn) / (float)top;
+    compressed[0] = (uint8_t)b;
+    compressed[1] = tail;
+    memcpy(compressed + 2, &mn, 4);
+    memcpy(compressed + 6, &mx, 4);
+    memset(Q, 0, (size_t)nbytes);
+    for (int64_t i = 0; i < n; ++i) {
+        uint32_t code = 0;
+        if (gap > 0.0f) {
+            float r = (g[i] - mn) / gap + u[i];
+            float f = floorf(r);
+            code = f <= 0.0f ? 0u : (f >= (float)top ? top : (uint32_t)f);
+        }
+        Q[i * b / 8] |= (uint8_t)(code << ((i % (8 / b)) * b));
+    }
+    return 10 + nbytes;
+}
+
+/* The reference's generator for its rounding noise
+ * (/root/reference/src/CompLL/GCGen/output/naive_random.hpp:40-68): a 32-bit
+ * linear congruential sequence x <- 1103515245*x + 12345, mapped to [lo, hi] by
+ * float(x / (4294967295.0 / (hi - lo))) + lo (the division in double).  Fills
+ * out[0..n) with consecutive draws starting from `seed`. */
+void hpo_lcg_uniform(uint32_t seed, float lo, float hi, float *out, int64_t n)
+{
+    uint32_t x = seed;
+    double scale = 4294967295.0 / (double)(hi - lo);
+    for (int64_t i = 0; i < n; ++i) {
+        x = 1103515245u * x + 12345u;
+        out[i] = (float)((double)x / scale) + lo;
+    }
 }
