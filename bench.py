@@ -233,6 +233,35 @@ class MergeWorkload:
         self.chunks = []
 
 
+class CompllWorkload:
+    """The in-tree CompLL operator (bit width 2, 10-byte header) on the largest VGG19
+    tensor through the per-tensor entry points."""
+
+    def __init__(self, name, n, bitwidth=2):
+        self.name, self.sizes, self.elements, self.b = name, [n], n, bitwidth
+        self.enc_bytes, self.dec_bytes = 8.0 + bitwidth / 8.0, 4.0 + bitwidth / 8.0
+        self.dominant_kernel, self.dominant_bytes = "compll_quant_kernel", 8.0 + bitwidth / 8.0
+
+    def setup(self, dev):
+        import torch
+
+        import hipress_amd as hp
+        from hipress_amd import workloads as W
+
+        self.hp = hp
+        self.g = W.normal_set(self.sizes, dev, 0, sigma=1e-3)[0]
+        self.u = W.uniform_set(self.sizes, dev, 1000)[0]
+        self.pay = torch.zeros(hp.compll_payload_bytes(self.elements, self.b), dtype=torch.uint8, device=dev)
+        self.out = torch.empty(self.elements, device=dev)
+
+    def step(self, ev=None):
+        self.hp.compll_terngrad_encode(self.g, self.u, self.pay, self.b)
+        self.hp.compll_terngrad_decode(self.pay, self.out)
+
+    def close(self):
+        self.g = self.u = self.pay = self.out = None
+
+
 def make_workload(name):
     from hipress_amd import workloads as W
 
@@ -265,6 +294,8 @@ def make_workload(name):
                            "sparse_accum_kernel", 20.0, nphases=7)
     if name == "graddrop_bert_large":
         return SetWorkload(name, "graddrop", bert, "n1e-3", {"ratio": 0.01}, 12.0, 4.0, 0, "sparse_accum_kernel", 12.0, nphases=7)
+    if name == "compll_b2_fc6":
+        return CompllWorkload(name, max(vgg))
     if name == "merge_tbq_vgg19":
         return MergeWorkload(name, "tbq", W.chunk_sizes(vgg))
     if name == "merge_dgc_vgg19":
@@ -274,7 +305,7 @@ def make_workload(name):
 
 ALL_WORKLOADS = [
     "onebit_vgg19", "onebit_deferred_vgg19", "tbq_vgg19", "terngrad_vgg19", "dgc_vgg19", "graddrop_vgg19", "tbq_262144", "tbq_262144_x512",
-    "terngrad_resnet50", "dgc_bert_large", "graddrop_bert_large", "merge_tbq_vgg19", "merge_dgc_vgg19",
+    "terngrad_resnet50", "dgc_bert_large", "graddrop_bert_large", "merge_tbq_vgg19", "merge_dgc_vgg19", "compll_b2_fc6",
 ]
 
 

@@ -526,6 +526,7 @@ int hipress_compll_decode(const void* compressed, int64_t compressed_bytes, floa
     s.out = out;
     s.n = (unsigned long long)n;
     s.ntiles = tiles_of(n);
+    s.aligned = al16(out);
     return hiperr(launch_compll_decode(single_launch(s), static_cast<hipStream_t>(stream)));
 }
 

@@ -61,19 +61,23 @@ __global__ __launch_bounds__(kBlock) void compll_minmax_kernel(Src src, float* p
     }
 }
 
+constexpr int kHeaderBlock = 1024;
+
 template <class SegSrc>
-__global__ __launch_bounds__(kBlock) void compll_header_kernel(SegSrc src, const float* partial) {
-    __shared__ float smx[kBlock], smn[kBlock];
+__global__ __launch_bounds__(kHeaderBlock) void compll_header_kernel(SegSrc src, const float* partial) {
+    __shared__ float smx[kHeaderBlock], smn[kHeaderBlock];
     const Seg s = src.at(blockIdx.x);
     float mx = kMaxInit, mn = kMinInit;
-    for (unsigned t = threadIdx.x; t < s.ntiles; t += kBlock) {
-        mx = fmaxf(mx, partial[2 * (s.tile0 + t)]);
-        mn = fminf(mn, partial[2 * (s.tile0 + t) + 1]);
+    const float2* p2 = reinterpret_cast<const float2*>(partial) + s.tile0;
+    for (unsigned t = threadIdx.x; t < s.ntiles; t += kHeaderBlock) {
+        float2 v = p2[t];
+        mx = fmaxf(mx, v.x);
+        mn = fminf(mn, v.y);
     }
     smx[threadIdx.x] = mx;
     smn[threadIdx.x] = mn;
     __syncthreads();
-    for (int w = kBlock / 2; w >= 1; w >>= 1) {
+    for (int w = kHeaderBlock / 2; w >= 1; w >>= 1) {
         if ((int)threadIdx.x < w) {
             smx[threadIdx.x] = fmaxf(smx[threadIdx.x], smx[threadIdx.x + w]);
             smn[threadIdx.x] = fminf(smn[threadIdx.x], smn[threadIdx.x + w]);
@@ -156,18 +160,41 @@ __global__ __launch_bounds__(kBlock) void compll_decode_kernel(Src src) {
     if (count > (long long)s.n) count = (long long)s.n;
     const uint8_t* Q = s.pay + 10;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
-    const unsigned per = 8 / b, mask = (1u << b) - 1u;
+    const unsigned mask = (1u << b) - 1u;
+    const bool vec = s.aligned != 0;
+    unsigned bits[4];  // the 4*b code bits of this lane's four elements, per step
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         long long e = base + j * 256 + lane * 4;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            long long i = e + k;
-            if (i < count) {
-                unsigned code = (Q[i * b / 8] >> ((unsigned)(i % per) * b)) & mask;
-                s.out[i] = __fadd_rn(__fmul_rn((float)code, gap), mn);
+        bits[j] = 0;
+        if (e < count) {  // e is a multiple of 4, so its codes start on a byte (b >= 2) or nibble (b == 1) boundary
+            const long long byte0 = e * b / 8;
+            if (b == 8) {
+                bits[j] = Q[byte0];
+                if (e + 1 < count) bits[j] |= (unsigned)Q[byte0 + 1] << 8;
+                if (e + 2 < count) bits[j] |= (unsigned)Q[byte0 + 2] << 16;
+                if (e + 3 < count) bits[j] |= (unsigned)Q[byte0 + 3] << 24;
+            } else if (b == 4) {
+                bits[j] = Q[byte0];
+                if (e + 2 < count) bits[j] |= (unsigned)Q[byte0 + 1] << 8;
+            } else if (b == 2) {
+                bits[j] = Q[byte0];
+            } else {
+                bits[j] = (Q[byte0] >> ((e & 4) ? 4 : 0)) & 0xfu;
             }
         }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = base + j * 256 + lane * 4;
+        if (e >= count) continue;
+        f4 o;
+        o.x = __fadd_rn(__fmul_rn((float)(bits[j] & mask), gap), mn);
+        o.y = __fadd_rn(__fmul_rn((float)((bits[j] >> b) & mask), gap), mn);
+        o.z = __fadd_rn(__fmul_rn((float)((bits[j] >> (2 * b)) & mask), gap), mn);
+        o.w = __fadd_rn(__fmul_rn((float)((bits[j] >> (3 * b)) & mask), gap), mn);
+        if (vec && e + 3 < count) st4(s.out + e, o);
+        else st4_guard(s.out, e, count, o);
     }
 }
 
@@ -175,7 +202,7 @@ template <class Src, class SegSrcT>
 static hipError_t compll_encode_src(const Src& src, const SegSrcT& ssrc, unsigned ntiles, unsigned nsegs, int b,
                                     float* partial, hipStream_t st) {
     hipLaunchKernelGGL((compll_minmax_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src, partial);
-    hipLaunchKernelGGL((compll_header_kernel<SegSrcT>), dim3(nsegs), dim3(kBlock), 0, st, ssrc, partial);
+    hipLaunchKernelGGL((compll_header_kernel<SegSrcT>), dim3(nsegs), dim3(kHeaderBlock), 0, st, ssrc, partial);
     if (b == 1) hipLaunchKernelGGL((compll_quant_kernel<Src, 1>), dim3(ntiles), dim3(kBlock), 0, st, src);
     else if (b == 2) hipLaunchKernelGGL((compll_quant_kernel<Src, 2>), dim3(ntiles), dim3(kBlock), 0, st, src);
     else if (b == 4) hipLaunchKernelGGL((compll_quant_kernel<Src, 4>), dim3(ntiles), dim3(kBlock), 0, st, src);
