@@ -1,0 +1,214 @@
+"""Selective compression and partitioning planner (SeCoPa).
+
+For every gradient of a model the planner decides whether compressing it pays off
+and into how many partitions it should be cut, from piecewise-linear cost models
+of the synchronisation steps.  It restates the reference planner
+(/root/reference/src/SeCoPa/SeCoPa.py:4-113) - same cost formulas, same
+tie-breaking, same `name,size,y|n,K` plan lines (SeCoPa.py:139-151) - and adds what
+the reference leaves to its users (/root/reference/src/SeCoPa/README.md:14-16):
+fitting the encode / decode coefficients from measurements of this library's own
+kernels on the GPU at hand.
+
+    python -m hipress_amd.planner --input input.txt --output SeCoPaPlan.txt --topology PS --nnodes 4
+    python -m hipress_amd.planner --calibrate tbq ...     # encode/decode models measured on cuda:0
+"""
+import argparse
+import json
+from dataclasses import dataclass, field
+
+
+@dataclass(frozen=True)
+class CostModel:
+    """t(x) = overhead below the break-even size, weight * x + bias above it
+    (SeCoPa.py:4-20).  The break-even size is where the line reaches the floor."""
+
+    weight: float
+    bias: float
+    overhead: float
+
+    @property
+    def threshold(self):
+        if self.weight == 0:
+            return 0
+        return max(0, (self.overhead - self.bias) / self.weight)
+
+    def cost(self, x):
+        return self.overhead if x < self.threshold else self.weight * x + self.bias
+
+
+# Coefficients the reference ships (SeCoPa.py:25-39); their unit and hardware are not stated there.
+REFERENCE_ENCODE = CostModel(1.4133e-8, 5.8938e-2, 0.05408)
+REFERENCE_DECODE = CostModel(6.2041e-9, 1.3956e-1, 0.07287)
+REFERENCE_RING_SEND = CostModel(8.5005e-7, 2.0337e-1, 0.09766)
+REFERENCE_GATHER = {4: CostModel(2.7156e-6, 4.1930e-1, 0.15573), 8: CostModel(6.1167e-6, 8.0768e-1, 0.28778),
+                    16: CostModel(1.2937e-5, 1.4406, 0.59503)}
+REFERENCE_BROADCAST = {4: CostModel(2.7157e-6, 2.2156e-1, 0.14820), 8: CostModel(6.1172e-6, 2.7285e-1, 0.29666),
+                       16: CostModel(1.2915e-5, 4.5538e-1, 0.58353)}
+
+
+@dataclass
+class Planner:
+    """Cluster of `nodes` workers; every model can be replaced (e.g. by a fit from `calibrate`)."""
+
+    nodes: int = 16
+    comp_ratio: float = 1.0 / 16
+    encode: CostModel = REFERENCE_ENCODE
+    decode: CostModel = REFERENCE_DECODE
+    aggregate: CostModel = CostModel(0, 0, 0)
+    ring_send: CostModel = REFERENCE_RING_SEND
+    gather: CostModel = field(default=None)
+    broadcast: CostModel = field(default=None)
+
+    def __post_init__(self):
+        if self.gather is None or self.broadcast is None:
+            if self.nodes not in REFERENCE_GATHER:
+                raise ValueError("reference gather/broadcast models exist for 4, 8 and 16 nodes only")
+            self.gather = self.gather or REFERENCE_GATHER[self.nodes]
+            self.broadcast = self.broadcast or REFERENCE_BROADCAST[self.nodes]
+
+    # Each *_costs method returns the cost for K = 1..nodes partitions, terms added in the
+    # reference's order so that ties fall the same way.
+    def uncompressed_costs(self, size, topology="PS"):
+        n = self.nodes
+        out = []
+        for k in range(1, n + 1):
+            part = size / k
+            agg = (n - 1) * self.aggregate.cost(part)
+            if topology == "PS":  # co-located servers: gather, N-1 aggregations, broadcast (SeCoPa.py:46-59)
+                out.append(self.gather.cost(part) + self.broadcast.cost(part) + agg)
+            else:  # ring: 2(N-1) sends, N-1 aggregations (SeCoPa.py:61-71)
+                out.append(2 * (n - 1) * self.ring_send.cost(part) + agg)
+        return out
+
+    def compressed_costs(self, size, topology="PS"):
+        n, r = self.nodes, self.comp_ratio
+        out = []
+        for k in range(1, n + 1):
+            part, cpart = size / k, size * r / k
+            agg = (n - 1) * self.aggregate.cost(part)
+            if topology == "PS":  # SeCoPa.py:75-88
+                enc = min(k + 1, n) * self.encode.cost(part)
+                dec = min(n - 1 + k, 2 * (n - 1)) * self.decode.cost(cpart)
+                out.append(self.gather.cost(cpart) + self.broadcast.cost(cpart) + enc + dec + agg)
+            else:  # SeCoPa.py:90-102
+                send = 2 * (n - 1) * self.ring_send.cost(cpart)
+                out.append(send + n * self.encode.cost(part) + n * self.decode.cost(cpart) + agg)
+        return out
+
+    @staticmethod
+    def _best(costs):
+        best = min(costs)
+        return best, costs.index(best) + 1  # the smallest K among equals
+
+    def decide(self, size, topology="PS"):
+        """-> ('y' | 'n', partitions): compress only if strictly cheaper (SeCoPa.py:105-113)."""
+        plain, plain_k = self._best(self.uncompressed_costs(size, topology))
+        comp, comp_k = self._best(self.compressed_costs(size, topology))
+        return ("y", comp_k) if plain > comp else ("n", plain_k)
+
+    def plan(self, gradients, topology="PS"):
+        """gradients: iterable of (name, size) -> plan lines `name,size,y|n,K`."""
+        lines = []
+        for name, size in gradients:
+            flag, parts = self.decide(size, topology)
+            lines.append(f"{name},{size},{flag},{parts}")
+        return lines
+
+
+def read_gradients(path):
+    out = []
+    with open(path) as f:
+        for line in f:
+            if line.strip():
+                cols = line.split(",")
+                out.append((str(cols[0]), int(cols[1])))
+    return out
+
+
+# ---------------------------------------------------------------- fitting
+def fit_cost_model(sizes, times):
+    """Least-squares line through the measurements that rise above the floor; the floor
+    (overhead) is the smallest time seen.  Returns a CostModel in the unit of `times`."""
+    pts = sorted(zip(sizes, times))
+    floor = min(t for _, t in pts)
+    rising = [(x, t) for x, t in pts if t > 1.25 * floor] or pts[-2:]
+    if len(rising) < 2:
+        rising = pts[-2:]
+    n = len(rising)
+    sx = sum(x for x, _ in rising)
+    st = sum(t for _, t in rising)
+    sxx = sum(x * x for x, _ in rising)
+    sxt = sum(x * t for x, t in rising)
+    den = n * sxx - sx * sx
+    weight = (n * sxt - sx * st) / den if den else 0.0
+    bias = (st - weight * sx) / n
+    return CostModel(weight, bias, floor)
+
+
+def calibrate(alg="tbq", sizes=None, reps=20, comp_ratio=None):
+    """Measures encode and decode of `alg` on cuda:0 over a range of tensor sizes (one tensor
+    per launch sequence, as the planner's per-partition costs assume) and fits both models.
+    Times are in milliseconds; encode is a function of the element count, decode of the
+    compressed size in elements (count * ratio), the arguments the planner passes them."""
+    import torch
+
+    import hipress_amd as hp
+
+    sizes = sizes or [1 << k for k in range(10, 28, 2)]
+    ratio = comp_ratio if comp_ratio is not None else {"onebit": 1 / 32}.get(alg, 1 / 16)
+    enc_t, dec_t = [], []
+    for n in sizes:
+        g = torch.randn(n, device="cuda") * 1e-2
+        t = {"gradient": g, "out": torch.empty_like(g)}
+        if alg in ("tbq", "onebit"):
+            t["residual"] = torch.zeros_like(g)
+            nb = hp.tbq_payload_bytes(n) if alg == "tbq" else hp.onebit_payload_bytes(n)
+        elif alg == "terngrad":
+            t["uniform"] = torch.rand(n, device="cuda")
+            nb = hp.terngrad_payload_bytes(n, 512)
+        elif alg == "dgc":
+            t["momentum"], t["accumulator"] = torch.zeros_like(g), torch.zeros_like(g)
+            nb = hp.dgc_payload_bytes(n, 0.001)
+        else:
+            t["accumulator"] = torch.zeros_like(g)
+            nb = hp.graddrop_payload_bytes(n, 0.01)
+        t["compressed"] = torch.zeros(nb, dtype=torch.uint8, device="cuda")
+        b = hp.Batch(alg, [t], threshold=0.05, ratio=0.01 if alg == "graddrop" else 0.001)
+        for fn, acc in ((b.encode, enc_t), (b.decode, dec_t)):
+            for _ in range(3):
+                fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            acc.append(e0.elapsed_time(e1) / reps)
+        b.close()
+    return {"alg": alg, "unit": "ms", "sizes": sizes, "encode_ms": enc_t, "decode_ms": dec_t, "comp_ratio": ratio,
+            "encode": fit_cost_model(sizes, enc_t), "decode": fit_cost_model([n * ratio for n in sizes], dec_t)}
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description="SeCoPa: selective compression and partitioning plan")
+    ap.add_argument("--input", default="input.txt", help="lines of name,size (fp32 elements)")
+    ap.add_argument("--output", default="SeCoPaPlan.txt")
+    ap.add_argument("--topology", default="PS", choices=["PS", "RING"])
+    ap.add_argument("--nnodes", type=int, default=16)
+    ap.add_argument("--calibrate", metavar="ALG", default=None,
+                    help="measure ALG's encode/decode on cuda:0 and plan with the fitted models "
+                         "(communication models stay the reference's)")
+    args = ap.parse_args(argv)
+    kw = {}
+    if args.calibrate:
+        cal = calibrate(args.calibrate)
+        kw = {"encode": cal["encode"], "decode": cal["decode"], "comp_ratio": cal["comp_ratio"]}
+        print(json.dumps({k: (v.__dict__ if isinstance(v, CostModel) else v) for k, v in cal.items()}))
+    planner = Planner(nodes=args.nnodes, **kw)
+    with open(args.output, "w") as f:
+        for line in planner.plan(read_gradients(args.input), args.topology):
+            f.write(line + "\n")
+
+
+if __name__ == "__main__":
+    main()

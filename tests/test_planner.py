@@ -1,0 +1,86 @@
+"""The SeCoPa planner against the reference's own example: its input.txt and the
+SeCoPaPlan.txt shipped beside it (/root/reference/src/SeCoPa/input.txt,
+SeCoPaPlan.txt; copied as data under tests/golden/).  The shipped plan is what
+`--topology PS --nnodes 4` produces; its last line was made from a different size
+(1048576 instead of input.txt's 1000), so it is checked with the size it states."""
+import os
+
+import pytest
+
+from hipress_amd import planner as P
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def read_plan():
+    with open(os.path.join(GOLDEN, "secopa_plan_ps4.txt")) as f:
+        return [l.strip() for l in f if l.strip()]
+
+
+def test_reference_plan_is_reproduced():
+    grads = P.read_gradients(os.path.join(GOLDEN, "secopa_input.txt"))
+    want = read_plan()
+    assert len(grads) == len(want) == 38
+    got = P.Planner(nodes=4).plan(grads, "PS")
+    assert got[:37] == want[:37]
+    # every line of the shipped plan, with the size that line states
+    pl = P.Planner(nodes=4)
+    for line in want:
+        name, size, flag, parts = line.split(",")
+        assert pl.decide(int(size), "PS") == (flag, int(parts)), line
+
+
+def test_cli_writes_the_same_file(tmp_path):
+    out = tmp_path / "plan.txt"
+    P.main(["--input", os.path.join(GOLDEN, "secopa_input.txt"), "--output", str(out), "--topology", "PS", "--nnodes", "4"])
+    assert out.read_text().splitlines()[:37] == read_plan()[:37]
+
+
+def test_cost_model_break_even():
+    m = P.CostModel(2.0, 1.0, 5.0)  # floor 5 until 2x + 1 reaches it at x = 2
+    assert m.threshold == 2.0
+    assert m.cost(1.9) == 5.0 and m.cost(2.0) == 5.0 and m.cost(3.0) == 7.0
+    assert P.CostModel(0, 0, 0).threshold == 0 and P.CostModel(0, 0, 0).cost(10) == 0
+    assert P.CostModel(1.0, 3.0, 1.0).threshold == 0  # floor below the intercept: always linear
+    assert P.CostModel(1.0, 3.0, 1.0).cost(0) == 3.0
+
+
+def test_hand_worked_ps_decision():
+    # 2 nodes, unit-free models chosen so that every term is easy to follow
+    pl = P.Planner(nodes=2, comp_ratio=0.25, encode=P.CostModel(0.0, 1.0, 1.0), decode=P.CostModel(0.0, 1.0, 1.0),
+                   gather=P.CostModel(1.0, 0.0, 0.0), broadcast=P.CostModel(1.0, 0.0, 0.0))
+    # plain: K=1 -> 2x, K=2 -> x ; compressed: K=1 -> x/2 + min(2,2)*1 + min(2,2)*1 = x/2 + 4, K=2 -> x/4 + 2 + 2
+    assert pl.uncompressed_costs(16) == [32.0, 16.0]
+    assert pl.compressed_costs(16) == [12.0, 8.0]
+    assert pl.decide(16) == ("y", 2)
+    assert pl.decide(4) == ("n", 2)  # plain 4 vs compressed 5
+    # ties keep the uncompressed path and the smallest K
+    flat = P.Planner(nodes=2, encode=P.CostModel(0, 0, 0), decode=P.CostModel(0, 0, 0),
+                     gather=P.CostModel(0, 0, 1.0), broadcast=P.CostModel(0, 0, 1.0))
+    assert flat.decide(1000) == ("n", 1)
+
+
+def test_ring_formulas():
+    pl = P.Planner(nodes=4, comp_ratio=0.5, encode=P.CostModel(0, 2.0, 2.0), decode=P.CostModel(0, 1.0, 1.0),
+                   ring_send=P.CostModel(1.0, 0.0, 0.0))
+    # plain: 2*(N-1)*x/K = 6x/K ; compressed: 6*(x/2)/K + 4*2 + 4*1
+    assert pl.uncompressed_costs(8, "RING") == [48.0, 24.0, 16.0, 12.0]
+    assert pl.compressed_costs(8, "RING") == [36.0, 24.0, 20.0, 18.0]
+    assert pl.decide(8, "RING") == ("n", 4)
+    assert pl.decide(80, "RING") == ("y", 4)  # 120 vs 72
+
+
+def test_unsupported_cluster_size_needs_models():
+    with pytest.raises(ValueError):
+        P.Planner(nodes=5)
+    P.Planner(nodes=5, gather=P.CostModel(1, 0, 0), broadcast=P.CostModel(1, 0, 0))
+
+
+def test_fit_recovers_a_piecewise_line():
+    true = P.CostModel(3e-6, 0.02, 0.05)
+    xs = [1 << k for k in range(8, 26)]
+    ts = [true.cost(x) for x in xs]
+    fit = P.fit_cost_model(xs, ts)
+    assert fit.overhead == 0.05
+    assert abs(fit.weight - true.weight) / true.weight < 1e-6
+    assert abs(fit.bias - true.bias) < 1e-6
