@@ -16,6 +16,7 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libhipress_oracle.so")
+_SO_OMP = os.path.join(_HERE, "libhipress_oracle_omp.so")
 HEADER_BYTES = 16
 
 
@@ -24,8 +25,25 @@ def build(force=False):
     if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(
         os.path.join(_HERE, "hipress_oracle.c")
     ):
-        subprocess.check_call(["make", "-C", _HERE, "-B", "libhipress_oracle.so"], stdout=subprocess.DEVNULL)
+        subprocess.check_call(["make", "-C", _HERE, "-B", "all"], stdout=subprocess.DEVNULL)
     return _SO
+
+
+def omp_lib():
+    """The all-cores (OpenMP) build of the same source, for the CPU-baseline timing only:
+    hpo_tbq_* and hpo_onebit_* run their loops on every core."""
+    build()
+    if not os.path.exists(_SO_OMP):
+        subprocess.check_call(["make", "-C", _HERE, "libhipress_oracle_omp.so"], stdout=subprocess.DEVNULL)
+    L = ctypes.CDLL(_SO_OMP)
+    L.hpo_threads.restype = ctypes.c_int
+    L.hpo_onebit_encode.argtypes = [_ptr, _ptr, _i64, _ptr]
+    L.hpo_onebit_decode.argtypes = [_ptr, _ptr, _i64]
+    L.hpo_tbq_encode.argtypes = [_ptr, _ptr, _i64, _ptr, _f32]
+    L.hpo_tbq_decode.argtypes = [_ptr, _ptr, _i64]
+    L.hpo_onebit_scale.restype = _f32
+    L.hpo_onebit_scale.argtypes = [_ptr, _ptr, _i64]
+    return L
 
 
 _lib = None

@@ -51,6 +51,20 @@
 
 #define HPO_HEADER_BYTES 16
 
+/* The same source builds the all-cores variant of the CPU baseline (-fopenmp
+ * -DHPO_OMP, libhipress_oracle_omp.so): the TBQ and onebit loops run one packed
+ * word per iteration, so iterations never share a word.  Without HPO_OMP the
+ * pragmas vanish and every loop is sequential. */
+#ifdef HPO_OMP
+#define HPO_PRAGMA(x) _Pragma(#x)
+#define HPO_PARALLEL_FOR HPO_PRAGMA(omp parallel for schedule(static))
+#define HPO_PARALLEL_SUM(v) HPO_PRAGMA(omp parallel for schedule(static) reduction(+ : v))
+int hpo_threads(void);
+#else
+#define HPO_PARALLEL_FOR
+#define HPO_PARALLEL_SUM(v)
+#endif
+
 /* ------------------------------------------------------------------ */
 /* wire rule                                                          */
 /* ------------------------------------------------------------------ */
@@ -123,23 +137,29 @@ void hpo_tbq_encode(const float *g, float *r, int64_t n, uint8_t *payload, float
 {
     uint32_t *hdr = (uint32_t *)payload;
     uint32_t *w = (uint32_t *)(payload + HPO_HEADER_BYTES);
+    int64_t nw = words_for(n, 2);
     memcpy(&hdr[0], &tau, 4);
     hdr[1] = (uint32_t)n;
     hdr[2] = 0;
     hdr[3] = 0;
-    memset(w, 0, 4 * words_for(n, 2));
-    for (int64_t i = 0; i < n; ++i) {
-        float v = r[i] + g[i];
-        uint32_t code = 0;
-        if (v >= tau) {
-            code = 1;
-            v = v - tau;
-        } else if (v <= -tau) {
-            code = 2;
-            v = v + tau;
+    /* one word (16 codes) at a time, so that the OpenMP build can share the loop */
+    HPO_PARALLEL_FOR
+    for (int64_t k = 0; k < nw; ++k) {
+        int64_t hi = 16 * k + 16 < n ? 16 * k + 16 : n;
+        w[k] = 0;
+        for (int64_t i = 16 * k; i < hi; ++i) {
+            float v = r[i] + g[i];
+            uint32_t code = 0;
+            if (v >= tau) {
+                code = 1;
+                v = v - tau;
+            } else if (v <= -tau) {
+                code = 2;
+                v = v + tau;
+            }
+            r[i] = v;
+            hpo_put_code(w, i, 2, code);
         }
-        r[i] = v;
-        hpo_put_code(w, i, 2, code);
     }
 }
 
@@ -154,6 +174,7 @@ void hpo_tbq_decode(const uint8_t *payload, float *out, int64_t n)
     float tau;
     const uint32_t *w = (const uint32_t *)(payload + HPO_HEADER_BYTES);
     memcpy(&tau, payload, 4);
+    HPO_PARALLEL_FOR
     for (int64_t i = 0; i < n; ++i)
         out[i] = tbq_value(hpo_get_code(w, i, 2), tau);
 }
@@ -168,6 +189,7 @@ void hpo_tbq_decode(const uint8_t *payload, float *out, int64_t n)
 float hpo_onebit_scale(const float *g, const float *r, int64_t n)
 {
     double acc = 0.0;
+    HPO_PARALLEL_SUM(acc)
     for (int64_t i = 0; i < n; ++i) {
         float v = r[i] + g[i];
         acc += (double)fabsf(v);
@@ -181,17 +203,22 @@ void hpo_onebit_encode_with_scale(const float *g, float *r, int64_t n, uint8_t *
 {
     uint32_t *hdr = (uint32_t *)payload;
     uint32_t *w = (uint32_t *)(payload + HPO_HEADER_BYTES);
+    int64_t nw = words_for(n, 1);
     memcpy(&hdr[0], &s, 4);
     hdr[1] = (uint32_t)n;
     hdr[2] = 0;
     hdr[3] = 0;
-    memset(w, 0, 4 * words_for(n, 1));
-    for (int64_t i = 0; i < n; ++i) {
-        float v = r[i] + g[i];
-        uint32_t bit = v >= 0.0f ? 1u : 0u;
-        float d = bit ? s : -s;
-        r[i] = v - d;
-        hpo_put_code(w, i, 1, bit);
+    HPO_PARALLEL_FOR
+    for (int64_t k = 0; k < nw; ++k) {
+        int64_t hi = 32 * k + 32 < n ? 32 * k + 32 : n;
+        w[k] = 0;
+        for (int64_t i = 32 * k; i < hi; ++i) {
+            float v = r[i] + g[i];
+            uint32_t bit = v >= 0.0f ? 1u : 0u;
+            float d = bit ? s : -s;
+            r[i] = v - d;
+            hpo_put_code(w, i, 1, bit);
+        }
     }
 }
 
@@ -205,6 +232,7 @@ void hpo_onebit_decode(const uint8_t *payload, float *out, int64_t n)
     float s;
     const uint32_t *w = (const uint32_t *)(payload + HPO_HEADER_BYTES);
     memcpy(&s, payload, 4);
+    HPO_PARALLEL_FOR
     for (int64_t i = 0; i < n; ++i)
         out[i] = hpo_get_code(w, i, 1) ? s : -s;
 }
@@ -581,3 +609,11 @@ void hpo_lcg_uniform(uint32_t seed, float lo, float hi, float *out, int64_t n)
         out[i] = (float)((double)x / scale) + lo;
     }
 }
+
+/* Threads the all-cores build runs its parallel loops on (1 for the plain build). */
+#ifdef HPO_OMP
+#include <omp.h>
+int hpo_threads(void) { return omp_get_max_threads(); }
+#else
+int hpo_threads(void) { return 1; }
+#endif
