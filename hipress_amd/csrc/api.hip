@@ -52,7 +52,7 @@ inline bool bad_ratio(double r) { return !(r > 0.0 && r <= 1.0); }
 
 // Workspace of a sparse launch: six uint32 arrays, each starting on a 256-byte boundary.
 struct SparseWsLayout {
-    int64_t sample_off, gmax_off, counts_off, thr_off, hist_off, ctl_off, bytes;
+    int64_t sample_off, grec_off, counts_off, thr_off, hist_off, ctl_off, bytes;
 };
 
 inline SparseWsLayout sparse_ws_layout(int64_t total_ns, int64_t total_tiles, int64_t nsegs) {
@@ -60,8 +60,8 @@ inline SparseWsLayout sparse_ws_layout(int64_t total_ns, int64_t total_tiles, in
     int64_t off = 0;
     l.sample_off = off;
     off += round_up(4 * total_ns, 256);
-    l.gmax_off = off;
-    off += round_up(4 * 64 * total_tiles, 256);
+    l.grec_off = off;
+    off += round_up(8 * 64 * total_tiles, 256);
     l.counts_off = off;
     off += round_up(4 * 2 * total_tiles, 256);
     l.thr_off = off;
@@ -78,7 +78,7 @@ inline SparseWs sparse_ws_at(void* base, const SparseWsLayout& l) {
     uint8_t* b = static_cast<uint8_t*>(base);
     SparseWs w;
     w.sample = reinterpret_cast<uint32_t*>(b + l.sample_off);
-    w.gmax = reinterpret_cast<uint32_t*>(b + l.gmax_off);
+    w.grec = reinterpret_cast<uint2*>(b + l.grec_off);
     w.counts = reinterpret_cast<uint32_t*>(b + l.counts_off);
     w.thr = reinterpret_cast<uint32_t*>(b + l.thr_off);
     w.hist = reinterpret_cast<uint32_t*>(b + l.hist_off);

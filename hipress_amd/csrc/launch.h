@@ -23,7 +23,8 @@ hipError_t launch_dense_merge(const MergeLaunch& L, int alg, hipStream_t st);
 // Sparse (DGC / GradDrop) pipeline.  ws is the launch's workspace.
 struct SparseWs {
     uint32_t* sample;   // |acc'| keys at the sample positions, all tensors back to back
-    uint32_t* gmax;     // max |acc'| key of every 64-element group: 64 per tile
+    uint2* grec;        // per 64-element group (64 per tile): {bits of the acc' value with the largest |.|,
+                        //  (upper bound of the second-largest key, multiple of 64) | position of the largest}
     uint32_t* counts;   // per tile {above, equal} counts, then their exclusive scans
     uint32_t* thr;      // per tensor {threshold key, equal-quota}
     uint32_t* hist;     // per tensor 3 x 2048 bins, one histogram per select pass

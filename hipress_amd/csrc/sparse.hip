@@ -1,24 +1,27 @@
 // Sampled-threshold sparsifiers for gfx950: DGC and GradDrop encode, the shared
-// sparse decode, and the scatter-add half of sparse decode-and-merge.
+// sparse decode, and the tile-owner sparse decode-and-merge.
 //
 // Encode is seven launches over the whole tensor set:
 //   0. accumulate   one streaming pass: mom' = m*mom + g, acc' = acc + mom'
 //                   (GradDrop: acc' = acc + g), written back; the |acc'| keys at
-//                   the sample positions are gathered and the maximum key of
-//                   every 64-element group is recorded on the way;
+//                   the sample positions are gathered and every 64-element group
+//                   leaves a record on the way: its largest |acc'| with value and
+//                   place, and a bound on its second largest;
 //   1-3. select     the k-th largest sample key of every tensor by radix
 //                   selection, 11 + 10 + 10 bits from the top: every pass is one
 //                   launch over all sample tiles, LDS histograms merged into a
 //                   per-tensor global one, the last workgroup of a tensor to
 //                   finish picks the digit;
-//   4. count        only groups whose maximum reaches the threshold are read
-//                   again; per-tile counts of keys above / equal to it;
+//   4. count        per-tile counts of keys above / equal to the threshold: a
+//                   group whose record shows no or one such key is counted from
+//                   the record, only the others are read again;
 //   5. scan         one workgroup per tensor turns the counts into output
 //                   offsets, writes the header and, if more than `capacity`
 //                   elements qualify, re-thresholds on the whole tensor;
-//   6. emit         the flagged groups are read once more and the selected
-//                   (index, value) pairs are written in ascending index order,
-//                   the accumulator (and momentum) being zeroed at those places.
+//   6. emit         the selected (index, value) pairs are written in ascending
+//                   index order, from the record for single-pair groups and from
+//                   one more read for the others, the accumulator (and momentum)
+//                   being zeroed at those places.
 // |x| is handled as the integer key bits(x) & 0x7fffffff, which orders like |x|.
 #include "common.h"
 #include "launch.h"
@@ -32,6 +35,22 @@ constexpr int kBins = 2048;        // histogram bins per select pass (11-bit fir
 __device__ __forceinline__ unsigned key_of(float x) { return __float_as_uint(x) & 0x7fffffffu; }
 
 __device__ __forceinline__ unsigned umax(unsigned a, unsigned b) { return a > b ? a : b; }
+__device__ __forceinline__ unsigned umin(unsigned a, unsigned b) { return a < b ? a : b; }
+
+// What a group record says about threshold thr: `flagged` when the group holds a
+// selected element at all, `multi` when it may hold more than one (the group has
+// to be read), otherwise its only selected element is the recorded one.
+struct GroupView {
+    unsigned key;   // largest key of the group
+    bool flagged, multi;
+};
+__device__ __forceinline__ GroupView view_group(uint2 rec, unsigned thr) {
+    GroupView v;
+    v.key = rec.x & 0x7fffffffu;
+    v.flagged = v.key >= thr && v.key > 0u;
+    v.multi = v.flagged && (rec.y & ~63u) >= thr;
+    return v;
+}
 
 // max over the 16 lanes of a DPP row; every lane of the row gets the result
 __device__ __forceinline__ unsigned row_max16(unsigned x) {
@@ -101,9 +120,22 @@ __device__ __forceinline__ void sparse_accum_tile(const Seg& s, unsigned tile, c
             k2 = (v & 4u) ? k2 : 0u;
             k3 = (v & 8u) ? k3 : 0u;
         }
-        unsigned gm = row_max16(umax(umax(k0, k1), umax(k2, k3)));
-        if ((lane & 15u) == 0)
-            ws.gmax[(unsigned long long)(s.tile0 + tile) * 64 + wave * 16 + j * 4 + (lane >> 4)] = gm;
+        {   // group record: the largest key with its value and place, and a bound on the runner-up
+            const unsigned lo1 = umax(k0, k1), lo2 = umin(k0, k1), plo = k1 > k0 ? 1u : 0u;
+            const unsigned hi1 = umax(k2, k3), hi2 = umin(k2, k3), phi = k3 > k2 ? 3u : 2u;
+            const bool bw = hi1 > lo1;
+            const unsigned l1 = bw ? hi1 : lo1, lp = bw ? phi : plo;       // this lane's largest key and its place
+            const unsigned l2 = bw ? umax(lo1, hi2) : umax(hi1, lo2);     // and its second largest
+            const unsigned m1 = row_max16(l1);
+            const unsigned rowbits = (unsigned)(__ballot(l1 == m1) >> (lane & 48u)) & 0xffffu;  // never empty
+            const bool own = (lane & 15u) == (unsigned)__ffs((int)rowbits) - 1u;
+            const unsigned m2 = row_max16(own ? l2 : l1);
+            if (own) {
+                const float top = lp == 0 ? acc.x : (lp == 1 ? acc.y : (lp == 2 ? acc.z : acc.w));
+                ws.grec[(unsigned long long)(s.tile0 + tile) * 64 + wave * 16 + j * 4 + (lane >> 4)] =
+                    make_uint2(__float_as_uint(top), (((m2 + 63u) >> 6) << 6) | ((lane & 15u) * 4 + lp));
+            }
+        }
         if (s.sstride == 1) {  // small tensor: every element is a sample
             if (e < n) sample[e] = k0;
             if (e + 1 < n) sample[e + 1] = k1;
@@ -246,20 +278,22 @@ __device__ __forceinline__ unsigned pick_row(unsigned row, unsigned a, unsigned 
 }
 
 // Counts, for tile `tile` (4096 elements) of tensor s, the keys above and equal
-// to thr; lane l looks at the maximum of 64-element group l and only groups
-// whose maximum reaches thr are read, eight per round, the next round's loads in
-// flight while this round is counted.  Wavefront-uniform result.
+// to thr; lane l looks at the record of 64-element group l and only groups that
+// may hold more than one such key are read, eight per round, the next round's
+// loads in flight while this round is counted.  Wavefront-uniform result.
 __device__ __forceinline__ void count_tile(const Seg& s, const SparseWs& ws, unsigned tile, unsigned thr,
                                            unsigned lane, unsigned& gt, unsigned& eq) {
     const long long n = (long long)s.n;
     const bool aligned = s.aligned != 0;
     const float* acc = s.s1;
-    unsigned gm = ws.gmax[(unsigned long long)(s.tile0 + tile) * 64 + lane];
-    unsigned long long mask = __ballot(gm >= thr && gm > 0u);
+    const GroupView gv = view_group(ws.grec[(unsigned long long)(s.tile0 + tile) * 64 + lane], thr);
+    unsigned long long mask = __ballot(gv.multi);
     const unsigned row = lane >> 4;
     const long long base = (long long)tile * kTile + (lane & 15u) * 4;
     const f4 zero4 = {0.f, 0.f, 0.f, 0.f};
-    unsigned cg = 0, ce = 0;
+    // a group with a single selected element is counted from its record alone
+    const bool single = gv.flagged && !gv.multi;
+    unsigned cg = single && gv.key > thr, ce = single && gv.key == thr;
     auto fetch = [&](f4& va, f4& vb) {
         unsigned a0 = pop_bit(mask), a1 = pop_bit(mask), a2 = pop_bit(mask), a3 = pop_bit(mask);
         unsigned b0 = pop_bit(mask), b1 = pop_bit(mask), b2 = pop_bit(mask), b3 = pop_bit(mask);
@@ -442,10 +476,10 @@ __global__ __launch_bounds__(kScanBlock) void sparse_scan_kernel(SegSrc src, Spa
         const unsigned old = thr;
         const long long n = (long long)s.n;
         const unsigned long long ngroups = (unsigned long long)s.ntiles * 64;
-        const uint32_t* gmax = ws.gmax + (unsigned long long)s.tile0 * 64;
+        const uint2* grec = ws.grec + (unsigned long long)s.tile0 * 64;
         thr = block_kth_largest(sc, s.cap, [&](auto f) {
             for (unsigned long long g = wave; g < ngroups; g += kScanWaves) {
-                unsigned gm = gmax[g];
+                unsigned gm = grec[g].x & 0x7fffffffu;
                 if (gm >= old && gm > 0u) {
                     long long e = (long long)g * 64 + lane;
                     unsigned key = e < n ? key_of(s.s1[e]) : 0u;
@@ -502,33 +536,39 @@ __global__ __launch_bounds__(kBlock) void sparse_emit_kernel(Src src, SparseWs w
     unsigned pos = G + (E < quota ? E : quota);  // pairs written by earlier tiles
     int32_t* idx = reinterpret_cast<int32_t*>(s.pay + kHeaderBytes);
     float* val = reinterpret_cast<float*>(s.pay + kHeaderBytes + 4ull * s.cap);
-    unsigned gm = ws.gmax[(unsigned long long)(s.tile0 + tile) * 64 + lane];
-    unsigned long long mask = __ballot(gm >= thr && gm > 0u);
+    const uint2 rec = ws.grec[(unsigned long long)(s.tile0 + tile) * 64 + lane];
+    const GroupView gv = view_group(rec, thr);
     if (quota == kNoQuota) {
-        // Usual case: everything at or above the threshold is taken.  Row r of the
-        // wavefront reads the r-th flagged group of a round of four; positions come
-        // from a row prefix sum of the per-lane counts plus the totals of the rows
-        // before.  The next round's loads are issued before this round's stores
-        // (they touch different groups), so rounds overlap.
+        // Usual case: everything at or above the threshold is taken.  Lane l speaks for
+        // group l.  A group with one selected element yields its pair straight from the
+        // record; groups that may hold more are read, four per round: row r of the
+        // wavefront reads the r-th of them, positions come from a row prefix sum of the
+        // per-lane counts, the totals of the rows before and the single-pair groups
+        // below.  The next round's loads are issued before this round's stores (they
+        // touch different groups), so rounds overlap.
+        const unsigned long long smask = __ballot(gv.flagged && !gv.multi);
+        unsigned long long mask = __ballot(gv.multi);
+        const unsigned pos0 = pos;
+        unsigned from_multi = 0;  // pairs of read groups below group `lane`
         const unsigned row = lane >> 4;
         const bool aligned = s.aligned != 0;
         const long long base = (long long)tile * kTile + (lane & 15u) * 4;
         const f4 zero4 = {0.f, 0.f, 0.f, 0.f};
-        unsigned gi;
+        unsigned gi = 64u, c0 = 64u, c1 = 64u, c2 = 64u, c3 = 64u;  // this round's groups (64: none)
         f4 v = zero4;
-        {
-            unsigned g0 = pop_bit(mask), g1 = pop_bit(mask), g2 = pop_bit(mask), g3 = pop_bit(mask);
-            gi = pick_row(row, g0, g1, g2, g3);
+        bool more = mask != 0;
+        if (more) {
+            c0 = pop_bit(mask); c1 = pop_bit(mask); c2 = pop_bit(mask); c3 = pop_bit(mask);
+            gi = pick_row(row, c0, c1, c2, c3);
             if (gi < 64u) v = load_group4(s.s1, base + gi * 64, n, aligned);
         }
-        bool more = true;
         while (more) {
             more = mask != 0;
-            unsigned gi_next = 64u;
+            unsigned gi_next = 64u, n0 = 64u, n1 = 64u, n2 = 64u, n3 = 64u;
             f4 v_next = zero4;
             if (more) {
-                unsigned g0 = pop_bit(mask), g1 = pop_bit(mask), g2 = pop_bit(mask), g3 = pop_bit(mask);
-                gi_next = pick_row(row, g0, g1, g2, g3);
+                n0 = pop_bit(mask); n1 = pop_bit(mask); n2 = pop_bit(mask); n3 = pop_bit(mask);
+                gi_next = pick_row(row, n0, n1, n2, n3);
                 if (gi_next < 64u) v_next = load_group4(s.s1, base + gi_next * 64, n, aligned);
             }
             const long long e = base + gi * 64;
@@ -541,7 +581,8 @@ __global__ __launch_bounds__(kBlock) void sparse_emit_kernel(Src src, SparseWs w
             unsigned t1 = (unsigned)__builtin_amdgcn_readlane((int)incl, 31);
             unsigned t2 = (unsigned)__builtin_amdgcn_readlane((int)incl, 47);
             unsigned t3 = (unsigned)__builtin_amdgcn_readlane((int)incl, 63);
-            unsigned p = pos + (incl - c) + (row > 0 ? t0 : 0u) + (row > 1 ? t1 : 0u) + (row > 2 ? t2 : 0u);
+            unsigned p = pos + (incl - c) + (row > 0 ? t0 : 0u) + (row > 1 ? t1 : 0u) + (row > 2 ? t2 : 0u) +
+                         (gi < 64u ? popc_lt(smask, gi) : 0u);
             if (c && p + c <= s.cap) {  // the scan guarantees room; the test only guards the buffer
                 f4 keep = v;
                 if (s0) { idx[p] = (int32_t)e; val[p] = v.x; keep.x = 0.f; ++p; }
@@ -563,11 +604,24 @@ __global__ __launch_bounds__(kBlock) void sparse_emit_kernel(Src src, SparseWs w
                 }
             }
             pos += t0 + t1 + t2 + t3;
+            from_multi += (lane > c0 ? t0 : 0u) + (lane > c1 ? t1 : 0u) + (lane > c2 ? t2 : 0u) + (lane > c3 ? t3 : 0u);
             gi = gi_next;
             v = v_next;
+            c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+        }
+        if (gv.flagged && !gv.multi) {
+            const unsigned p = pos0 + popc_lt(smask, lane) + from_multi;
+            const long long e = (long long)tile * kTile + lane * 64 + (rec.y & 63u);
+            if (p < s.cap) {
+                idx[p] = (int32_t)e;
+                val[p] = __uint_as_float(rec.x);
+                s.s1[e] = 0.f;
+                if (s.s0) s.s0[e] = 0.f;
+            }
         }
         return;
     }
+    unsigned long long mask = __ballot(gv.flagged);
     // Overflow case: ties at the threshold are rationed in index order, one group
     // of 64 at a time across the whole wavefront.
     unsigned eq_seen = E;
