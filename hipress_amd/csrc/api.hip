@@ -316,6 +316,9 @@ struct hipress_batch {
     uint2* d_map = nullptr;
     uint2* d_smap = nullptr;  // sparse: sample tiles
     uint2* d_cmap = nullptr;  // sparse decode: payload-slot tiles
+    uint32_t* d_tptr = nullptr;      // sparse decode: first payload slot of every tile
+    uint32_t* d_disorder = nullptr;  // sparse decode: per tensor, the epoch in which its payload was last seen out of order
+    unsigned epoch = 0;
     unsigned ntiles = 0, nstiles = 0, nctiles = 0;
     void* ws = nullptr;  // onebit: one float per tile; sparse: SparseWsLayout
     SparseWsLayout swl{};
@@ -704,6 +707,8 @@ int hipress_batch_destroy(hipress_batch* b) {
     (void)hipFree(b->d_map);
     (void)hipFree(b->d_smap);
     (void)hipFree(b->d_cmap);
+    (void)hipFree(b->d_tptr);
+    (void)hipFree(b->d_disorder);
     (void)hipFree(b->ws);
     delete b;
     return HIPRESS_OK;
@@ -767,6 +772,10 @@ int hipress_batch_create(hipress_batch** out, int32_t alg, const hipress_tensor*
             for (unsigned j = 0; j < b->dec[i].ncblk; ++j) cmap.push_back(make_uint2((unsigned)i, j));
         b->nctiles = (unsigned)cmap.size();
         if ((rc = upload(cmap, &b->d_cmap))) return fail(rc);
+        const size_t tptr_bytes = 4 * (size_t)(b->ntiles ? b->ntiles : 1), flag_bytes = 4 * (size_t)(count ? count : 1);
+        if (hipMalloc(reinterpret_cast<void**>(&b->d_tptr), tptr_bytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
+        if (hipMalloc(reinterpret_cast<void**>(&b->d_disorder), flag_bytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
+        if (hipMemset(b->d_disorder, 0, flag_bytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
     }
     if ((rc = upload(b->enc, &b->d_enc))) return fail(rc);
     if ((rc = upload(b->dec, &b->d_dec))) return fail(rc);
@@ -836,7 +845,9 @@ int hipress_batch_decode(hipress_batch* b, void* stream) {
         case HIPRESS_TBQ: return hiperr(launch_tbq_decode(L, st));
         case HIPRESS_TERNGRAD: return hiperr(launch_terngrad_decode(L, st));
         case HIPRESS_DGC:
-        case HIPRESS_GRADDROP: return hiperr(launch_sparse_decode(L, st));
+        case HIPRESS_GRADDROP:
+            if (++b->epoch == 0) b->epoch = 1;  // the flags start at 0, which no call uses
+            return hiperr(launch_sparse_decode_indexed(L, b->d_tptr, b->d_disorder, b->epoch, st));
     }
     return HIPRESS_ERR_PARAM;
 }

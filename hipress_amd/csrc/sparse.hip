@@ -350,7 +350,7 @@ __global__ __launch_bounds__(kBlock) void sparse_count_kernel(Src src, SparseWs 
 // In-place exclusive scan of nw {above, equal} pairs by one workgroup of
 // kScanBlock threads; returns the totals to every thread.  Each wavefront owns a
 // contiguous span: one coalesced sweep for the span totals, a second one that
-// scans 64 pairs at a time with shuffles.
+// scans 256 pairs at a time.
 constexpr int kScanBlock = 1024;
 constexpr int kScanWaves = kScanBlock / 64;
 
@@ -371,6 +371,7 @@ __device__ __forceinline__ void block_scan_pairs(uint32_t* c, unsigned nw, unsig
     const unsigned lo = wave * span < nw ? wave * span : nw;
     const unsigned hi = lo + span < nw ? lo + span : nw;
     unsigned sg = 0, se = 0;
+#pragma unroll 4
     for (unsigned i = lo + lane; i < hi; i += 64) {
         uint2 v = c2[i];
         sg += v.x;
@@ -397,11 +398,22 @@ __device__ __forceinline__ void block_scan_pairs(uint32_t* c, unsigned nw, unsig
         tot_gt += g;
         tot_eq += e;
     }
-    for (unsigned i0 = lo; i0 < hi; i0 += 64) {
-        unsigned i = i0 + lane;
-        uint2 v = i < hi ? c2[i] : make_uint2(0u, 0u);
-        unsigned ig = wave_incl_scan(v.x, lane), ie = wave_incl_scan(v.y, lane);
-        if (i < hi) c2[i] = make_uint2(bg + ig - v.x, be + ie - v.y);
+    // 256 pairs per trip: every lane owns four consecutive pairs, adds them up on its
+    // own, and one wavefront scan of the lane sums places them
+    for (unsigned i0 = lo; i0 < hi; i0 += 256) {
+        const unsigned i = i0 + lane * 4;
+        uint2 v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = i + r < hi ? c2[i + r] : make_uint2(0u, 0u);
+        const unsigned lg = v[0].x + v[1].x + v[2].x + v[3].x, le = v[0].y + v[1].y + v[2].y + v[3].y;
+        const unsigned ig = wave_incl_scan(lg, lane), ie = wave_incl_scan(le, lane);
+        unsigned xg = bg + ig - lg, xe = be + ie - le;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            if (i + r < hi) c2[i + r] = make_uint2(xg, xe);
+            xg += v[r].x;
+            xe += v[r].y;
+        }
         bg += (unsigned)__builtin_amdgcn_readlane((int)ig, 63);
         be += (unsigned)__builtin_amdgcn_readlane((int)ie, 63);
     }
@@ -683,10 +695,8 @@ __device__ __forceinline__ unsigned sparse_header(const uint8_t* pay, unsigned s
 // One workgroup per 1024 slots of a tensor's payload; workgroups past nnz exit.
 constexpr int kSlotTile = 1024;
 
-template <class Src>
-__global__ __launch_bounds__(kBlock) void sparse_scatter_kernel(Src src) {
-    unsigned ct;
-    const Seg s = src.get(ct, blockIdx.x);
+// out[idx[j]] = val[j] for the 1024 slots of slot tile ct
+__device__ __forceinline__ void scatter_slots(const Seg& s, unsigned ct) {
     const int32_t* idx;
     const float* val;
     const unsigned nnz = sparse_header(s.pay, s.cap, idx, val);
@@ -698,6 +708,146 @@ __global__ __launch_bounds__(kBlock) void sparse_scatter_kernel(Src src) {
             long long i = idx[j];
             if (i >= 0 && i < (long long)s.n) s.out[i] = val[j];
         }
+    }
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void sparse_scatter_kernel(Src src) {
+    unsigned ct;
+    const Seg s = src.get(ct, blockIdx.x);
+    scatter_slots(s, ct);
+}
+
+// The same scatter for the tensors of a table whose payload the index kernel found out
+// of order (their tiles were only cleared); workgroups of other tensors leave at once.
+__global__ __launch_bounds__(kBlock) void sparse_scatter_if_disordered_kernel(BatchSrc src, const uint32_t* disorder,
+                                                                              unsigned epoch) {
+    if (disorder[src.map[blockIdx.x].x] != epoch) return;
+    unsigned ct;
+    const Seg s = src.get(ct, blockIdx.x);
+    scatter_slots(s, ct);
+}
+
+// ---- decode with tile pointers (launches over a tensor table) -------------------------
+// A payload in ascending index order holds the pairs of a 4096-element tile as one
+// contiguous run.  The index kernel walks the payload once, records where every
+// tile's run starts and notices disorder; the tile kernel then builds each output
+// tile in LDS (zeros plus the tile's pairs) and writes it once, so no line of the
+// output is written twice.  The tensors whose payload is not in order are only
+// cleared by the tile kernel and then filled by a scatter launch.
+
+// One workgroup per 1024 slots.  ptr[t] (t < ntiles) = first slot whose index lies in
+// tile t or later.  Slot j starts every tile after the tile of slot j-1 up to its
+// own; long stretches of empty tiles are queued and filled by the whole workgroup.
+template <class Src>
+__global__ __launch_bounds__(kBlock) void sparse_decode_index_kernel(Src src, uint32_t* tptr, uint32_t* disorder,
+                                                                     unsigned epoch) {
+    __shared__ unsigned gap_first[kSlotTile + 2], gap_count[kSlotTile + 2], gap_value[kSlotTile + 2];
+    __shared__ unsigned ngaps;
+    unsigned ct;
+    const Seg s = src.get(ct, blockIdx.x);
+    const int32_t* idx;
+    const float* val;
+    const unsigned nnz = sparse_header(s.pay, s.cap, idx, val);
+    const unsigned nt = s.ntiles;
+    if (nt == 0) return;
+    uint32_t* ptr = tptr + s.tile0;
+    if (threadIdx.x == 0) ngaps = 0;
+    __syncthreads();
+    auto tile_of = [&](int32_t i) -> unsigned {  // indices outside the tensor count for the first / last tile
+        if (i < 0) return 0u;
+        unsigned t = (unsigned)i / kTile;
+        return t < nt ? t : nt - 1;
+    };
+    auto start = [&](unsigned t0, unsigned t1, unsigned v) {  // ptr[t0, t1) = v
+        if (t1 - t0 <= 8u) {
+            for (unsigned t = t0; t < t1; ++t) ptr[t] = v;
+        } else {
+            unsigned g = atomicAdd(&ngaps, 1u);
+            gap_first[g] = t0;
+            gap_count[g] = t1 - t0;
+            gap_value[g] = v;
+        }
+    };
+    bool bad = false;
+    const unsigned long long lo = (unsigned long long)ct * kSlotTile;
+#pragma unroll
+    for (int k = 0; k < kSlotTile / kBlock; ++k) {
+        const unsigned long long j = lo + k * kBlock + threadIdx.x;
+        if (j < nnz) {
+            const int32_t cur = idx[j];
+            const unsigned tc = tile_of(cur);
+            unsigned first = 0;
+            if (j) {
+                const int32_t prev = idx[j - 1];
+                bad |= prev > cur;
+                first = tile_of(prev) + 1;
+            }
+            if (tc + 1 > first) start(first, tc + 1, (unsigned)j);
+            if (j == nnz - 1 && tc + 1 < nt) start(tc + 1, nt, nnz);
+        }
+    }
+    if (ct == 0 && threadIdx.x == 0 && nnz == 0 && nt) start(0, nt, 0u);
+    if (bad) disorder[s.id] = epoch;  // every writer stores the same value
+    __syncthreads();
+    const unsigned ng = ngaps;
+    for (unsigned g = 0; g < ng; ++g)
+        for (unsigned t = threadIdx.x; t < gap_count[g]; t += kBlock) ptr[gap_first[g] + t] = gap_value[g];
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void sparse_decode_tile_kernel(Src src, const uint32_t* tptr,
+                                                                    const uint32_t* disorder, unsigned epoch) {
+    __shared__ __attribute__((aligned(16))) float lds[kTile];
+    unsigned tile;
+    const Seg s = src.get(tile, blockIdx.x);
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const long long t_lo = (long long)tile * kTile, t_hi = t_lo + kTile < n ? t_lo + kTile : n;
+    const int32_t* idx;
+    const float* val;
+    const unsigned nnz = sparse_header(s.pay, s.cap, idx, val);
+    unsigned lo = 0, hi = 0;  // a payload out of order: the tile is cleared here and filled by the scatter that follows
+    if (disorder[s.id] != epoch) {
+        lo = tptr[s.tile0 + tile];
+        hi = tile + 1 < s.ntiles ? tptr[s.tile0 + tile + 1] : nnz;
+        if (hi > nnz) hi = nnz;
+        if (lo > hi) lo = hi;
+    }
+    const bool fast = s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n;
+    const f4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    if (lo == hi) {  // nothing lands in this tile
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            long long e = t_lo + wave * kWaveTile + j * 256 + lane * 4;
+            if (fast) st4(s.out + e, zero4);
+            else st4_guard(s.out, e, n, zero4);
+        }
+        return;
+    }
+    // the first round of pairs is requested before the LDS tile is cleared
+    unsigned j0 = lo + threadIdx.x;
+    long long i0 = -1;
+    float v0 = 0.f;
+    if (j0 < hi) {
+        i0 = idx[j0];
+        v0 = val[j0];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<f4*>(&lds[wave * kWaveTile + j * 256 + lane * 4]) = zero4;
+    __syncthreads();
+    if (i0 >= t_lo && i0 < t_hi) lds[i0 - t_lo] = v0;
+    for (unsigned j = j0 + kBlock; j < hi; j += kBlock) {
+        long long i = idx[j];
+        if (i >= t_lo && i < t_hi) lds[i - t_lo] = val[j];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        long long e = t_lo + wave * kWaveTile + j * 256 + lane * 4;
+        f4 v = *reinterpret_cast<const f4*>(&lds[wave * kWaveTile + j * 256 + lane * 4]);
+        if (fast) st4(s.out + e, v);
+        else st4_guard(s.out, e, n, v);
     }
 }
 
@@ -879,6 +1029,24 @@ hipError_t launch_sparse_decode(const Launch& L, hipStream_t st) {
         if (L.nctiles)
             hipLaunchKernelGGL((sparse_scatter_kernel<BatchSrc>), dim3(L.nctiles), dim3(kBlock), 0, st, csrc);
     }
+    return hipGetLastError();
+}
+
+// Decode of a tensor table through tile pointers: tptr has one word per tile of the
+// launch, disorder one word per tensor; epoch must differ from call to call.
+hipError_t launch_sparse_decode_indexed(const Launch& L, uint32_t* tptr, uint32_t* disorder, unsigned epoch,
+                                        hipStream_t st) {
+    if (L.ntiles == 0 || L.single) return hipSuccess;
+    BatchSrc csrc{L.dsegs, L.dcmap};
+    if (L.nctiles)
+        hipLaunchKernelGGL((sparse_decode_index_kernel<BatchSrc>), dim3(L.nctiles), dim3(kBlock), 0, st, csrc, tptr,
+                           disorder, epoch);
+    BatchSrc src{L.dsegs, L.dmap};
+    hipLaunchKernelGGL((sparse_decode_tile_kernel<BatchSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src, tptr, disorder,
+                       epoch);
+    if (L.nctiles)
+        hipLaunchKernelGGL(sparse_scatter_if_disordered_kernel, dim3(L.nctiles), dim3(kBlock), 0, st, csrc, disorder,
+                           epoch);
     return hipGetLastError();
 }
 

@@ -488,10 +488,10 @@ def test_batch_matches_oracle(hp, alg):
 
 @pytest.mark.parametrize("alg,ratio", [("dgc", 0.001), ("graddrop", 0.01)])
 def test_sparse_batch_many_steps(hp, alg, ratio):
-    """A batch keeps a threshold prediction between steps and stages candidates
-    against it.  The steps below make the prediction hold, fail (threshold drops),
-    overflow single staging areas (a local burst) and overflow the payload capacity
-    (many equal large values); every step must still match the oracle bit for bit."""
+    """A batch object is reused step after step and its workspace keeps the previous
+    step's contents.  The steps below change the threshold abruptly, put a burst of
+    large neighbours into one place and overflow the payload capacity (many equal large
+    values); every step must still match the oracle bit for bit."""
     rng = np.random.default_rng(91)
     sizes = [1000003, 262144, 4097, 70001, 300000, 64]
     tensors, refs = [], []
@@ -529,6 +529,63 @@ def test_sparse_batch_many_steps(hp, alg, ratio):
             check_sparse(host(t["compressed"]), want)
             np.testing.assert_array_equal(host(t["accumulator"]), ref["acc"], err_msg=f"step {step} {kind} n={n}")
             np.testing.assert_array_equal(host(t["out"]), oracle.sparse_decode(want, n))
+    b.close()
+
+
+def make_sparse_payload(n, cap, idx, val, nnz=None):
+    """A hand-made dgc/graddrop payload: header {nnz, n, cap, thr}, idx[cap], val[cap]."""
+    pay = np.zeros(16 + 8 * cap, np.uint8)
+    hdr = pay[:16].view(np.uint32)
+    hdr[0], hdr[1], hdr[2] = (len(idx) if nnz is None else nnz), n, cap
+    pay[16 : 16 + 4 * len(idx)].view(np.int32)[:] = idx
+    pay[16 + 4 * cap : 16 + 4 * cap + 4 * len(val)].view(F)[:] = val
+    return pay
+
+
+def test_sparse_batch_decode_handmade_payloads(hp):
+    """The batched sparse decode places every tile's run of pairs through tile pointers.
+    Payloads made by hand: empty, one pair in a large tensor (long stretches of empty
+    tiles), all slots used with the capacity a multiple of 1024, indices outside the
+    tensor at both ends, a tensor shorter than a tile, and two payloads out of order
+    (decoded by the scatter fall-back) between ordered ones.  Two rounds with the payloads
+    exchanged between the rounds, since the batch keeps its pointers and flags."""
+    rng = np.random.default_rng(123)
+
+    def ordered(n, k):
+        return np.sort(rng.choice(n, size=k, replace=False)).astype(np.int32)
+
+    cases = []  # (n, cap, idx, nnz)
+    cases.append((1000003, 4096, np.zeros(0, np.int32), None))                       # empty
+    cases.append((3000000, 1024, np.array([2999999], np.int32), None))              # one pair, last element
+    cases.append((3000000, 1024, np.array([0], np.int32), None))                    # one pair, first element
+    cases.append((500000, 2048, ordered(500000, 2048), None))                       # every slot used
+    cases.append((262144, 512, np.concatenate([[-7, -1], ordered(262144, 300), [262144, 2**31 - 1]]).astype(np.int32), None))
+    cases.append((1000, 64, ordered(1000, 40), None))                               # shorter than a tile
+    cases.append((700001, 8192, rng.permutation(ordered(700001, 5000)).astype(np.int32), None))  # out of order
+    cases.append((700001, 8192, ordered(700001, 5000), None))
+    cases.append((4097, 64, np.array([4096, 0], np.int32), None))                   # out of order, two tiles
+    cases.append((900000, 1024, ordered(900000, 1024), 5000))                       # nnz in the header beyond the capacity
+    tensors, pays = [], []
+    for n, cap, idx, nnz in cases:
+        val = rng.normal(0, 1, idx.size).astype(F)
+        val[val == 0] = 1
+        pays.append(make_sparse_payload(n, cap, idx, val, nnz))
+        tensors.append({"compressed": dev(pays[-1]), "out": torch.full((n,), 7.0, device="cuda")})
+    b = hp.Batch("dgc", tensors, ratio=0.001)
+    for rnd in range(3):
+        b.decode()
+        for t, pay, (n, *_rest) in zip(tensors, pays, cases):
+            np.testing.assert_array_equal(host(t["out"]), oracle.sparse_decode(pay, n), err_msg=f"round {rnd} n={n}")
+        # same buffers, new contents: an ordered payload where a disordered one was and the other way round
+        if rnd == 0:
+            for k in (6, 7):
+                n, cap, idx, _ = cases[k]
+                idx2 = np.sort(idx) if k == 6 else rng.permutation(idx).astype(np.int32)
+                val = rng.normal(0, 1, idx2.size).astype(F)
+                pays[k] = make_sparse_payload(n, cap, idx2, val)
+                tensors[k]["compressed"].copy_(dev(pays[k]))
+        for t in tensors:
+            t["out"].fill_(-3.0)
     b.close()
 
 
