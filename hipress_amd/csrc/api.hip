@@ -847,7 +847,8 @@ int hipress_batch_decode(hipress_batch* b, void* stream) {
         case HIPRESS_DGC:
         case HIPRESS_GRADDROP:
             if (++b->epoch == 0) b->epoch = 1;  // the flags start at 0, which no call uses
-            return hiperr(launch_sparse_decode_indexed(L, b->d_tptr, b->d_disorder, b->epoch, st));
+            return hiperr(launch_sparse_decode_indexed(L, b->d_tptr, b->d_disorder, b->epoch,
+                                                       b->params.ratio * kTile <= 8.0, st));
     }
     return HIPRESS_ERR_PARAM;
 }

@@ -161,6 +161,16 @@ __device__ __forceinline__ unsigned valid4(long long e, long long n) {
     return left >= 4 ? 0xfu : (left <= 0 ? 0u : ((1u << left) - 1u));
 }
 
+// ---- workgroup -> tile order ----------------------------------------------------
+// Consecutive workgroup ids are dealt to the eight XCDs in turn, so with the plain
+// order every XCD (and its L2) writes every eighth 16 KiB tile.  Kernels that mostly
+// write do better when an XCD's tiles are neighbours: of every 64 consecutive tiles,
+// XCD x takes tiles 8x .. 8x+7.  The tail that does not fill a group of 64 keeps
+// the plain order.  A permutation of [0, nblocks).
+__device__ __forceinline__ unsigned xcd_grouped(unsigned b, unsigned nblocks) {
+    return b < (nblocks & ~63u) ? ((b & ~63u) | ((b & 7u) << 3) | ((b >> 3) & 7u)) : b;
+}
+
 // ---- cross-lane -------------------------------------------------------------
 // quad_perm broadcast of lane k of every group of four lanes (DPP, no LDS traffic)
 template <int K>
@@ -200,6 +210,16 @@ __device__ __forceinline__ unsigned wave_sum_u(unsigned x) {
     return x;
 }
 #endif  // __HIPCC__
+
+// ---- occupancy caps ----------------------------------------------------------------
+// A launch may ask for dynamic LDS that no kernel touches, only to cap how many
+// workgroups share a CU (160 KiB of LDS each).  The plain streaming kernels move more
+// bytes per second with four or five workgroups per CU than with eight: fewer tiles
+// in flight keep the addresses the memory controllers see closer together.  Kernels
+// with a chain of dependent loads before their stores want every wave they can get
+// and ask for none.  Values chosen per kernel from measurements on MI355X.
+constexpr unsigned kLdsFor5 = 32 * 1024;  // five workgroups per CU
+constexpr unsigned kLdsFor4 = 40 * 1024;  // four
 
 // ---- host-side launch description -----------------------------------------------
 struct Launch {

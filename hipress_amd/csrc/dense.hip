@@ -130,7 +130,7 @@ __device__ __forceinline__ void tbq_decode_tile(const Seg& s, unsigned tile) {
 template <class Src>
 __global__ __launch_bounds__(kBlock) void tbq_decode_kernel(Src src) {
     unsigned tile;
-    const Seg s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, xcd_grouped(blockIdx.x, gridDim.x));
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) tbq_decode_tile<true>(s, tile);
     else tbq_decode_tile<false>(s, tile);
 }
@@ -382,7 +382,7 @@ __device__ __forceinline__ void onebit_decode_tile(const Seg& s, unsigned tile) 
 template <class Src>
 __global__ __launch_bounds__(kBlock) void onebit_decode_kernel(Src src) {
     unsigned tile;
-    const Seg s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, xcd_grouped(blockIdx.x, gridDim.x));
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) onebit_decode_tile<true>(s, tile);
     else onebit_decode_tile<false>(s, tile);
 }
@@ -527,19 +527,24 @@ __global__ __launch_bounds__(kBlock) void terngrad_quant_generic_kernel(Src src)
     if (widx < (long long)((n + 15) >> 4)) words[widx] = myword;
 }
 
-// Decode.  The bucket size comes from the payload header, and with it the place
-// of the packed words behind the scale array; a header that does not fit the
-// buffer decodes to zeros.  BUCKET256 means the bucket size is a multiple of 256,
-// so one step of a wavefront (256 aligned elements) lies inside one bucket.
+// Decode.  The bucket size is in the payload header, and with it the place of the
+// packed words behind the scale array; a header that does not fit the buffer
+// decodes to zeros.  A launch whose host side knows the bucket size (descriptor
+// field `bucket`, with `words_off` already checked against the buffer) starts its
+// loads from that and only compares the header with it afterwards, so the header
+// is not on the path to the first load; on a mismatch the header decides.
+// BUCKET256 means the bucket size is a multiple of 256, so one step of a
+// wavefront (256 aligned elements) lies inside one bucket.
 template <bool FAST, bool BUCKET256>
 __device__ __forceinline__ void terngrad_decode_tile(const Seg& s, unsigned tile, long long B,
-                                                     const uint32_t* words) {
+                                                     const uint32_t* words, bool verify) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long n = (long long)s.n;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
     if (base >= n) return;
     const float* scales = reinterpret_cast<const float*>(s.pay + kHeaderBytes);
     const long long nwords = words ? (n + 15) >> 4 : 0;
+    const uint32_t header_bucket = verify ? reinterpret_cast<const uint32_t*>(s.pay)[1] : 0u;
     unsigned b[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -547,14 +552,25 @@ __device__ __forceinline__ void terngrad_decode_tile(const Seg& s, unsigned tile
         uint32_t w = widx < nwords ? words[widx] : 0u;
         b[j] = (w >> (8 * (lane & 3u))) & 0xffu;
     }
+    float sc4[4] = {0.f, 0.f, 0.f, 0.f};
+    if (BUCKET256) {
+        // one division per wavefront: the four steps start 0, 256, 512, 768 elements
+        // further on and B >= 256, so each step is at most three buckets ahead
+        const long long q0 = base / B, r0 = base - q0 * B;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const long long x = r0 + j * 256;
+            const long long q = q0 + (x >= B) + (x >= 2 * B) + (x >= 3 * B);
+            sc4[j] = (base + j * 256 < n && words) ? scales[q] : 0.f;
+        }
+    }
+    if (verify && header_bucket != (uint32_t)B) return;  // the caller falls back to the header
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         long long e = base + j * 256 + lane * 4;
         f4 o;
         if (BUCKET256) {
-            long long e0 = base + j * 256;
-            float sc = (e0 < n && words) ? scales[e0 / B] : 0.f;
-            o = expand2(b[j], sc);
+            o = expand2(b[j], sc4[j]);
         } else {
             o.x = (e < n && b[j]) ? code_value(b[j] & 3u, scales[e / B]) : 0.f;
             o.y = (e + 1 < n && b[j]) ? code_value((b[j] >> 2) & 3u, scales[(e + 1) / B]) : 0.f;
@@ -582,43 +598,53 @@ template <class Src>
 __global__ __launch_bounds__(kBlock) void terngrad_decode_kernel(Src src) {
     unsigned tile;
     const Seg s = src.get(tile, blockIdx.x);
+    const bool fast = s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n;
+    if (s.bucket && (s.bucket & 255u) == 0) {
+        const uint32_t* words = reinterpret_cast<const uint32_t*>(s.pay + s.words_off);
+        if (fast) terngrad_decode_tile<true, true>(s, tile, s.bucket, words, true);
+        else terngrad_decode_tile<false, true>(s, tile, s.bucket, words, true);
+        if (reinterpret_cast<const uint32_t*>(s.pay)[1] == s.bucket) return;
+    }
     long long B;
     const uint32_t* words = terngrad_words(s.pay, s.pay_bytes, s.n, B);
-    const bool fast = s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n;
     const bool b256 = (B & 255) == 0;
-    if (fast && b256) terngrad_decode_tile<true, true>(s, tile, B, words);
-    else if (b256) terngrad_decode_tile<false, true>(s, tile, B, words);
-    else terngrad_decode_tile<false, false>(s, tile, B, words);
+    if (fast && b256) terngrad_decode_tile<true, true>(s, tile, B, words, false);
+    else if (b256) terngrad_decode_tile<false, true>(s, tile, B, words, false);
+    else terngrad_decode_tile<false, false>(s, tile, B, words, false);
 }
 
 // =============================================================================
 // launchers
 // =============================================================================
 
-#define HP_LAUNCH(KERNEL, L, st, ...)                                                         \
+#define HP_LAUNCH(KERNEL, LDS, L, st, ...)                                                        \
     do {                                                                                      \
         if ((L).ntiles == 0) return hipSuccess;                                               \
         if ((L).single) {                                                                     \
             SingleSrc src{(L).seg};                                                           \
-            hipLaunchKernelGGL((KERNEL<SingleSrc>), dim3((L).ntiles), dim3(kBlock), 0, st, src, \
+            hipLaunchKernelGGL((KERNEL<SingleSrc>), dim3((L).ntiles), dim3(kBlock), LDS, st, src, \
                                ##__VA_ARGS__);                                                \
         } else {                                                                              \
             BatchSrc src{(L).dsegs, (L).dmap};                                                \
-            hipLaunchKernelGGL((KERNEL<BatchSrc>), dim3((L).ntiles), dim3(kBlock), 0, st, src, \
+            hipLaunchKernelGGL((KERNEL<BatchSrc>), dim3((L).ntiles), dim3(kBlock), LDS, st, src, \
                                ##__VA_ARGS__);                                                \
         }                                                                                     \
         return hipGetLastError();                                                             \
     } while (0)
 
-hipError_t launch_tbq_encode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_encode_kernel, L, st); }
-hipError_t launch_tbq_decode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_decode_kernel, L, st); }
-hipError_t launch_onebit_decode(const Launch& L, hipStream_t st) { HP_LAUNCH(onebit_decode_kernel, L, st); }
-hipError_t launch_terngrad_decode(const Launch& L, hipStream_t st) { HP_LAUNCH(terngrad_decode_kernel, L, st); }
+hipError_t launch_tbq_encode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_encode_kernel, kLdsFor5, L, st); }
+hipError_t launch_tbq_decode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_decode_kernel, kLdsFor5, L, st); }
+hipError_t launch_onebit_decode(const Launch& L, hipStream_t st) { HP_LAUNCH(onebit_decode_kernel, kLdsFor5, L, st); }
+// A single-tensor call learns the bucket size from the header on the device, a chain of
+// dependent loads that wants full occupancy; a table launch carries it in the descriptors.
+hipError_t launch_terngrad_decode(const Launch& L, hipStream_t st) {
+    HP_LAUNCH(terngrad_decode_kernel, (L.single ? 0u : kLdsFor5), L, st);
+}
 
 static hipError_t onebit_abs(const Launch& L, float* partial, hipStream_t st) {
-    HP_LAUNCH(onebit_abs_kernel, L, st, partial);
+    HP_LAUNCH(onebit_abs_kernel, kLdsFor4, L, st, partial);
 }
-static hipError_t onebit_quant(const Launch& L, hipStream_t st) { HP_LAUNCH(onebit_quant_kernel, L, st); }
+static hipError_t onebit_quant(const Launch& L, hipStream_t st) { HP_LAUNCH(onebit_quant_kernel, kLdsFor4, L, st); }
 
 static hipError_t onebit_scale(const Launch& L, const float* partial, hipStream_t st) {
     if (L.single) {
@@ -648,7 +674,7 @@ hipError_t launch_onebit_encode(const Launch& L, float* partial, int phase, hipS
 }
 
 static hipError_t onebit_deferred(const Launch& L, float* partial, hipStream_t st) {
-    HP_LAUNCH(onebit_deferred_kernel, L, st, partial);
+    HP_LAUNCH(onebit_deferred_kernel, kLdsFor5, L, st, partial);
 }
 
 // phase < 0: both launches; 0: the fused pass; 1: the scale.
@@ -663,13 +689,13 @@ hipError_t launch_onebit_encode_deferred(const Launch& L, float* partial, int ph
     return hipSuccess;
 }
 
-hipError_t launch_onebit_materialize(const Launch& L, hipStream_t st) { HP_LAUNCH(onebit_materialize_kernel, L, st); }
+hipError_t launch_onebit_materialize(const Launch& L, hipStream_t st) { HP_LAUNCH(onebit_materialize_kernel, kLdsFor5, L, st); }
 
 template <class Src>
 static hipError_t terngrad_encode_src(const Src& src, unsigned ntiles, unsigned bucket, hipStream_t st) {
-    if (bucket == 256) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 4>), dim3(ntiles), dim3(kBlock), 0, st, src);
-    else if (bucket == 512) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 2>), dim3(ntiles), dim3(kBlock), 0, st, src);
-    else if (bucket == 1024) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 1>), dim3(ntiles), dim3(kBlock), 0, st, src);
+    if (bucket == 256) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 4>), dim3(ntiles), dim3(kBlock), kLdsFor5, st, src);
+    else if (bucket == 512) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 2>), dim3(ntiles), dim3(kBlock), kLdsFor5, st, src);
+    else if (bucket == 1024) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 1>), dim3(ntiles), dim3(kBlock), kLdsFor5, st, src);
     else {
         hipLaunchKernelGGL((terngrad_scale_generic_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);
         hipLaunchKernelGGL((terngrad_quant_generic_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);

@@ -33,7 +33,7 @@ struct SparseWs {
 hipError_t launch_sparse_encode(const Launch& L, bool dgc, const SparseWs& ws, int phase, hipStream_t st);
 hipError_t launch_sparse_decode(const Launch& L, hipStream_t st);
 hipError_t launch_sparse_decode_indexed(const Launch& L, uint32_t* tptr, uint32_t* disorder, unsigned epoch,
-                                        hipStream_t st);
+                                        bool few_pairs, hipStream_t st);
 constexpr int kSparseAfterAccum = 100;  // launch_sparse_encode phase: everything after the accumulate launch
 hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, uint32_t* tileptr, uint32_t* unsorted,
                                int phase, hipStream_t st);

@@ -675,7 +675,7 @@ __device__ __forceinline__ void zero_tile(float* out, long long n, unsigned tile
 template <class Src>
 __global__ __launch_bounds__(kBlock) void zero_fill_kernel(Src src) {
     unsigned tile;
-    const Seg s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, xcd_grouped(blockIdx.x, gridDim.x));
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) zero_tile<true>(s.out, (long long)s.n, tile);
     else zero_tile<false>(s.out, (long long)s.n, tile);
 }
@@ -800,7 +800,7 @@ __global__ __launch_bounds__(kBlock) void sparse_decode_tile_kernel(Src src, con
                                                                     const uint32_t* disorder, unsigned epoch) {
     __shared__ __attribute__((aligned(16))) float lds[kTile];
     unsigned tile;
-    const Seg s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, xcd_grouped(blockIdx.x, gridDim.x));
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long n = (long long)s.n;
     const long long t_lo = (long long)tile * kTile, t_hi = t_lo + kTile < n ? t_lo + kTile : n;
@@ -993,7 +993,7 @@ static hipError_t sparse_encode_src(const Src& src, const Src& ssrc_tiles, const
     const unsigned g4 = (ntiles + 3) / 4;
     if (on(0)) {
         if (dgc) hipLaunchKernelGGL((sparse_accum_kernel<Src, true>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
-        else hipLaunchKernelGGL((sparse_accum_kernel<Src, false>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
+        else hipLaunchKernelGGL((sparse_accum_kernel<Src, false>), dim3(ntiles), dim3(kBlock), kLdsFor4, st, src, ws);
     }
     for (int pass = 0; pass < 3; ++pass)
         if (on(1 + pass) && nstiles)
@@ -1019,12 +1019,12 @@ hipError_t launch_sparse_decode(const Launch& L, hipStream_t st) {
     if (L.ntiles == 0) return hipSuccess;
     if (L.single) {
         SingleSrc src{L.seg};
-        hipLaunchKernelGGL((zero_fill_kernel<SingleSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
+        hipLaunchKernelGGL((zero_fill_kernel<SingleSrc>), dim3(L.ntiles), dim3(kBlock), kLdsFor5, st, src);
         if (L.seg.ncblk)
             hipLaunchKernelGGL((sparse_scatter_kernel<SingleSrc>), dim3(L.seg.ncblk), dim3(kBlock), 0, st, src);
     } else {
         BatchSrc src{L.dsegs, L.dmap};
-        hipLaunchKernelGGL((zero_fill_kernel<BatchSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src);
+        hipLaunchKernelGGL((zero_fill_kernel<BatchSrc>), dim3(L.ntiles), dim3(kBlock), kLdsFor5, st, src);
         BatchSrc csrc{L.dsegs, L.dcmap};
         if (L.nctiles)
             hipLaunchKernelGGL((sparse_scatter_kernel<BatchSrc>), dim3(L.nctiles), dim3(kBlock), 0, st, csrc);
@@ -1034,16 +1034,19 @@ hipError_t launch_sparse_decode(const Launch& L, hipStream_t st) {
 
 // Decode of a tensor table through tile pointers: tptr has one word per tile of the
 // launch, disorder one word per tensor; epoch must differ from call to call.
+// few_pairs: most tiles receive no or a handful of pairs, so the tile kernel is a plain
+// stream of stores and runs with the occupancy cap of one; with tens of pairs per tile
+// every workgroup waits on a chain of loads first and the cap would cost throughput.
 hipError_t launch_sparse_decode_indexed(const Launch& L, uint32_t* tptr, uint32_t* disorder, unsigned epoch,
-                                        hipStream_t st) {
+                                        bool few_pairs, hipStream_t st) {
     if (L.ntiles == 0 || L.single) return hipSuccess;
     BatchSrc csrc{L.dsegs, L.dcmap};
     if (L.nctiles)
         hipLaunchKernelGGL((sparse_decode_index_kernel<BatchSrc>), dim3(L.nctiles), dim3(kBlock), 0, st, csrc, tptr,
                            disorder, epoch);
     BatchSrc src{L.dsegs, L.dmap};
-    hipLaunchKernelGGL((sparse_decode_tile_kernel<BatchSrc>), dim3(L.ntiles), dim3(kBlock), 0, st, src, tptr, disorder,
-                       epoch);
+    hipLaunchKernelGGL((sparse_decode_tile_kernel<BatchSrc>), dim3(L.ntiles), dim3(kBlock),
+                       few_pairs ? kLdsFor4 - 4 * kTile : 0u, st, src, tptr, disorder, epoch);
     if (L.nctiles)
         hipLaunchKernelGGL(sparse_scatter_if_disordered_kernel, dim3(L.nctiles), dim3(kBlock), 0, st, csrc, disorder,
                            epoch);

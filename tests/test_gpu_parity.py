@@ -532,6 +532,28 @@ def test_sparse_batch_many_steps(hp, alg, ratio):
     b.close()
 
 
+def test_terngrad_batch_decode_follows_the_header_bucket(hp):
+    """A batch is created with one bucket size, and its decoder starts from it; a payload
+    whose header names another bucket size must still be decoded by its header."""
+    rng = np.random.default_rng(5)
+    sizes = [100000, 4097, 70000]
+    tensors, pays = [], []
+    for k, n in enumerate(sizes):
+        g = rng.normal(0, 1e-2, n).astype(F)
+        u = rng.random(n, dtype=F)
+        bucket = 256 if k == 1 else 512  # the middle payload disagrees with the batch
+        pays.append(oracle.terngrad_encode(g, u, bucket))
+        room = max(hp.terngrad_payload_bytes(n, 256), hp.terngrad_payload_bytes(n, 512))
+        buf = torch.zeros(room, dtype=torch.uint8, device="cuda")
+        buf[: pays[-1].size].copy_(dev(pays[-1]))
+        tensors.append({"compressed": buf, "out": torch.full((n,), 7.0, device="cuda")})
+    b = hp.Batch("terngrad", tensors, bucket=512)
+    b.decode()
+    for t, pay, n in zip(tensors, pays, sizes):
+        np.testing.assert_array_equal(host(t["out"]), oracle.terngrad_decode(pay, n), err_msg=f"n={n}")
+    b.close()
+
+
 def make_sparse_payload(n, cap, idx, val, nnz=None):
     """A hand-made dgc/graddrop payload: header {nnz, n, cap, thr}, idx[cap], val[cap]."""
     pay = np.zeros(16 + 8 * cap, np.uint8)
