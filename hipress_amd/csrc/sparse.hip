@@ -900,7 +900,7 @@ __global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs
     __shared__ __attribute__((aligned(16))) float lds[kTile];
     __shared__ unsigned plo[kMaxPeers], pcnt[kMaxPeers], pcap[kMaxPeers];
     unsigned tile;
-    const MergeSeg& m = src.get(tile, blockIdx.x);
+    const MergeSeg& m = src.get(tile, xcd_grouped(blockIdx.x, gridDim.x));
     const Seg s = m.s;
     const Seg r = m.r;  // re-encode descriptor of this chunk: same tile numbering
     const long long n = (long long)s.n;
