@@ -206,14 +206,25 @@ __global__ __launch_bounds__(kBlock) void sparse_select_kernel(Src src, SparseWs
         }
     }
     __syncthreads();
-    for (unsigned i = threadIdx.x; i < nb; i += kBlock) {
-        unsigned c = lh[i];
-        if (c) atomicAdd(&gh[i], c);
+    unsigned was[kBins / kBlock];  // what the adds return; all are issued before any is waited for
+#pragma unroll
+    for (int q = 0; q < kBins / kBlock; ++q) {
+        const unsigned i = q * kBlock + threadIdx.x;
+        const unsigned c = i < nb ? lh[i] : 0u;
+        was[q] = 0;
+        if (c) was[q] = atomicAdd(&gh[i], c);
     }
+    unsigned seen = 0;
+#pragma unroll
+    for (int q = 0; q < kBins / kBlock; ++q) seen |= was[q];
     // Everything workgroups exchange here travels through device-scope atomics
     // (the histogram adds above, the ticket below, the atomic loads after it), so
-    // no cache write-back is needed: the barrier waits until this workgroup's
-    // adds have been performed, and only then is its ticket taken.
+    // no cache write-back is needed.  The ticket may only be taken once this
+    // workgroup's adds have been performed where all XCDs meet.  An add without a
+    // result counts as done when the local L2 has accepted it, which is too early;
+    // one whose result is waited for has been performed, so the results are kept
+    // alive up to the barrier.
+    asm volatile("" ::"v"(seen));
     __syncthreads();
     if (threadIdx.x == 0) is_last = atomicAdd(&ctl[kCtlDone + pass], 1u) == s.nsblk - 1;
     __syncthreads();

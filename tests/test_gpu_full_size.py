@@ -131,6 +131,37 @@ def test_dgc_bert_large_full_set_properties(hp):
     b.close()
 
 
+def test_graddrop_150m_elements_three_steps(hp):
+    """One tensor of 150,000,000 elements (36,622 tiles, 367 workgroups in every threshold
+    pass), three steps against the oracle: with this many workgroups a threshold pass that
+    lets its last workgroup read the histogram before every other one's adds have landed
+    picks a key a few ranks off."""
+    n, ratio = 150_000_000, 0.01
+    gen = torch.Generator(device="cuda").manual_seed(17)
+    acc = torch.zeros(n, device="cuda")
+    pay = torch.zeros(hp.graddrop_payload_bytes(n, ratio), dtype=torch.uint8, device="cuda")
+    out = torch.empty(n, device="cuda")
+    g = torch.empty(n, device="cuda")
+    b = hp.Batch("graddrop", [{"gradient": g, "accumulator": acc, "compressed": pay, "out": out}], ratio=ratio)
+    ref_acc = np.zeros(n, F)
+    for step in range(3):
+        g.normal_(0, 1e-3, generator=gen)
+        b.encode()
+        b.decode()
+        want, ref_acc = oracle.graddrop_encode(host(g), ref_acc, ratio)
+        got = host(pay)
+        nnz, _, cap, thr, idx, val = oracle.sparse_unpack(got)
+        w = oracle.sparse_unpack(want)
+        assert (nnz, cap) == (w[0], w[2]) and thr.view(np.uint32) == w[3].view(np.uint32), f"step {step}"
+        np.testing.assert_array_equal(idx, w[4])
+        np.testing.assert_array_equal(val, w[5])
+        np.testing.assert_array_equal(host(acc), ref_acc)
+        o = host(out)
+        assert np.count_nonzero(o) == nnz
+        np.testing.assert_array_equal(o[idx], val)
+    b.close()
+
+
 def test_merge_vgg19_chunks_tbq(hp):
     """configs[4], TBQ half: 8 peers x 168 chunks of at most 4 MB, decode-and-merge with the
     fused re-encode; oracle comparison on a sample of chunks, identities on all."""
