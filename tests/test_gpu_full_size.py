@@ -198,6 +198,71 @@ def test_merge_vgg19_chunks_tbq(hp):
     mb.close()
 
 
+def test_graddrop_vgg19_full_set_three_steps(hp):
+    """GradDrop 1 % over the 38 VGG19 tensors (143,667,240 elements), three steps, every
+    tensor against the oracle: payload, accumulator and decoded gradient."""
+    from hipress_amd import workloads as W
+
+    sizes = W.vgg19_sizes()
+    dev = torch.device("cuda:0")
+    ratio = 0.01
+    ts = [{"gradient": torch.empty(n, device=dev), "accumulator": torch.zeros(n, device=dev),
+           "out": torch.empty(n, device=dev),
+           "compressed": torch.zeros(hp.graddrop_payload_bytes(n, ratio), dtype=torch.uint8, device=dev)} for n in sizes]
+    b = hp.Batch("graddrop", ts, ratio=ratio)
+    refs = [np.zeros(n, F) for n in sizes]
+    for step in range(3):
+        for t, g in zip(ts, W.normal_set(sizes, dev, 100 + step, log_sigma_range=(-4.0, -2.0))):
+            t["gradient"].copy_(g)
+        b.encode()
+        b.decode()
+        for i, (t, n) in enumerate(zip(ts, sizes)):
+            want, refs[i] = oracle.graddrop_encode(host(t["gradient"]), refs[i], ratio)
+            np.testing.assert_array_equal(host(t["compressed"])[:16], want[:16], err_msg=f"header, step {step} tensor {i}")
+            got = oracle.sparse_unpack(host(t["compressed"]))
+            w = oracle.sparse_unpack(want)
+            np.testing.assert_array_equal(got[4], w[4], err_msg=f"indices, step {step} tensor {i}")
+            np.testing.assert_array_equal(got[5], w[5], err_msg=f"values, step {step} tensor {i}")
+            np.testing.assert_array_equal(host(t["accumulator"]), refs[i], err_msg=f"accumulator, step {step} tensor {i}")
+            np.testing.assert_array_equal(host(t["out"]), oracle.sparse_decode(want, n), err_msg=f"decode, step {step} tensor {i}")
+    b.close()
+
+
+def test_merge_vgg19_chunks_dgc(hp):
+    """configs[4], DGC half: 8 peers x 168 chunks, sparse decode-and-merge with the GradDrop-style
+    re-encode of the aggregate; two rounds on the same batch object, every chunk against the oracle."""
+    from hipress_amd import workloads as W
+
+    sizes = W.chunk_sizes(W.vgg19_sizes())
+    dev = torch.device("cuda:0")
+    ratio, P = 0.001, 8
+    chunks = [{"compressed": [torch.zeros(hp.dgc_payload_bytes(n, ratio), dtype=torch.uint8, device=dev) for _ in range(P)],
+               "aggregate": torch.empty(n, device=dev), "state": torch.zeros(n, device=dev),
+               "out_compressed": torch.zeros(hp.dgc_payload_bytes(n, ratio), dtype=torch.uint8, device=dev)} for n in sizes]
+    mb = hp.MergeBatch("dgc", chunks, ratio=ratio)
+    ref_acc = [np.zeros(n, F) for n in sizes]
+    for rnd in range(2):
+        for p in range(P):
+            grads = W.normal_set(sizes, dev, 10 * rnd + p + 1, sigma=1e-3)
+            enc = hp.Batch("dgc", [{"gradient": g, "momentum": torch.zeros_like(g), "accumulator": torch.zeros_like(g),
+                                    "compressed": c["compressed"][p]} for g, c in zip(grads, chunks)],
+                           momentum_factor=0.9, ratio=ratio)
+            enc.encode()
+            torch.cuda.synchronize()
+            enc.close()
+        mb.run()
+        for i, (c, n) in enumerate(zip(chunks, sizes)):
+            pays = [host(q) for q in c["compressed"]]
+            agg, out, ref_acc[i] = oracle.sparse_decode_merge(pays, n, ref_acc[i], ratio)
+            np.testing.assert_array_equal(host(c["aggregate"]), agg, err_msg=f"aggregate, round {rnd} chunk {i}")
+            np.testing.assert_array_equal(host(c["out_compressed"])[:16], out[:16], err_msg=f"header, round {rnd} chunk {i}")
+            got, w = oracle.sparse_unpack(host(c["out_compressed"])), oracle.sparse_unpack(out)
+            np.testing.assert_array_equal(got[4], w[4], err_msg=f"indices, round {rnd} chunk {i}")
+            np.testing.assert_array_equal(got[5], w[5], err_msg=f"values, round {rnd} chunk {i}")
+            np.testing.assert_array_equal(host(c["state"]), ref_acc[i], err_msg=f"accumulator, round {rnd} chunk {i}")
+    mb.close()
+
+
 def test_hip_graph_replay_matches_eager(hp):
     """encode + decode enqueue only kernels (no allocation, no host synchronisation),
     so they can be captured in a HIP graph; every replay must equal the eager result."""
