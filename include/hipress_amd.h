@@ -181,7 +181,12 @@ int hipress_sparse_decode_merge(const void *const *payloads, const int64_t *payl
 /* A training step compresses every tensor of the model; a batch object holds a
  * device-resident table of the tensors so that one launch sequence covers all of
  * them (the per-tensor calls cost one launch sequence each).  Fields a given
- * algorithm does not use may be NULL. */
+ * algorithm does not use may be NULL.  A batch owns scratch memory on the device, so
+ * calls on one batch must not overlap (one stream, or ordered by events); distinct
+ * batches are independent.  All calls only enqueue kernels: they may be captured in a
+ * HIP graph.  The sparse decode passes a per-call counter to its kernels, which a graph
+ * freezes: in replays a tensor whose payload was once found out of order keeps taking
+ * the slower scatter path (results stay correct). */
 typedef struct hipress_tensor {
     const float *grad;    /* encode input, fp32[n] */
     float *state0;        /* residual (onebit, tbq) | momentum (dgc) | accumulator (graddrop) */

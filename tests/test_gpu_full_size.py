@@ -297,3 +297,52 @@ def test_hip_graph_replay_matches_eager(hp):
         np.testing.assert_array_equal(host(pay), eager[step][0], err_msg=f"payload, replay {step}")
         np.testing.assert_array_equal(host(r), eager[step][1], err_msg=f"residual, replay {step}")
         np.testing.assert_array_equal(host(out), eager[step][2], err_msg=f"decode, replay {step}")
+
+
+def test_hip_graph_replay_of_a_sparse_batch(hp):
+    """The batched DGC encode + decode (ten launches, idle dynamic LDS on some, a per-call
+    counter in the decode) captured once and replayed: every replay equals the eager run
+    that started from the same state."""
+    sizes = [1000003, 262144, 4097]
+    ratio, m = 0.001, 0.9
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    grads = [torch.randn(n, device="cuda", generator=gen) * 1e-3 for n in sizes]
+
+    def make():
+        return [{"gradient": g, "momentum": torch.zeros_like(g), "accumulator": torch.zeros_like(g),
+                 "out": torch.empty_like(g),
+                 "compressed": torch.zeros(hp.dgc_payload_bytes(g.numel(), ratio), dtype=torch.uint8, device="cuda")}
+                for g in grads]
+
+    eager_ts = make()
+    eb = hp.Batch("dgc", eager_ts, momentum_factor=m, ratio=ratio)
+    eager = []
+    for _ in range(3):
+        eb.encode()
+        eb.decode()
+        eager.append([(host(t["compressed"]).copy(), host(t["accumulator"]).copy(), host(t["out"]).copy()) for t in eager_ts])
+    eb.close()
+    ts = make()
+    b = hp.Batch("dgc", ts, momentum_factor=m, ratio=ratio)
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        b.encode()  # warm-up on the capture stream, then back to the initial state
+        b.decode()
+        stream.synchronize()
+        for t in ts:
+            t["momentum"].zero_()
+            t["accumulator"].zero_()
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            b.encode()
+            b.decode()
+    for step in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        _ = (ts[0]["out"] * 2).sum().item()  # unrelated eager work between replays
+        for t, (pay, acc, out) in zip(ts, eager[step]):
+            np.testing.assert_array_equal(host(t["compressed"]), pay, err_msg=f"payload, replay {step}")
+            np.testing.assert_array_equal(host(t["accumulator"]), acc, err_msg=f"accumulator, replay {step}")
+            np.testing.assert_array_equal(host(t["out"]), out, err_msg=f"decode, replay {step}")
+    b.close()
