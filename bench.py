@@ -237,8 +237,8 @@ class CompllWorkload:
     """The in-tree CompLL operator (bit width 2, 10-byte header) on the largest VGG19
     tensor through the per-tensor entry points."""
 
-    def __init__(self, name, n, bitwidth=2):
-        self.name, self.sizes, self.elements, self.b = name, [n], n, bitwidth
+    def __init__(self, name, n, bitwidth=2, generated=False):
+        self.name, self.sizes, self.elements, self.b, self.generated = name, [n], n, bitwidth, generated
         self.enc_bytes, self.dec_bytes = 8.0 + bitwidth / 8.0, 4.0 + bitwidth / 8.0
         self.dominant_kernel, self.dominant_bytes = "compll_quant_kernel", 8.0 + bitwidth / 8.0
 
@@ -253,10 +253,18 @@ class CompllWorkload:
         self.u = W.uniform_set(self.sizes, dev, 1000)[0]
         self.pay = torch.zeros(hp.compll_payload_bytes(self.elements, self.b), dtype=torch.uint8, device=dev)
         self.out = torch.empty(self.elements, device=dev)
+        if self.generated:
+            from hipress_amd.compll import runtime
+
+            self.gen = runtime.load()
 
     def step(self, ev=None):
-        self.hp.compll_terngrad_encode(self.g, self.u, self.pay, self.b)
-        self.hp.compll_terngrad_decode(self.pay, self.out)
+        if self.generated:  # the same operator, generated from its program in the CompLL language
+            self.gen.MinMaxQuantEncode(self.g, self.pay, self.b, uniform=self.u)
+            self.gen.MinMaxQuantDecode(self.pay, self.out)
+        else:
+            self.hp.compll_terngrad_encode(self.g, self.u, self.pay, self.b)
+            self.hp.compll_terngrad_decode(self.pay, self.out)
 
     def close(self):
         self.g = self.u = self.pay = self.out = None
@@ -296,6 +304,8 @@ def make_workload(name):
         return SetWorkload(name, "graddrop", bert, "n1e-3", {"ratio": 0.01}, 12.0, 4.0, 0, "sparse_accum_kernel", 12.0, nphases=7)
     if name == "compll_b2_fc6":
         return CompllWorkload(name, max(vgg))
+    if name == "compll_generated_b2_fc6":
+        return CompllWorkload(name, max(vgg), generated=True)
     if name == "merge_tbq_vgg19":
         return MergeWorkload(name, "tbq", W.chunk_sizes(vgg))
     if name == "merge_dgc_vgg19":
@@ -306,6 +316,7 @@ def make_workload(name):
 ALL_WORKLOADS = [
     "onebit_vgg19", "onebit_deferred_vgg19", "tbq_vgg19", "terngrad_vgg19", "dgc_vgg19", "graddrop_vgg19", "tbq_262144", "tbq_262144_x512",
     "terngrad_resnet50", "dgc_bert_large", "graddrop_bert_large", "merge_tbq_vgg19", "merge_dgc_vgg19", "compll_b2_fc6",
+    "compll_generated_b2_fc6",
 ]
 
 

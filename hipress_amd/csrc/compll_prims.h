@@ -1,0 +1,343 @@
+// Primitive library for operators generated from the CompLL operator language
+// (hipress_amd/compll): the device-side pieces every generated operator is put
+// together from, written for gfx950.  It takes the place of the Thrust calls
+// the reference's generator emits (thrust::reduce / thrust::transform /
+// thrust::copy in /root/reference/src/CompLL/GCGen/output/TernGradEncode/
+// TernGradEncode_body.h:110-125), with three differences that matter on this
+// hardware: several folds over the same vector share one sweep, scalars that
+// come out of a reduction or a payload header stay on the device (no host
+// round trip between launches), and packed codes are produced in place behind
+// the header instead of in a temporary that is copied.
+//
+// Conventions.  A generated operator has a struct of host-known values (`Args`,
+// passed to every kernel by value) and a struct of device-computed scalars
+// (`Dev`, in the caller's workspace).  The user-written lambdas become static
+// member functions of small structs that take both.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace cl {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+constexpr int kBlock = 256;   // threads per workgroup (four wave64 wavefronts)
+constexpr int kTile = 4096;   // elements per workgroup in the sweeps
+constexpr int kFinalBlock = 1024;
+
+// ---- packed codes ---------------------------------------------------------------
+// uint<bits> vectors live in bytes: code i at bit (i mod 8/bits)*bits of byte
+// floor(i*bits/8), the placement the reference's decoder reads
+// (/root/reference/src/CompLL/GCGen/output/TernGradDecode/TernGradDecode_body.h:44).
+// bits is one of 1, 2, 4, 8.
+__device__ __forceinline__ bool valid_bits(int bits) { return bits == 1 || bits == 2 || bits == 4 || bits == 8; }
+
+__device__ __forceinline__ int log2_per_byte(int bits) { return bits == 1 ? 3 : (bits == 2 ? 2 : (bits == 4 ? 1 : 0)); }
+
+__device__ __forceinline__ unsigned get_code(const uint8_t* bytes, long long i, int bits) {
+    const int sh = log2_per_byte(bits);
+    return ((unsigned)bytes[i >> sh] >> ((int)(i & ((1 << sh) - 1)) * bits)) & ((1u << bits) - 1u);
+}
+
+// Conversion of a computed value to uint<bits>: saturating, NaN gives 0.
+__device__ __forceinline__ unsigned to_code(float x, int bits) {
+    const float top = (float)((1u << bits) - 1u);
+    return x >= top ? (unsigned)top : (x > 0.f ? (unsigned)x : 0u);
+}
+__device__ __forceinline__ unsigned to_code(long long x, int bits) {
+    const long long top = (1ll << bits) - 1;
+    return (unsigned)(x < 0 ? 0 : (x > top ? top : x));
+}
+__device__ __forceinline__ unsigned to_code(int x, int bits) { return to_code((long long)x, bits); }
+__device__ __forceinline__ unsigned to_code(unsigned x, int bits) { return to_code((long long)x, bits); }
+
+// ---- header fields at any byte offset ----------------------------------------------
+template <class T>
+__device__ __forceinline__ void put(uint8_t* p, T v) {
+    uint8_t raw[sizeof(T)];
+    __builtin_memcpy(raw, &v, sizeof(T));
+    for (unsigned k = 0; k < sizeof(T); ++k) p[k] = raw[k];
+}
+template <class T>
+__device__ __forceinline__ T get(const uint8_t* p) {
+    uint8_t raw[sizeof(T)];
+    for (unsigned k = 0; k < sizeof(T); ++k) raw[k] = p[k];
+    T v;
+    __builtin_memcpy(&v, raw, sizeof(T));
+    return v;
+}
+
+// ---- rounding noise -------------------------------------------------------------------
+// random<float>(lo, hi) of the language reads an explicit uniform[0,1) tensor at
+// the element being mapped, so that an operator is a function of its inputs.
+__device__ __forceinline__ float uniform_from(float u, float lo, float hi) { return lo + (hi - lo) * u; }
+__device__ __forceinline__ float uniform_draw(const float* u, long long i, float lo, float hi) {
+    return uniform_from(u[i], lo, hi);
+}
+
+// ---- serial block ------------------------------------------------------------------------
+// Scalar statements that depend on device values (and header reads / writes) run
+// in one thread between the sweeps.
+template <class Args, class Dev, class Body>
+__global__ void serial_kernel(Args a, Dev* d) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) Body::run(a, *d);
+}
+
+// ---- reduce --------------------------------------------------------------------------------
+// Folds::K folds over one float vector in one sweep.  Folds provides
+//   static float init(const Args&, const Dev&, int k)
+//   static float apply(const Args&, const Dev&, int k, float acc, float x)   (the user's lambda)
+//   static void  store(Dev&, int k, float value)
+// reduce(v, init, f) is f folded over init and the elements; as in any parallel
+// reduce f has to be associative and commutative, and the order in which elements
+// meet is this kernel's business.  init enters exactly once, at the very end, so f
+// need not be idempotent in it (a sum with a non-zero init stays correct).
+template <class Args, class Dev, class Folds>
+__global__ __launch_bounds__(kBlock) void reduce_tiles_kernel(Args a, const Dev* d, const float* v, long long n,
+                                                              float* partial) {
+    __shared__ float wave_acc[4][Folds::K];
+    __shared__ int wave_any[4];
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long base = (long long)blockIdx.x * kTile + wave * 1024;
+    const bool vec_ok = (reinterpret_cast<uintptr_t>(v) & 15u) == 0;
+    f4 x[4];
+    unsigned ok[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const long long e = base + j * 256 + lane * 4;
+        const long long left = n - e;
+        ok[j] = left >= 4 ? 0xfu : (left <= 0 ? 0u : ((1u << left) - 1u));
+        if (ok[j] == 0xfu && vec_ok) {
+            x[j] = __builtin_nontemporal_load(reinterpret_cast<const f4*>(v + e));
+        } else {
+            x[j].x = (ok[j] & 1u) ? v[e] : 0.f;
+            x[j].y = (ok[j] & 2u) ? v[e + 1] : 0.f;
+            x[j].z = (ok[j] & 4u) ? v[e + 2] : 0.f;
+            x[j].w = (ok[j] & 8u) ? v[e + 3] : 0.f;
+        }
+    }
+    float acc[Folds::K];
+    bool any;  // whether acc holds at least one element yet
+    if ((long long)(blockIdx.x + 1) * kTile <= n) {
+        // a full tile: every lane has all sixteen elements, nothing to keep track of
+#pragma unroll
+        for (int k = 0; k < Folds::K; ++k) acc[k] = x[0].x;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float xs[4] = {x[j].x, x[j].y, x[j].z, x[j].w};
+#pragma unroll
+            for (int c = (j == 0 ? 1 : 0); c < 4; ++c)
+#pragma unroll
+                for (int k = 0; k < Folds::K; ++k) acc[k] = Folds::apply(a, *d, k, acc[k], xs[c]);
+        }
+#pragma unroll
+        for (int m = 1; m < 64; m <<= 1)
+#pragma unroll
+            for (int k = 0; k < Folds::K; ++k) acc[k] = Folds::apply(a, *d, k, acc[k], __shfl_xor(acc[k], m, 64));
+        any = true;
+    } else {
+#pragma unroll
+        for (int k = 0; k < Folds::K; ++k) acc[k] = 0.f;
+        any = false;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float xs[4] = {x[j].x, x[j].y, x[j].z, x[j].w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const bool have = (ok[j] >> c) & 1u;
+#pragma unroll
+                for (int k = 0; k < Folds::K; ++k)
+                    acc[k] = have ? (any ? Folds::apply(a, *d, k, acc[k], xs[c]) : xs[c]) : acc[k];
+                any = any || have;
+            }
+        }
+#pragma unroll
+        for (int m = 1; m < 64; m <<= 1) {
+            const bool other_any = __shfl_xor((int)any, m, 64) != 0;
+#pragma unroll
+            for (int k = 0; k < Folds::K; ++k) {
+                const float other = __shfl_xor(acc[k], m, 64);
+                acc[k] = (any && other_any) ? Folds::apply(a, *d, k, acc[k], other) : (any ? acc[k] : other);
+            }
+            any = any || other_any;
+        }
+    }
+    if (lane == 0) {
+        wave_any[wave] = any;
+#pragma unroll
+        for (int k = 0; k < Folds::K; ++k) wave_acc[wave][k] = acc[k];
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {  // the first wavefront of a launched tile always holds an element
+        float t[Folds::K];
+#pragma unroll
+        for (int k = 0; k < Folds::K; ++k) t[k] = wave_acc[0][k];
+        for (int w = 1; w < 4; ++w)
+            if (wave_any[w]) {
+#pragma unroll
+                for (int k = 0; k < Folds::K; ++k) t[k] = Folds::apply(a, *d, k, t[k], wave_acc[w][k]);
+            }
+#pragma unroll
+        for (int k = 0; k < Folds::K; ++k) partial[(long long)blockIdx.x * Folds::K + k] = t[k];
+    }
+}
+
+// One workgroup folds the per-tile results (every tile of a launch holds at least
+// one element), combines them with the initial values and stores the K results.
+// With no tile at all the results are the initial values.
+struct Nothing {
+    template <class Args, class Dev>
+    static __device__ void run(const Args&, Dev&) {}
+};
+
+// After::run: the scalar statements that follow the reduce in the program, if any.
+template <class Args, class Dev, class Folds, class After>
+__global__ __launch_bounds__(kFinalBlock) void reduce_final_kernel(Args a, Dev* d, const float* partial, unsigned ntiles) {
+    __shared__ float sh[kFinalBlock][Folds::K];
+    __shared__ int sh_any[kFinalBlock];
+    float acc[Folds::K];
+#pragma unroll
+    for (int k = 0; k < Folds::K; ++k) acc[k] = 0.f;
+    bool any = false;
+    for (unsigned t = threadIdx.x; t < ntiles; t += kFinalBlock) {
+#pragma unroll
+        for (int k = 0; k < Folds::K; ++k) {
+            const float p = partial[(long long)t * Folds::K + k];
+            acc[k] = any ? Folds::apply(a, *d, k, acc[k], p) : p;
+        }
+        any = true;
+    }
+    sh_any[threadIdx.x] = any;
+#pragma unroll
+    for (int k = 0; k < Folds::K; ++k) sh[threadIdx.x][k] = acc[k];
+    __syncthreads();
+    for (int w = kFinalBlock / 2; w >= 1; w >>= 1) {
+        if ((int)threadIdx.x < w && sh_any[threadIdx.x + w]) {
+#pragma unroll
+            for (int k = 0; k < Folds::K; ++k)
+                sh[threadIdx.x][k] = sh_any[threadIdx.x] ? Folds::apply(a, *d, k, sh[threadIdx.x][k], sh[threadIdx.x + w][k])
+                                                         : sh[threadIdx.x + w][k];
+            sh_any[threadIdx.x] = 1;
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 0; k < Folds::K; ++k) {
+            const float init = Folds::init(a, *d, k);
+            Folds::store(*d, k, sh_any[0] ? Folds::apply(a, *d, k, init, sh[0][k]) : init);
+        }
+        After::run(a, *d);
+    }
+}
+
+// ---- map ---------------------------------------------------------------------------------------
+// Fn describes the mapped lambda:
+//   count(a, d)              length of the range
+//   NS, stream(a, k)         the float vectors the lambda reads at its own index (its
+//                            random draws among them); the kernel loads them as 16-byte
+//                            vectors, whole rows per wavefront, and hands the lambda values
+//   call(a, d, i, s)         the lambda; s[k] is the element of stream k at index i
+//   bits(a, d)               (packed maps) width of the codes
+// A lane owns four consecutive indices of each of four rows of 256, as in the other
+// operators of this library.
+
+template <class Args, class Fn>
+__device__ __forceinline__ void load_streams(const Args& a, long long base, long long count, f4 (&x)[Fn::NS > 0 ? Fn::NS : 1][4]) {
+#pragma unroll
+    for (int k = 0; k < Fn::NS; ++k) {
+        const float* p = Fn::stream(a, k);
+        const bool vec_ok = (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const long long e = base + j * 256;
+            if (e + 3 < count && vec_ok) {
+                x[k][j] = __builtin_nontemporal_load(reinterpret_cast<const f4*>(p + e));
+            } else {
+                x[k][j].x = e < count ? p[e] : 0.f;
+                x[k][j].y = e + 1 < count ? p[e + 1] : 0.f;
+                x[k][j].z = e + 2 < count ? p[e + 2] : 0.f;
+                x[k][j].w = e + 3 < count ? p[e + 3] : 0.f;
+            }
+        }
+    }
+}
+
+// out[i] = Fn::call(...) for i < min(count, cap).
+template <class Args, class Dev, class Fn>
+__global__ __launch_bounds__(kBlock) void map_float_kernel(Args a, const Dev* d, float* out, long long cap) {
+    long long count = Fn::count(a, *d);
+    if (count > cap) count = cap;
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long base = (long long)blockIdx.x * kTile + wave * 1024 + lane * 4;
+    const bool vec_ok = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
+    f4 x[Fn::NS > 0 ? Fn::NS : 1][4];
+    load_streams<Args, Fn>(a, base, count, x);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const long long e = base + j * 256;
+        float s[4][Fn::NS > 0 ? Fn::NS : 1];
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int k = 0; k < Fn::NS; ++k) s[c][k] = x[k][j][c];
+        if (e + 3 < count && vec_ok) {  // the common case carries no per-element test
+            f4 q;
+            q.x = Fn::call(a, *d, e, s[0]);
+            q.y = Fn::call(a, *d, e + 1, s[1]);
+            q.z = Fn::call(a, *d, e + 2, s[2]);
+            q.w = Fn::call(a, *d, e + 3, s[3]);
+            __builtin_nontemporal_store(q, reinterpret_cast<f4*>(out + e));
+        } else {
+            for (int c = 0; c < 4; ++c)
+                if (e + c < count) out[e + c] = Fn::call(a, *d, e + c, s[c]);
+        }
+    }
+}
+
+// bytes[...] = packed Fn::call(...) for i < count.  A lane's four codes of a row are
+// 4 * bits bits: half a byte, one, two or four bytes; with 1-bit codes two lanes share
+// a byte and the even one writes it.  The pad bits of the last byte are written as zero.
+template <class Args, class Dev, class Fn>
+__global__ __launch_bounds__(kBlock) void map_packed_kernel(Args a, const Dev* d, uint8_t* bytes, long long cap_bytes) {
+    const int bits = Fn::bits(a, *d);
+    if (!valid_bits(bits)) return;
+    const long long count = Fn::count(a, *d);
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long base = (long long)blockIdx.x * kTile + wave * 1024 + lane * 4;
+    if (base - lane * 4 >= count) return;  // the whole wavefront leaves together
+    f4 x[Fn::NS > 0 ? Fn::NS : 1][4];
+    load_streams<Args, Fn>(a, base, count, x);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const long long e = base + j * 256;
+        float s[4][Fn::NS > 0 ? Fn::NS : 1];
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int k = 0; k < Fn::NS; ++k) s[c][k] = x[k][j][c];
+        unsigned chunk = 0;
+        if (e + 3 < count) {  // the common case carries no per-element test
+#pragma unroll
+            for (int c = 0; c < 4; ++c) chunk |= to_code(Fn::call(a, *d, e + c, s[c]), bits) << (c * bits);
+        } else {
+            for (int c = 0; c < 4; ++c)
+                if (e + c < count) chunk |= to_code(Fn::call(a, *d, e + c, s[c]), bits) << (c * bits);
+        }
+        if (bits == 8) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                if (e + c < count && e + c < cap_bytes) bytes[e + c] = (uint8_t)(chunk >> (8 * c));
+        } else if (bits == 4) {
+            if (e < count && e / 2 < cap_bytes) bytes[e / 2] = (uint8_t)chunk;
+            if (e + 2 < count && e / 2 + 1 < cap_bytes) bytes[e / 2 + 1] = (uint8_t)(chunk >> 8);
+        } else if (bits == 2) {
+            if (e < count && e / 4 < cap_bytes) bytes[e / 4] = (uint8_t)chunk;
+        } else {
+            const unsigned other = (unsigned)__shfl_xor((int)chunk, 1, 64);
+            if ((lane & 1u) == 0 && e < count && e / 8 < cap_bytes) bytes[e / 8] = (uint8_t)(chunk | (other << 4));
+        }
+    }
+}
+
+}  // namespace cl

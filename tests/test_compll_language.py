@@ -1,0 +1,114 @@
+"""The CompLL operator language front end and back end (hipress_amd/compll), on the CPU:
+tokens, syntax tree, the host/device classification of scalars, the launch plan and
+the error messages.  The generated library is only checked for its symbols here."""
+import ctypes
+import os
+
+import pytest
+
+from hipress_amd import compll
+from hipress_amd.compll import backend, frontend as F
+from hipress_amd.compll.build import LIB, manifests, programs
+
+
+def test_tokens_and_comments():
+    toks = F.tokenize("a<<2 // note\n /* block\n */ x -> uint<b>* [&] 1.5e-3 >= 7")
+    assert [t.text for t in toks[:-1]] == ["a", "<<", "2", "x", "->", "uint", "<", "b", ">", "*", "[&]", "1.5e-3", ">=", "7"]
+    assert toks[3].line == 3 and toks[11].kind == "float" and toks[13].kind == "int"
+    with pytest.raises(F.CompileError, match="line 2"):
+        F.tokenize("ok\n $")
+
+
+def test_precedence_and_tree():
+    prog = F.parse("void f(float* v, uint8* out, uint8 b){ int k = 1 + 2 * 3 << 1; uint8 t = v.size % (1<<b); }")
+    fn = prog.functions[0]
+    assert [p.name for p in fn.params] == ["v", "out", "b"] and fn.params[0].type.pointer
+    k = fn.body[0].value  # ((1 + (2*3)) << 1)
+    assert isinstance(k, F.Binary) and k.op == "<<" and k.lhs.op == "+" and k.lhs.rhs.op == "*"
+    t = fn.body[1].value
+    assert t.op == "%" and isinstance(t.lhs, F.SizeOf) and t.rhs.op == "<<"
+
+
+def test_uint_width_expression_stops_at_the_closing_bracket():
+    prog = F.parse("void f(float* v, uint8* out, uint8 b){ lambda_func q = [&](int i) -> uint<b+1> { return i > 3; } }")
+    lam = prog.functions[0].body[0]
+    assert isinstance(lam, F.Lambda) and lam.ret.base == "uint" and lam.ret.bits.op == "+"
+    assert lam.body[0].value.op == ">"
+
+
+def test_param_block_is_accepted():
+    prog = F.parse("param P { uint8 bitwidth; } void f(float* v, uint8* o){ }")
+    assert prog.param_blocks["P"][0].name == "bitwidth"
+
+
+PROGRAM = """
+void Enc(float* g, uint8* out, uint8 b) {
+    lambda_func hi = [&](float x, float y) -> float { if (x > y) { return x; } return y; }
+    lambda_func lo = [&](float x, float y) -> float { if (x < y) { return x; } return y; }
+    float top = reduce(g, -1, hi);
+    float bottom = reduce(g, 1, lo);
+    float step = (top - bottom) / ((1 << b) - 1);
+    uint8 rest = g.size % (1 << b);
+    lambda_func q = [&](int i) -> uint<b> { return floor((g[i] - bottom) / step + random<float>(0, 1)); }
+    uint<b>* codes = map(range(g.size), q);
+    out = concat(b, rest, bottom, top, codes);
+}
+"""
+
+
+def test_plan_classifies_scalars_and_fuses_reductions():
+    g = backend.FunctionGen(F.parse(PROGRAM).functions[0])
+    cls = {n: s.cls for n, s in g.scalars.items()}
+    assert cls == {"b": "host", "top": "dev", "bottom": "dev", "step": "dev", "rest": "host"}
+    # both folds in one sweep; the scalars and header fields that follow are computed by the
+    # reduce's last kernel, so the operator is two sweeps and no launch of one thread
+    assert g.launch_kinds() == ["reduce", "map_packed"]
+    assert [s.kind for s in g.stages] == ["reduce", "serial", "map_packed"]
+    assert len(g.stages[0].folds) == 2 and g.needs_uniform
+    src, man = compll.compile_text(PROGRAM)
+    assert 'extern "C" int Enc(float* g, int32_t g_size, uint8_t* out, int32_t out_size, uint8_t b, const float* uniform, ' \
+           "void* workspace, int64_t workspace_bytes, void* stream)" in src
+    assert "cl::put<float>(a.v_out + 2, (float)d.v_bottom);" in src  # header offsets 0, 1, 2, 6; codes behind byte 10
+    assert "(a.v_out + 10)" in src
+    assert man[0]["params"] == [{"name": "g", "kind": "float*"}, {"name": "out", "kind": "uint8*"}, {"name": "b", "kind": "uint8"}]
+
+
+@pytest.mark.parametrize("body,message", [
+    ("float m = reduce(g, 0, nothing);", "unknown lambda"),
+    ("uint<2>* c = map(range(g.size), f); ", "never stored"),
+    ("b = 3;", "cannot be assigned"),
+    ("float r = random<float>(0, 1);", "inside a lambda"),
+    ("float x = y + 1;", "unknown scalar"),
+    ("float x; float z = x * 2;", "before it has a value"),
+    ("out = concat(c, b);", "unknown"),
+    ("lambda_func h = [&](float x) -> float { return x; } float m = reduce(g, 0, h);", r"\(float, float\) -> float"),
+    ("float s = 1.5 << 2;", "needs integers"),
+])
+def test_errors_name_the_problem(body, message):
+    text = "void Op(float* g, uint8* out, uint8 b) { lambda_func f = [&](int i) -> uint<2> { return i; } " + body + " }"
+    with pytest.raises(F.CompileError, match=message):
+        compll.compile_text(text)
+
+
+def test_syntax_errors_carry_the_line():
+    with pytest.raises(F.CompileError, match="line 3"):
+        F.parse("void f(float* g, uint8* o) {\n float x = 1;\n float = 2;\n}")
+    with pytest.raises(F.CompileError, match="no function"):
+        F.parse("// nothing here")
+
+
+def test_shipped_programs_compile_and_the_library_exports_them():
+    assert programs(), "no operator programs shipped"
+    man = manifests()
+    assert {"MinMaxQuantEncode", "MinMaxQuantDecode", "ThresholdTernaryEncode", "ThresholdTernaryDecode",
+            "MeanAndSpread"} <= set(man)
+    assert man["MinMaxQuantEncode"]["launches"] == ["reduce", "map_packed"]
+    assert man["MinMaxQuantDecode"]["launches"] == ["serial", "map_float"]
+    assert man["MeanAndSpread"]["launches"] == ["reduce"]  # three folds, one sweep
+    assert os.path.exists(LIB), "generated library not built: python -m hipress_amd.compll.build"
+    lib = ctypes.CDLL(LIB)
+    for name in man:
+        assert hasattr(lib, name) and hasattr(lib, name + "_workspace_bytes")
+    ws = lib.MinMaxQuantEncode_workspace_bytes
+    ws.argtypes, ws.restype = [ctypes.c_int64], ctypes.c_int64
+    assert ws(0) >= 256 and ws(1 << 20) >= 256 + 4 * 2 * 256 and ws(-1) < 0

@@ -1,0 +1,124 @@
+"""Operators generated from the shipped CompLL programs, on the GPU, against the CPU oracle
+and the hand-written kernels.  MinMaxQuant is the in-tree operator of the reference
+restated in the language, so its payload must equal the oracle's byte for byte given
+the same uniform tensor; ThresholdTernary produces the code words of the TBQ operator
+with a zero residual."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+F = np.float32
+SIZES = [1, 3, 4, 5, 31, 1000, 4095, 4096, 4097, 12289, 262144, 1000003]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from hipress_amd.compll import runtime
+
+    assert torch.cuda.is_available()
+    return runtime.load()  # fails loudly if the generated library is missing
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+@pytest.mark.parametrize("b", [1, 2, 4, 8])
+@pytest.mark.parametrize("n", SIZES)
+def test_minmax_quant_matches_the_oracle(ops, n, b):
+    import hipress_amd as hp
+
+    rng = np.random.default_rng(1000 * b + n)
+    g = rng.normal(0, 1e-2, n).astype(F)
+    u = rng.random(n, dtype=F)
+    want = oracle.compll_encode(g, u, b)
+    pay = torch.full((want.size + 5,), 0xAB, dtype=torch.uint8, device="cuda")
+    ops.MinMaxQuantEncode(dev(g), pay[: want.size], b, uniform=dev(u))
+    got = host(pay)
+    np.testing.assert_array_equal(got[: want.size], want)
+    assert (got[want.size:] == 0xAB).all(), "wrote past the payload"
+    # the hand-written operator produces the same bytes
+    pay2 = torch.zeros(hp.compll_payload_bytes(n, b), dtype=torch.uint8, device="cuda")
+    hp.compll_terngrad_encode(dev(g), dev(u), pay2, b)
+    np.testing.assert_array_equal(host(pay2), want)
+    # decode: as many elements as the payload says, bounded by the output
+    ref = oracle.compll_decode(want, n + 8)
+    out = torch.full((n + 8,), 7.0, device="cuda")
+    ops.MinMaxQuantDecode(pay[: want.size], out)
+    o = host(out)
+    np.testing.assert_array_equal(o[: ref.size], ref)
+    assert (o[ref.size:] == 7.0).all()
+    short = torch.full((max(n - 2, 0),), 7.0, device="cuda")
+    ops.MinMaxQuantDecode(pay[: want.size], short)
+    k = min(short.numel(), ref.size)
+    np.testing.assert_array_equal(host(short)[:k], ref[:k])
+    assert (host(short)[k:] == 7.0).all()
+
+
+def test_minmax_quant_constant_and_extreme_inputs(ops):
+    n = 5000
+    u = np.random.default_rng(3).random(n, dtype=F)
+    for g in (np.full(n, 0.25, F), np.zeros(n, F), np.linspace(-2e5, 2e5, n).astype(F)):
+        want = oracle.compll_encode(g, u, 2)
+        pay = torch.zeros(want.size, dtype=torch.uint8, device="cuda")
+        ops.MinMaxQuantEncode(dev(g), pay, 2, uniform=dev(u))
+        np.testing.assert_array_equal(host(pay), want)
+
+
+@pytest.mark.parametrize("n", SIZES)
+def test_threshold_ternary_matches_tbq_codes(ops, n):
+    rng = np.random.default_rng(n)
+    t = F(0.05)
+    g = rng.normal(0, 0.04, n).astype(F)
+    g[:: 7] = t  # exactly on the threshold: taken
+    g[3:: 11] = -t
+    nbytes = 4 + (2 * n + 7) // 8
+    pay = torch.full((nbytes + 3,), 0xAB, dtype=torch.uint8, device="cuda")
+    ops.ThresholdTernaryEncode(dev(g), pay[:nbytes], float(t))
+    got = host(pay)
+    assert got[:4].view(F)[0] == t and (got[nbytes:] == 0xAB).all()
+    tbq, _ = oracle.tbq_encode(g, np.zeros(n, F), t)  # 16-byte header, then the same code words
+    np.testing.assert_array_equal(got[4:nbytes], tbq[16 : 16 + nbytes - 4])
+    out = torch.full((n,), 7.0, device="cuda")
+    ops.ThresholdTernaryDecode(pay[:nbytes], out)
+    np.testing.assert_array_equal(host(out), oracle.tbq_decode(tbq, n))
+
+
+@pytest.mark.parametrize("n", [1, 100, 4096, 4097, 1000003])
+def test_mean_and_spread(ops, n):
+    g = np.random.default_rng(n).normal(0.5, 1.0, n).astype(F)
+    pay = torch.zeros(8, dtype=torch.uint8, device="cuda")
+    ops.MeanAndSpread(dev(g), pay)
+    mean, spread = host(pay).view(F)
+    assert abs(float(mean) - float(g.astype(np.float64).mean())) <= 1e-5 * max(1.0, abs(float(g.mean())))  # a sum: order differs
+    assert spread == F(g.max()) - F(g.min())  # max and min are exact
+
+
+def test_generated_ops_report_errors(ops):
+    from hipress_amd.compll.runtime import GeneratedOpError
+
+    g = torch.zeros(100, device="cuda")
+    u = torch.zeros(100, device="cuda")
+    with pytest.raises(GeneratedOpError, match="too small"):
+        ops.MinMaxQuantEncode(g, torch.zeros(20, dtype=torch.uint8, device="cuda"), 2, uniform=u)
+    with pytest.raises(GeneratedOpError, match="bad parameter"):
+        ops.MinMaxQuantEncode(g, torch.zeros(200, dtype=torch.uint8, device="cuda"), 3, uniform=u)
+    with pytest.raises(TypeError):
+        ops.MinMaxQuantEncode(g, torch.zeros(200, dtype=torch.uint8, device="cuda"), 2)  # no uniform tensor
+    with pytest.raises(TypeError):
+        ops.MinMaxQuantEncode(g.double(), torch.zeros(200, dtype=torch.uint8, device="cuda"), 2, uniform=u)
+    # a payload whose header names an impossible width decodes to nothing
+    bad = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    bad[0] = 3
+    out = torch.full((50,), 7.0, device="cuda")
+    ops.MinMaxQuantDecode(bad, out)
+    assert (host(out) == 7.0).all()
