@@ -71,6 +71,7 @@ class Vector:
     bits_cls: str = "host"
     pending_map: Optional[tuple] = None  # packed vector defined by map, waiting for its place: (count, lambda)
     bits_ast: Optional[F.Expr] = None    # code width not resolvable at the declaration (it is extracted later)
+    virtual: Optional[tuple] = None      # float vector that is a map never stored: (count Value, lambda name)
 
 
 @dataclass
@@ -183,6 +184,12 @@ class FunctionGen:
             return Value(f"({v.size})", "int", v.size_cls)
         if isinstance(e, F.Index):
             v = self.vector(e.vec, e.line)
+            if v.virtual:  # an element of a mapped vector that is never stored is a call of its lambda
+                i = self.expr(e.index, scope, index_name)
+                if i.kind != "int":
+                    raise CompileError("a vector index must be an integer", e.line)
+                self.compile_lambda(v.virtual[1])
+                return Value(f"fn_{v.virtual[1]}(a, d, {i.code})", "float", "dev")
             if v.ptr is None:
                 raise CompileError(f"vector {e.vec!r} has no storage yet (it is waiting for concat)", e.line)
             i = self.expr(e.index, scope, index_name)
@@ -370,8 +377,12 @@ class FunctionGen:
 
     def reduce(self, target: Scalar, r: F.Reduce):
         vec = self.vector(r.vec, r.line)
-        if vec.elem != "float" or vec.ptr is None:
+        if vec.elem != "float" or (vec.ptr is None and not vec.virtual):
             raise CompileError("reduce works on float vectors", r.line)
+        if vec.virtual:
+            if vec.virtual[0].cls != "host":
+                raise CompileError("a mapped vector that is reduced needs a host-known length", r.line)
+            self.compile_map_lambda(vec.virtual[1])
         if target.base != "float":
             raise CompileError("the result of reduce is a float", r.line)
         if r.fn not in self.lambdas:
@@ -414,7 +425,7 @@ class FunctionGen:
         if isinstance(value, F.Map):
             if v.elem == "float":
                 if not v.is_param:
-                    raise CompileError("a float vector produced by map must be a parameter of the operator", line)
+                    raise CompileError("a local float vector is defined once, where it is declared", line)
                 _, count = self.map_check(value, "float")
                 self.compile_map_lambda(value.fn)
                 st = Stage("map_float", vec=v, fn=value.fn, count=count)
@@ -515,8 +526,15 @@ class FunctionGen:
                     if st.value is not None:
                         raise
                     v = Vector(st.name, "packed", bits_ast=t.bits)  # the width comes out of an extract
+            elif t.base == "float":
+                if not isinstance(st.value, F.Map):
+                    raise CompileError("a local float vector must be defined by map(...)", st.line)
+                _, count = self.map_check(st.value, "float")
+                v = Vector(st.name, "float", size=count.code, size_cls=count.cls, virtual=(count, st.value.fn))
+                self.vectors[st.name] = v
+                return
             else:
-                raise CompileError("local vectors must be uint<bits>* (float vectors are parameters)", st.line)
+                raise CompileError("local vectors must be float* or uint<bits>*", st.line)
             self.vectors[st.name] = v
             if st.value is not None:
                 self.assign_vector(v, st.value, st.line)
@@ -636,8 +654,28 @@ class FunctionGen:
                 o.append("    }")
                 o.append("};")
                 n = st.vec.size
-                launches.append(f"{{ const long long n = {n}; const unsigned tiles = (unsigned)((n + cl::kTile - 1) / cl::kTile);")
-                launches.append(f"  if (tiles) hipLaunchKernelGGL((cl::reduce_tiles_kernel<Args, Dev, Folds{k}>), dim3(tiles), dim3(cl::kBlock), 0, st, a, d, {st.vec.ptr}, n, partial);")
+                o.append(f"struct Source{k} {{  // what is folded: a stored vector, or a mapped one computed on the way")
+                o.append(f"    static __device__ __forceinline__ long long count(const Args& a, const Dev& d) {{ return (long long)({n}); }}")
+                if st.vec.virtual:
+                    fn = st.vec.virtual[1]
+                    streams = self.map_streams[fn]
+                    call = f"mfn_{fn}(a, d, i, s)"
+                else:
+                    streams, call = [st.vec.ptr], "s[0]"
+                o.append(f"    static constexpr int NS = {len(streams)};")
+                o.append("    static __device__ __forceinline__ const float* stream(const Args& a, int k) {")
+                for i, ptr in enumerate(streams):
+                    o.append(f"        if (k == {i}) return {ptr};")
+                o.append("        return nullptr;")
+                o.append("    }")
+                o.append(f"    static __device__ __forceinline__ float call(const Args& a, const Dev& d, long long i, const float* s) {{ return {call}; }}")
+                o.append("};")
+                if st.vec.virtual:
+                    for ptr in streams:
+                        if ptr != "a.uniform":
+                            self.checks.append(f"if ((long long)({n}) > (long long){ptr}_size) return -2;")
+                launches.append(f"{{ const long long n = {n}; const unsigned tiles = (unsigned)(n > 0 ? (n + cl::kTile - 1) / cl::kTile : 0);")
+                launches.append(f"  if (tiles) hipLaunchKernelGGL((cl::reduce_tiles_kernel<Args, Dev, Folds{k}, Source{k}>), dim3(tiles), dim3(cl::kBlock), 0, st, a, d, partial);")
                 after = f"Serial{k + 1}" if k + 1 in fused else "cl::Nothing"
                 launches.append(f"  hipLaunchKernelGGL((cl::reduce_final_kernel<Args, Dev, Folds{k}, {after}>), dim3(1), dim3(cl::kFinalBlock), 0, st, a, d, partial, tiles); }}")
             else:

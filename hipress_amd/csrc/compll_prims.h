@@ -83,6 +83,31 @@ __global__ void serial_kernel(Args a, Dev* d) {
     if (blockIdx.x == 0 && threadIdx.x == 0) Body::run(a, *d);
 }
 
+// ---- streamed operands ---------------------------------------------------------------------
+// A lane owns four consecutive indices of each of four rows of 256 of its
+// wavefront's 1024.  Fn::stream(a, k), k < Fn::NS, are the float vectors a lambda
+// reads at its own index; they are loaded as 16-byte vectors, whole rows per wavefront.
+template <class Args, class Fn>
+__device__ __forceinline__ void load_streams(const Args& a, long long base, long long count, f4 (&x)[Fn::NS > 0 ? Fn::NS : 1][4]) {
+#pragma unroll
+    for (int k = 0; k < Fn::NS; ++k) {
+        const float* p = Fn::stream(a, k);
+        const bool vec_ok = (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const long long e = base + j * 256;
+            if (e + 3 < count && vec_ok) {
+                x[k][j] = __builtin_nontemporal_load(reinterpret_cast<const f4*>(p + e));
+            } else {
+                x[k][j].x = e < count ? p[e] : 0.f;
+                x[k][j].y = e + 1 < count ? p[e + 1] : 0.f;
+                x[k][j].z = e + 2 < count ? p[e + 2] : 0.f;
+                x[k][j].w = e + 3 < count ? p[e + 3] : 0.f;
+            }
+        }
+    }
+}
+
 // ---- reduce --------------------------------------------------------------------------------
 // Folds::K folds over one float vector in one sweep.  Folds provides
 //   static float init(const Args&, const Dev&, int k)
@@ -92,28 +117,40 @@ __global__ void serial_kernel(Args a, Dev* d) {
 // reduce f has to be associative and commutative, and the order in which elements
 // meet is this kernel's business.  init enters exactly once, at the very end, so f
 // need not be idempotent in it (a sum with a non-zero init stays correct).
-template <class Args, class Dev, class Folds>
-__global__ __launch_bounds__(kBlock) void reduce_tiles_kernel(Args a, const Dev* d, const float* v, long long n,
-                                                              float* partial) {
+// Src says what is folded: count(a, d), NS / stream(a, k) and call(a, d, i, s) as for a
+// map - a stored vector is the lambda that returns its one streamed operand, a
+// mapped vector that is never stored is computed here, on the way into the fold.
+template <class Args, class Dev, class Folds, class Src>
+__global__ __launch_bounds__(kBlock) void reduce_tiles_kernel(Args a, const Dev* d, float* partial) {
     __shared__ float wave_acc[4][Folds::K];
     __shared__ int wave_any[4];
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const long long base = (long long)blockIdx.x * kTile + wave * 1024;
-    const bool vec_ok = (reinterpret_cast<uintptr_t>(v) & 15u) == 0;
+    const long long n = Src::count(a, *d);
+    const long long base = (long long)blockIdx.x * kTile + wave * 1024 + lane * 4;
+    f4 in[Src::NS > 0 ? Src::NS : 1][4];
+    load_streams<Args, Src>(a, base, n, in);
     f4 x[4];
     unsigned ok[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const long long e = base + j * 256 + lane * 4;
+        const long long e = base + j * 256;
         const long long left = n - e;
         ok[j] = left >= 4 ? 0xfu : (left <= 0 ? 0u : ((1u << left) - 1u));
-        if (ok[j] == 0xfu && vec_ok) {
-            x[j] = __builtin_nontemporal_load(reinterpret_cast<const f4*>(v + e));
+        float s[4][Src::NS > 0 ? Src::NS : 1];
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int k = 0; k < Src::NS; ++k) s[c][k] = in[k][j][c];
+        if (ok[j] == 0xfu) {
+            x[j].x = Src::call(a, *d, e, s[0]);
+            x[j].y = Src::call(a, *d, e + 1, s[1]);
+            x[j].z = Src::call(a, *d, e + 2, s[2]);
+            x[j].w = Src::call(a, *d, e + 3, s[3]);
         } else {
-            x[j].x = (ok[j] & 1u) ? v[e] : 0.f;
-            x[j].y = (ok[j] & 2u) ? v[e + 1] : 0.f;
-            x[j].z = (ok[j] & 4u) ? v[e + 2] : 0.f;
-            x[j].w = (ok[j] & 8u) ? v[e + 3] : 0.f;
+            x[j].x = (ok[j] & 1u) ? Src::call(a, *d, e, s[0]) : 0.f;
+            x[j].y = (ok[j] & 2u) ? Src::call(a, *d, e + 1, s[1]) : 0.f;
+            x[j].z = (ok[j] & 4u) ? Src::call(a, *d, e + 2, s[2]) : 0.f;
+            x[j].w = (ok[j] & 8u) ? Src::call(a, *d, e + 3, s[3]) : 0.f;
         }
     }
     float acc[Folds::K];
@@ -241,27 +278,6 @@ __global__ __launch_bounds__(kFinalBlock) void reduce_final_kernel(Args a, Dev* 
 //   bits(a, d)               (packed maps) width of the codes
 // A lane owns four consecutive indices of each of four rows of 256, as in the other
 // operators of this library.
-
-template <class Args, class Fn>
-__device__ __forceinline__ void load_streams(const Args& a, long long base, long long count, f4 (&x)[Fn::NS > 0 ? Fn::NS : 1][4]) {
-#pragma unroll
-    for (int k = 0; k < Fn::NS; ++k) {
-        const float* p = Fn::stream(a, k);
-        const bool vec_ok = (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const long long e = base + j * 256;
-            if (e + 3 < count && vec_ok) {
-                x[k][j] = __builtin_nontemporal_load(reinterpret_cast<const f4*>(p + e));
-            } else {
-                x[k][j].x = e < count ? p[e] : 0.f;
-                x[k][j].y = e + 1 < count ? p[e + 1] : 0.f;
-                x[k][j].z = e + 2 < count ? p[e + 2] : 0.f;
-                x[k][j].w = e + 3 < count ? p[e + 3] : 0.f;
-            }
-        }
-    }
-}
 
 // out[i] = Fn::call(...) for i < min(count, cap).
 template <class Args, class Dev, class Fn>

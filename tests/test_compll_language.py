@@ -83,6 +83,8 @@ def test_plan_classifies_scalars_and_fuses_reductions():
     ("out = concat(c, b);", "unknown"),
     ("lambda_func h = [&](float x) -> float { return x; } float m = reduce(g, 0, h);", r"\(float, float\) -> float"),
     ("float s = 1.5 << 2;", "needs integers"),
+    ("float* w; ", "defined by map"),
+    ("lambda_func m = [&](int i) -> float { return g[i]; } float* w = map(range(g.size), m); w = map(range(g.size), m);", "defined once"),
 ])
 def test_errors_name_the_problem(body, message):
     text = "void Op(float* g, uint8* out, uint8 b) { lambda_func f = [&](int i) -> uint<2> { return i; } " + body + " }"
@@ -101,10 +103,11 @@ def test_shipped_programs_compile_and_the_library_exports_them():
     assert programs(), "no operator programs shipped"
     man = manifests()
     assert {"MinMaxQuantEncode", "MinMaxQuantDecode", "ThresholdTernaryEncode", "ThresholdTernaryDecode",
-            "MeanAndSpread"} <= set(man)
+            "MeanAndSpread", "SignMeanEncode", "SignMeanDecode"} <= set(man)
     assert man["MinMaxQuantEncode"]["launches"] == ["reduce", "map_packed"]
     assert man["MinMaxQuantDecode"]["launches"] == ["serial", "map_float"]
     assert man["MeanAndSpread"]["launches"] == ["reduce"]  # three folds, one sweep
+    assert man["SignMeanEncode"]["launches"] == ["reduce", "map_packed"]  # the mapped magnitudes are folded, never stored
     assert os.path.exists(LIB), "generated library not built: python -m hipress_amd.compll.build"
     lib = ctypes.CDLL(LIB)
     for name in man:

@@ -103,6 +103,27 @@ def test_mean_and_spread(ops, n):
     assert spread == F(g.max()) - F(g.min())  # max and min are exact
 
 
+@pytest.mark.parametrize("n", SIZES)
+def test_sign_mean_matches_onebit_without_residual(ops, n):
+    """The magnitudes are a mapped vector that is only folded (never stored); the sign bits
+    are the onebit operator's with a zero residual, the scale its mean magnitude."""
+    g = np.random.default_rng(n + 7).normal(0, 1e-2, n).astype(F)
+    g[:: 13] = 0.0  # zero counts as not negative
+    nbytes = 4 + (n + 7) // 8
+    pay = torch.full((nbytes + 3,), 0xAB, dtype=torch.uint8, device="cuda")
+    ops.SignMeanEncode(dev(g), pay[:nbytes])
+    got = host(pay)
+    assert (got[nbytes:] == 0xAB).all()
+    scale = got[:4].view(F)[0]
+    want_scale = oracle.onebit_scale(g, np.zeros(n, F))
+    assert abs(float(scale) - float(want_scale)) <= 1e-5 * float(want_scale)
+    onebit, _ = oracle.onebit_encode(g, np.zeros(n, F), scale=scale)
+    np.testing.assert_array_equal(got[4:nbytes], onebit[16 : 16 + nbytes - 4])
+    out = torch.full((n,), 7.0, device="cuda")
+    ops.SignMeanDecode(pay[:nbytes], out)
+    np.testing.assert_array_equal(host(out), oracle.onebit_decode(onebit, n))
+
+
 def test_generated_ops_report_errors(ops):
     from hipress_amd.compll.runtime import GeneratedOpError
 
