@@ -115,3 +115,42 @@ def test_shipped_programs_compile_and_the_library_exports_them():
     ws = lib.MinMaxQuantEncode_workspace_bytes
     ws.argtypes, ws.restype = [ctypes.c_int64], ctypes.c_int64
     assert ws(0) >= 256 and ws(1 << 20) >= 256 + 4 * 2 * 256 and ws(-1) < 0
+
+
+def test_command_line_writes_source_and_manifest(tmp_path):
+    import json
+    import subprocess
+    import sys
+
+    prog = tmp_path / "op.pse"
+    prog.write_text(PROGRAM)
+    out, man = tmp_path / "op.hip", tmp_path / "op.json"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-m", "hipress_amd.compll", str(prog), "-o", str(out), "--manifest", str(man)],
+                       cwd=root, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    assert 'extern "C" int Enc(' in out.read_text()
+    assert json.loads(man.read_text())[0]["name"] == "Enc"
+    prog.write_text("void Broken(float* g, uint8* o) {\n float x = ;\n}")
+    r = subprocess.run([sys.executable, "-m", "hipress_amd.compll", str(prog)], cwd=root, capture_output=True, text=True)
+    assert r.returncode == 1 and "line 2" in r.stderr
+
+
+def test_lambda_bodies_translate_control_flow_and_helpers():
+    text = """
+void Op(float* g, uint8* out, float t) {
+    lambda_func clip = [&](float x) -> float { if (x > t) { return t; } else if (x < -t) { return -t; } return x; }
+    lambda_func level = [&](int i) -> uint<4> {
+        float v = clip(g[i]) / t;
+        int q = 0;
+        if (v >= 0.5) { q = 15; } else { q = 7; }
+        return q;
+    }
+    uint<4>* codes = map(range(g.size), level);
+    out = concat(t, codes);
+}
+"""
+    src, man = compll.compile_text(text)
+    assert "fn_clip(a, d, s[0])" in src          # g[i] arrives as a streamed operand; the helper is an ordinary call
+    assert "} else {" in src and "q = 15;" in src
+    assert man[0]["launches"] == ["serial", "map_packed"]
