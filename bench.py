@@ -27,18 +27,20 @@ HBM_PEAK_GBS = 8000.0
 # measured.  (FETCH_SIZE KiB * 2.0 + WRITE_SIZE KiB * 1.0) * 1024, the factors
 # being what the same counters read for a plain 1 GiB copy.
 MEASURED_TRAFFIC = {
-    "onebit_vgg19": 1747750604,           # onebit_quant_kernel
-    "onebit_deferred_vgg19": 1748885708,  # onebit_deferred_kernel
-    "tbq_vgg19": 1765707161,              # tbq_encode_kernel
+    "onebit_vgg19": 1747750092,           # onebit_quant_kernel
+    "onebit_deferred_vgg19": 1748885811,  # onebit_deferred_kernel
+    "tbq_vgg19": 1765707366,              # tbq_encode_kernel
     "terngrad_vgg19": 1193284403,         # terngrad_encode_kernel
-    "dgc_vgg19": 2904934092,              # sparse_accum_kernel
-    "graddrop_vgg19": 1755468902,         # sparse_accum_kernel
-    "tbq_262144_x512": 1650559385,        # tbq_encode_kernel
-    "terngrad_resnet50": 212500172,       # terngrad_encode_kernel
-    "dgc_bert_large": 6782811852,         # sparse_accum_kernel
-    "graddrop_bert_large": 4101437849,    # sparse_accum_kernel
-    "merge_tbq_vgg19": 2090603520,        # dense_merge_kernel
-    "merge_dgc_vgg19": 1780986470,        # sparse_merge_kernel
+    "dgc_vgg19": 2904932352,              # sparse_accum_kernel
+    "graddrop_vgg19": 1755470643,         # sparse_accum_kernel
+    "tbq_262144_x512": 1650560614,        # tbq_encode_kernel
+    "terngrad_resnet50": 212500377,       # terngrad_encode_kernel
+    "dgc_bert_large": 6782809395,         # sparse_accum_kernel
+    "graddrop_bert_large": 4101441843,    # sparse_accum_kernel
+    "merge_tbq_vgg19": 2090605363,        # dense_merge_kernel
+    "merge_dgc_vgg19": 1780991590,        # sparse_merge_kernel
+    "compll_b2_fc6": 848749465,           # compll_quant_kernel
+    "compll_generated_b2_fc6": 848736665, # map_packed_kernel of the generated operator
 }
 
 

@@ -83,12 +83,15 @@ class Operators:
                     raise ValueError(f"{name}: uniform= is shorter than the float vectors")
                 cargs.append(uniform.data_ptr())
             need = ws_bytes(biggest)
-            key = (device, name)
+            stream = torch.cuda.current_stream(device).cuda_stream
+            key = (device, stream, name)  # scratch is per stream: calls on one stream are ordered, others are not
             ws = self._workspaces.get(key)
             if ws is None or ws.numel() < need:
-                ws = self._workspaces[key] = torch.empty(need, dtype=torch.uint8, device=device)
-            cargs += [ws.data_ptr(), ws.numel(), torch.cuda.current_stream(device).cuda_stream]
-            rc = fn(*cargs)
+                with torch.cuda.device(device):
+                    ws = self._workspaces[key] = torch.empty(need, dtype=torch.uint8, device=device)
+            cargs += [ws.data_ptr(), ws.numel(), stream]
+            with torch.cuda.device(device):
+                rc = fn(*cargs)
             if rc != 0:
                 raise GeneratedOpError(f"{name}: {_ERRORS.get(rc, rc)}")
 
