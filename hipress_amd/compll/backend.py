@@ -31,6 +31,22 @@ _SCALAR_BYTES = {"float": 4, "int": 4, "int32": 4, "uint8": 1, "uint16": 2, "uin
 _CALLS = {"floor": "floorf", "ceil": "ceilf", "abs": "fabsf", "fabs": "fabsf", "sqrt": "sqrtf", "exp": "expf", "log": "logf"}
 
 
+def _rerunnable(lines) -> bool:
+    """Whether a block of serial statements gives the same result when it is run again on
+    its own output (no statement reads a device scalar that the block assigns at or after
+    that statement): such a block may be run by every workgroup of the sweep that follows."""
+    import re
+
+    targets = [re.match(r"d\.v_(\w+) = ", ln) for ln in lines]
+    names = [m.group(1) if m else None for m in targets]
+    for i, ln in enumerate(lines):
+        rhs = ln[targets[i].end():] if targets[i] else ln
+        later = {n for n in names[i:] if n}
+        if any(re.search(r"\bd\.v_%s\b" % re.escape(n), rhs) for n in later):
+            return False
+    return True
+
+
 def _unparen(code: str) -> str:
     """Drops one pair of parentheses that encloses the whole expression."""
     if code.startswith("(") and code.endswith(")"):
@@ -571,9 +587,13 @@ class FunctionGen:
         """The launches of the operator in order; a serial block right after a reduce
         runs inside the reduce's last kernel and is not a launch of its own."""
         out = []
+        last = len(self.stages) - 1
         for k, st in enumerate(self.stages):
-            if st.kind == "serial" and (not st.lines or (k and self.stages[k - 1].kind == "reduce")):
-                continue
+            if st.kind == "serial":
+                if not st.lines or (k and self.stages[k - 1].kind == "reduce"):
+                    continue
+                if k == last - 1 and self.stages[last].kind in ("map_float", "map_packed") and _rerunnable(st.lines):
+                    continue  # runs at the start of the last sweep
             out.append(st.kind)
         return out
 
@@ -621,6 +641,13 @@ class FunctionGen:
         for k, st in enumerate(self.stages):
             if st.kind == "reduce" and k + 1 < len(self.stages) and self.stages[k + 1].kind == "serial" and self.stages[k + 1].lines:
                 fused.add(k + 1)
+        # a serial block right before the last sweep of the operator runs at the start of that
+        # sweep, in every workgroup, if running it again changes nothing
+        before = {}
+        last = len(self.stages) - 1
+        if last >= 1 and self.stages[last].kind in ("map_float", "map_packed") and self.stages[last - 1].kind == "serial" \
+                and self.stages[last - 1].lines and (last - 1) not in fused and _rerunnable(self.stages[last - 1].lines):
+            before[last] = last - 1
         order = sorted(range(len(self.stages)), key=lambda k: (k - 1.5) if k in fused else k)  # a fused block is emitted first
         for k in order:
             st = self.stages[k]
@@ -632,7 +659,7 @@ class FunctionGen:
                 o += ["        " + ln for ln in st.lines]
                 o.append("    }")
                 o.append("};")
-                if k not in fused:
+                if k not in fused and k not in before.values():
                     launches.append(f"hipLaunchKernelGGL((cl::serial_kernel<Args, Dev, Serial{k}>), dim3(1), dim3(64), 0, st, a, d);")
             elif st.kind == "reduce":
                 K = len(st.folds)
@@ -701,10 +728,14 @@ class FunctionGen:
                         self.checks.append(f"if ((long long)({st.count.code}) > (long long){ptr}_size) return -2;")
                 launches.append(f"{{ long long bound = (long long)({st.bound}); if (bound < 0) bound = 0;")
                 launches.append("  const unsigned tiles = (unsigned)((bound + cl::kTile - 1) / cl::kTile);")
+                pre = f"Serial{before[k]}" if k in before else "cl::Nothing"
                 if st.kind == "map_packed":
-                    launches.append(f"  if (tiles) hipLaunchKernelGGL((cl::map_packed_kernel<Args, Dev, Map{k}>), dim3(tiles), dim3(cl::kBlock), 0, st, a, d, {st.dest}, {st.cap}); }}")
+                    launches.append(f"  if (tiles) hipLaunchKernelGGL((cl::map_packed_kernel<Args, Dev, Map{k}, {pre}>), dim3(tiles), dim3(cl::kBlock), 0, st, a, d, {st.dest}, {st.cap});")
                 else:
-                    launches.append(f"  if (tiles) hipLaunchKernelGGL((cl::map_float_kernel<Args, Dev, Map{k}>), dim3(tiles), dim3(cl::kBlock), 0, st, a, d, {st.vec.ptr}, (long long){st.vec.size}); }}")
+                    launches.append(f"  if (tiles) hipLaunchKernelGGL((cl::map_float_kernel<Args, Dev, Map{k}, {pre}>), dim3(tiles), dim3(cl::kBlock), 0, st, a, d, {st.vec.ptr}, (long long){st.vec.size});")
+                if k in before:  # an empty range launches no sweep; the block still has to run
+                    launches.append(f"  else hipLaunchKernelGGL((cl::serial_kernel<Args, Dev, {pre}>), dim3(1), dim3(64), 0, st, a, d);")
+                launches.append("}")
         o.append(f"}}  // namespace {self.ns}")
         o.append("")
         sig, _ = self.signature()

@@ -17,6 +17,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace cl {
 
 typedef float f4 __attribute__((ext_vector_type(4)));
@@ -74,6 +76,11 @@ __device__ __forceinline__ float uniform_from(float u, float lo, float hi) { ret
 __device__ __forceinline__ float uniform_draw(const float* u, long long i, float lo, float hi) {
     return uniform_from(u[i], lo, hi);
 }
+
+struct Nothing {
+    template <class Args, class Dev>
+    static __device__ void run(const Args&, Dev&) {}
+};
 
 // ---- serial block ------------------------------------------------------------------------
 // Scalar statements that depend on device values (and header reads / writes) run
@@ -222,11 +229,6 @@ __global__ __launch_bounds__(kBlock) void reduce_tiles_kernel(Args a, const Dev*
 // One workgroup folds the per-tile results (every tile of a launch holds at least
 // one element), combines them with the initial values and stores the K results.
 // With no tile at all the results are the initial values.
-struct Nothing {
-    template <class Args, class Dev>
-    static __device__ void run(const Args&, Dev&) {}
-};
-
 // After::run: the scalar statements that follow the reduce in the program, if any.
 template <class Args, class Dev, class Folds, class After>
 __global__ __launch_bounds__(kFinalBlock) void reduce_final_kernel(Args a, Dev* d, const float* partial, unsigned ntiles) {
@@ -279,9 +281,27 @@ __global__ __launch_bounds__(kFinalBlock) void reduce_final_kernel(Args a, Dev* 
 // A lane owns four consecutive indices of each of four rows of 256, as in the other
 // operators of this library.
 
+// Before::run: scalar statements that precede the sweep and may be run again freely.
+// Every workgroup runs them into its own copy of the device scalars and works from
+// that copy; the first workgroup also publishes it.  With Nothing the scalars are
+// read where they are.
+template <class Args, class Dev, class Before>
+__device__ __forceinline__ const Dev* device_scalars(const Args& a, Dev* d, Dev* mine) {
+    if (std::is_same<Before, Nothing>::value) return d;
+    if (threadIdx.x == 0) {
+        *mine = *d;
+        Before::run(a, *mine);
+        if (blockIdx.x == 0) *d = *mine;
+    }
+    __syncthreads();
+    return mine;
+}
+
 // out[i] = Fn::call(...) for i < min(count, cap).
-template <class Args, class Dev, class Fn>
-__global__ __launch_bounds__(kBlock) void map_float_kernel(Args a, const Dev* d, float* out, long long cap) {
+template <class Args, class Dev, class Fn, class Before>
+__global__ __launch_bounds__(kBlock) void map_float_kernel(Args a, Dev* dglobal, float* out, long long cap) {
+    __shared__ Dev mine;
+    const Dev* d = device_scalars<Args, Dev, Before>(a, dglobal, &mine);
     long long count = Fn::count(a, *d);
     if (count > cap) count = cap;
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
@@ -314,8 +334,10 @@ __global__ __launch_bounds__(kBlock) void map_float_kernel(Args a, const Dev* d,
 // bytes[...] = packed Fn::call(...) for i < count.  A lane's four codes of a row are
 // 4 * bits bits: half a byte, one, two or four bytes; with 1-bit codes two lanes share
 // a byte and the even one writes it.  The pad bits of the last byte are written as zero.
-template <class Args, class Dev, class Fn>
-__global__ __launch_bounds__(kBlock) void map_packed_kernel(Args a, const Dev* d, uint8_t* bytes, long long cap_bytes) {
+template <class Args, class Dev, class Fn, class Before>
+__global__ __launch_bounds__(kBlock) void map_packed_kernel(Args a, Dev* dglobal, uint8_t* bytes, long long cap_bytes) {
+    __shared__ Dev mine;
+    const Dev* d = device_scalars<Args, Dev, Before>(a, dglobal, &mine);
     const int bits = Fn::bits(a, *d);
     if (!valid_bits(bits)) return;
     const long long count = Fn::count(a, *d);

@@ -105,7 +105,7 @@ def test_shipped_programs_compile_and_the_library_exports_them():
     assert {"MinMaxQuantEncode", "MinMaxQuantDecode", "ThresholdTernaryEncode", "ThresholdTernaryDecode",
             "MeanAndSpread", "SignMeanEncode", "SignMeanDecode"} <= set(man)
     assert man["MinMaxQuantEncode"]["launches"] == ["reduce", "map_packed"]
-    assert man["MinMaxQuantDecode"]["launches"] == ["serial", "map_float"]
+    assert man["MinMaxQuantDecode"]["launches"] == ["map_float"]  # the header is read at the start of the sweep
     assert man["MeanAndSpread"]["launches"] == ["reduce"]  # three folds, one sweep
     assert man["SignMeanEncode"]["launches"] == ["reduce", "map_packed"]  # the mapped magnitudes are folded, never stored
     assert os.path.exists(LIB), "generated library not built: python -m hipress_amd.compll.build"
@@ -153,4 +153,19 @@ void Op(float* g, uint8* out, float t) {
     src, man = compll.compile_text(text)
     assert "fn_clip(a, d, s[0])" in src          # g[i] arrives as a streamed operand; the helper is an ordinary call
     assert "} else {" in src and "q = 15;" in src
-    assert man[0]["launches"] == ["serial", "map_packed"]
+    assert man[0]["launches"] == ["map_packed"]
+
+
+def test_a_block_that_reads_its_own_output_keeps_its_launch():
+    text = """
+void Op(uint8* packed, float* g) {
+    float k;
+    uint<2>* codes;
+    extract(packed, k, codes);
+    k = k * 2;
+    lambda_func f = [&](int i) -> float { return codes[i] * k; }
+    g = map(range(g.size), f);
+}
+"""
+    _, man = compll.compile_text(text)
+    assert man[0]["launches"] == ["serial", "map_float"]  # k = k * 2 must run exactly once
