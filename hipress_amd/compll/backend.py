@@ -109,6 +109,7 @@ class Stage:
     dest: str = ""
     cap: str = ""
     bits: Optional[Value] = None
+    float_map: Optional["Stage"] = None  # map_fused: the float map that shares the sweep of this packed map
 
 
 class FunctionGen:
@@ -135,6 +136,31 @@ class FunctionGen:
         for v in self.vectors.values():
             if v.pending_map:
                 raise CompileError(f"packed vector {v.name!r} is computed but never stored with concat", fn.line)
+        self._fuse_maps()
+
+    def _fuse_maps(self):
+        """A packed map directly followed by a float map over the same range becomes one
+        sweep when element i of either result depends on the vector being written only
+        through element i (so computing both from the values loaded first is what running
+        them one after the other would give)."""
+        k = 0
+        while k + 1 < len(self.stages):
+            p, f = self.stages[k], self.stages[k + 1]
+            if p.kind == "map_packed" and f.kind == "map_float" and p.count.code == f.count.code and p.count.cls == "host":
+                written = f.vec.name
+                ok = True
+                for fn in (p.fn, f.fn):
+                    _, vectors, elsewhere = self.uses(fn)
+                    if written in elsewhere:
+                        ok = False
+                _, fvec, _ = self.uses(f.fn)
+                if p.vec.name in fvec:  # the float map reads the codes themselves
+                    ok = False
+                if ok:
+                    p.kind, p.float_map = "map_fused", f
+                    del self.stages[k + 1]
+                    self.checks.append(f"if ((long long)({p.count.code}) > (long long){f.vec.size}) return -2;")
+            k += 1
 
     # ---------------------------------------------------------------- symbols
     def _declare_params(self):
@@ -300,6 +326,85 @@ class FunctionGen:
         self.lambda_code[name] = "\n".join(lines)
         self.lambda_order.append(name)
 
+    def uses(self, name: str, _seen=None):
+        """What a lambda reads from the operator's scope, found on the syntax tree:
+        (scalars, vectors, vectors read anywhere but at the lambda's own index).  Helpers it
+        calls and mapped vectors it indexes are followed; what they read counts as read at
+        other indices."""
+        _seen = _seen or set()
+        if name in _seen:
+            return set(), set(), set()
+        _seen = _seen | {name}
+        lam = self.lambdas[name]
+        local = {p.name for p in lam.params}
+        own = lam.params[0].name if len(lam.params) == 1 and self._kind_of(lam.params[0].type) == "int" else None
+        if own and self._assigns(lam.body, own):
+            own = None
+        scalars, vectors, elsewhere = set(), set(), set()
+
+        def follow(fn):
+            s2, v2, _ = self.uses(fn, _seen)
+            scalars.update(s2)
+            vectors.update(v2)
+            elsewhere.update(v2)
+
+        def ex(e):
+            if isinstance(e, F.Name):
+                if e.id not in local:
+                    scalars.add(e.id)
+            elif isinstance(e, F.Unary):
+                ex(e.arg)
+            elif isinstance(e, F.Binary):
+                ex(e.lhs)
+                ex(e.rhs)
+            elif isinstance(e, F.Index):
+                ex(e.index)
+                vec = self.vectors.get(e.vec)
+                if vec is not None and vec.virtual:
+                    follow(vec.virtual[1])
+                else:
+                    vectors.add(e.vec)
+                    if not (own and isinstance(e.index, F.Name) and e.index.id == own):
+                        elsewhere.add(e.vec)
+            elif isinstance(e, F.Call):
+                for x in e.args:
+                    ex(x)
+                if e.fn in self.lambdas:
+                    follow(e.fn)
+            elif isinstance(e, F.Random):
+                ex(e.lo)
+                ex(e.hi)
+
+        def body(stmts):
+            for st in stmts:
+                if isinstance(st, F.Declare):
+                    if st.value is not None:
+                        ex(st.value)
+                    local.add(st.name)
+                elif isinstance(st, F.Assign):
+                    ex(st.value)
+                elif isinstance(st, F.If):
+                    ex(st.cond)
+                    body(st.then)
+                    body(st.otherwise)
+                elif isinstance(st, F.Return):
+                    ex(st.value)
+
+        body(lam.body)
+        return scalars, vectors, elsewhere
+
+    def _guard_pending(self, line, scalar=None, vector=None):
+        """A packed vector computed by map is produced where concat places it.  Nothing its
+        lambda reads may change in between, or the codes would be computed from the new values."""
+        for v in self.vectors.values():
+            if not v.pending_map:
+                continue
+            scalars, vectors, _ = self.uses(v.pending_map[1])
+            if (scalar and scalar in scalars) or (vector and vector in vectors):
+                what = scalar or vector
+                raise CompileError(f"{what!r} changes before the codes {v.name!r} computed from it are stored; "
+                                   f"put the concat of {v.name!r} first", line)
+
     def _stream(self, ptr: str) -> int:
         if ptr not in self.streams:
             self.streams.append(ptr)
@@ -385,6 +490,11 @@ class FunctionGen:
             raise CompileError(f"parameter {s.name!r} cannot be assigned", line)
         if s.cls is not None and s.cls != v.cls and not (s.cls == "dev" and v.cls == "host"):
             raise CompileError(f"{s.name!r} cannot change from a host value to a device value", line)
+        if s.cls == "host":
+            # host-known scalars are all evaluated before the first launch, so a second value
+            # would also be seen by the launches that should see the first
+            raise CompileError(f"{s.name!r} is known on the host and can be assigned only once", line)
+        self._guard_pending(line, scalar=s.name)
         s.cls = s.cls or v.cls
         if s.cls == "host":
             self.host_lines.append(f"a.v_{s.name} = ({s.ctype})({v.code});")
@@ -443,6 +553,7 @@ class FunctionGen:
                 if not v.is_param:
                     raise CompileError("a local float vector is defined once, where it is declared", line)
                 _, count = self.map_check(value, "float")
+                self._guard_pending(line, vector=v.name)
                 self.compile_map_lambda(value.fn)
                 st = Stage("map_float", vec=v, fn=value.fn, count=count)
                 st.bound = count.code if count.cls == "host" else v.size
@@ -592,7 +703,7 @@ class FunctionGen:
             if st.kind == "serial":
                 if not st.lines or (k and self.stages[k - 1].kind == "reduce"):
                     continue
-                if k == last - 1 and self.stages[last].kind in ("map_float", "map_packed") and _rerunnable(st.lines):
+                if k == last - 1 and self.stages[last].kind in ("map_float", "map_packed", "map_fused") and _rerunnable(st.lines):
                     continue  # runs at the start of the last sweep
             out.append(st.kind)
         return out
@@ -645,7 +756,7 @@ class FunctionGen:
         # sweep, in every workgroup, if running it again changes nothing
         before = {}
         last = len(self.stages) - 1
-        if last >= 1 and self.stages[last].kind in ("map_float", "map_packed") and self.stages[last - 1].kind == "serial" \
+        if last >= 1 and self.stages[last].kind in ("map_float", "map_packed", "map_fused") and self.stages[last - 1].kind == "serial" \
                 and self.stages[last - 1].lines and (last - 1) not in fused and _rerunnable(self.stages[last - 1].lines):
             before[last] = last - 1
         order = sorted(range(len(self.stages)), key=lambda k: (k - 1.5) if k in fused else k)  # a fused block is emitted first
@@ -708,20 +819,33 @@ class FunctionGen:
             else:
                 o.append(f"struct Map{k} {{")
                 o.append(f"    static __device__ __forceinline__ long long count(const Args& a, const Dev& d) {{ return (long long)({st.count.code}); }}")
-                streams = self.map_streams[st.fn]
+                streams = list(self.map_streams[st.fn])
+                if st.kind == "map_fused":
+                    for ptr in self.map_streams[st.float_map.fn]:
+                        if ptr not in streams:
+                            streams.append(ptr)
                 o.append(f"    static constexpr int NS = {len(streams)};  // float vectors read at the index itself")
                 o.append("    static __device__ __forceinline__ const float* stream(const Args& a, int k) {")
                 for i, ptr in enumerate(streams):
                     o.append(f"        if (k == {i}) return {ptr};")
                 o.append("        return nullptr;")
                 o.append("    }")
-                if st.kind == "map_packed":
+                if st.kind in ("map_packed", "map_fused"):
                     o.append(f"    static __device__ __forceinline__ int bits(const Args& a, const Dev& d) {{ return (int)({st.bits.code}); }}")
                     lam = self.lambdas[st.fn]
                     ret = {"float": "float", "int": "long long"}[self.lambda_kind(lam)]
                 else:
                     ret = "float"
-                o.append(f"    static __device__ __forceinline__ {ret} call(const Args& a, const Dev& d, long long i, const float* s) {{ return mfn_{st.fn}(a, d, i, s); }}")
+                if st.kind == "map_fused":  # each lambda sees its own operands in its own order
+                    for label, fn, r in (("call_codes", st.fn, ret), ("call_values", st.float_map.fn, "float")):
+                        own = self.map_streams[fn]
+                        picks = ", ".join(f"s[{streams.index(ptr)}]" for ptr in own) or "0.f"
+                        o.append(f"    static __device__ __forceinline__ {r} {label}(const Args& a, const Dev& d, long long i, const float* s) {{")
+                        o.append(f"        const float mine[{max(len(own), 1)}] = {{{picks}}};")
+                        o.append(f"        return mfn_{fn}(a, d, i, mine);")
+                        o.append("    }")
+                else:
+                    o.append(f"    static __device__ __forceinline__ {ret} call(const Args& a, const Dev& d, long long i, const float* s) {{ return mfn_{st.fn}(a, d, i, s); }}")
                 o.append("};")
                 for ptr in streams:  # a streamed vector must cover the range
                     if ptr != "a.uniform" and st.count.cls == "host":
@@ -729,7 +853,9 @@ class FunctionGen:
                 launches.append(f"{{ long long bound = (long long)({st.bound}); if (bound < 0) bound = 0;")
                 launches.append("  const unsigned tiles = (unsigned)((bound + cl::kTile - 1) / cl::kTile);")
                 pre = f"Serial{before[k]}" if k in before else "cl::Nothing"
-                if st.kind == "map_packed":
+                if st.kind == "map_fused":
+                    launches.append(f"  if (tiles) hipLaunchKernelGGL((cl::map_fused_kernel<Args, Dev, Map{k}, {pre}>), dim3(tiles), dim3(cl::kBlock), 0, st, a, d, {st.dest}, {st.cap}, {st.float_map.vec.ptr});")
+                elif st.kind == "map_packed":
                     launches.append(f"  if (tiles) hipLaunchKernelGGL((cl::map_packed_kernel<Args, Dev, Map{k}, {pre}>), dim3(tiles), dim3(cl::kBlock), 0, st, a, d, {st.dest}, {st.cap});")
                 else:
                     launches.append(f"  if (tiles) hipLaunchKernelGGL((cl::map_float_kernel<Args, Dev, Map{k}, {pre}>), dim3(tiles), dim3(cl::kBlock), 0, st, a, d, {st.vec.ptr}, (long long){st.vec.size});")

@@ -378,4 +378,71 @@ __global__ __launch_bounds__(kBlock) void map_packed_kernel(Args a, Dev* dglobal
     }
 }
 
+// Two maps over the same range in one sweep: packed codes and a float vector (the shape
+// of a quantiser that also updates its error-feedback residual).  Fn provides count,
+// NS / stream for the operands of both lambdas, bits, call_codes and call_values.  All
+// operands of a thread are loaded before its first store, so the float output may be
+// one of the operands (an update in place).
+template <class Args, class Dev, class Fn, class Before>
+__global__ __launch_bounds__(kBlock) void map_fused_kernel(Args a, Dev* dglobal, uint8_t* bytes, long long cap_bytes,
+                                                           float* out) {
+    __shared__ Dev mine;
+    const Dev* d = device_scalars<Args, Dev, Before>(a, dglobal, &mine);
+    const int bits = Fn::bits(a, *d);
+    if (!valid_bits(bits)) return;
+    const long long count = Fn::count(a, *d);
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long base = (long long)blockIdx.x * kTile + wave * 1024 + lane * 4;
+    if (base - lane * 4 >= count) return;  // the whole wavefront leaves together
+    const bool vec_ok = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
+    f4 x[Fn::NS > 0 ? Fn::NS : 1][4];
+    load_streams<Args, Fn>(a, base, count, x);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const long long e = base + j * 256;
+        float s[4][Fn::NS > 0 ? Fn::NS : 1];
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int k = 0; k < Fn::NS; ++k) s[c][k] = x[k][j][c];
+        unsigned chunk = 0;
+        if (e + 3 < count) {
+            f4 q;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) chunk |= to_code(Fn::call_codes(a, *d, e + c, s[c]), bits) << (c * bits);
+            q.x = Fn::call_values(a, *d, e, s[0]);
+            q.y = Fn::call_values(a, *d, e + 1, s[1]);
+            q.z = Fn::call_values(a, *d, e + 2, s[2]);
+            q.w = Fn::call_values(a, *d, e + 3, s[3]);
+            if (vec_ok) {
+                __builtin_nontemporal_store(q, reinterpret_cast<f4*>(out + e));
+            } else {
+                out[e] = q.x;
+                out[e + 1] = q.y;
+                out[e + 2] = q.z;
+                out[e + 3] = q.w;
+            }
+        } else {
+            for (int c = 0; c < 4; ++c)
+                if (e + c < count) {
+                    chunk |= to_code(Fn::call_codes(a, *d, e + c, s[c]), bits) << (c * bits);
+                    out[e + c] = Fn::call_values(a, *d, e + c, s[c]);
+                }
+        }
+        if (bits == 8) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                if (e + c < count && e + c < cap_bytes) bytes[e + c] = (uint8_t)(chunk >> (8 * c));
+        } else if (bits == 4) {
+            if (e < count && e / 2 < cap_bytes) bytes[e / 2] = (uint8_t)chunk;
+            if (e + 2 < count && e / 2 + 1 < cap_bytes) bytes[e / 2 + 1] = (uint8_t)(chunk >> 8);
+        } else if (bits == 2) {
+            if (e < count && e / 4 < cap_bytes) bytes[e / 4] = (uint8_t)chunk;
+        } else {
+            const unsigned other = (unsigned)__shfl_xor((int)chunk, 1, 64);
+            if ((lane & 1u) == 0 && e < count && e / 8 < cap_bytes) bytes[e / 8] = (uint8_t)(chunk | (other << 4));
+        }
+    }
+}
+
 }  // namespace cl

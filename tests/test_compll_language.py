@@ -103,7 +103,8 @@ def test_shipped_programs_compile_and_the_library_exports_them():
     assert programs(), "no operator programs shipped"
     man = manifests()
     assert {"MinMaxQuantEncode", "MinMaxQuantDecode", "ThresholdTernaryEncode", "ThresholdTernaryDecode",
-            "MeanAndSpread", "SignMeanEncode", "SignMeanDecode"} <= set(man)
+            "MeanAndSpread", "SignMeanEncode", "SignMeanDecode", "ThresholdFeedbackEncode"} <= set(man)
+    assert man["ThresholdFeedbackEncode"]["launches"] == ["map_fused"]  # codes and residual in one sweep
     assert man["MinMaxQuantEncode"]["launches"] == ["reduce", "map_packed"]
     assert man["MinMaxQuantDecode"]["launches"] == ["map_float"]  # the header is read at the start of the sweep
     assert man["MeanAndSpread"]["launches"] == ["reduce"]  # three folds, one sweep
@@ -169,3 +170,25 @@ void Op(uint8* packed, float* g) {
 """
     _, man = compll.compile_text(text)
     assert man[0]["launches"] == ["serial", "map_float"]  # k = k * 2 must run exactly once
+
+
+FEEDBACK = """
+void Op(float* g, float* r, uint8* out, float t) {
+    lambda_func level = [&](int i) -> uint<2> { return r[%s] + g[i] >= t; }
+    lambda_func carry = [&](int i) -> float { return r[i] + g[i]; }
+    uint<2>* codes = map(range(g.size), level);
+    %s
+}
+"""
+
+
+def test_maps_share_a_sweep_only_when_that_is_what_the_program_says():
+    stored_first = "out = concat(t, codes); r = map(range(g.size), carry);"
+    assert compll.compile_text(FEEDBACK % ("i", stored_first))[1][0]["launches"] == ["map_fused"]
+    # the codes read a neighbour of the element being rewritten: two sweeps, in program order
+    assert compll.compile_text(FEEDBACK % ("i + 1", stored_first))[1][0]["launches"] == ["serial", "map_packed", "map_float"]
+    # the residual may not change between the map that reads it and the concat that runs it
+    with pytest.raises(F.CompileError, match="changes before the codes"):
+        compll.compile_text(FEEDBACK % ("i", "r = map(range(g.size), carry); out = concat(t, codes);"))
+    with pytest.raises(F.CompileError, match="only once"):
+        compll.compile_text("void Op(float* g, uint8* o, uint8 b) { int k = b + 1; k = 2; }")

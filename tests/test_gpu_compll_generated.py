@@ -93,6 +93,34 @@ def test_threshold_ternary_matches_tbq_codes(ops, n):
     np.testing.assert_array_equal(host(out), oracle.tbq_decode(tbq, n))
 
 
+@pytest.mark.parametrize("n", SIZES)
+def test_threshold_feedback_matches_tbq_over_steps(ops, n):
+    """Codes and the new residual come out of one fused sweep that updates the residual in
+    place; three steps against the TBQ oracle, residual carried."""
+    rng = np.random.default_rng(n + 99)
+    t = F(0.05)
+    r_ref = rng.normal(0, 0.02, n).astype(F)
+    r_gpu = dev(r_ref)
+    nbytes = 4 + (2 * n + 7) // 8
+    for step in range(3):
+        g = rng.normal(0, 0.03, n).astype(F)
+        pay = torch.full((nbytes + 3,), 0xAB, dtype=torch.uint8, device="cuda")
+        ops.ThresholdFeedbackEncode(dev(g), r_gpu, pay[:nbytes], float(t))
+        tbq, r_ref = oracle.tbq_encode(g, r_ref, t)
+        got = host(pay)
+        assert got[:4].view(F)[0] == t and (got[nbytes:] == 0xAB).all()
+        np.testing.assert_array_equal(got[4:nbytes], tbq[16 : 16 + nbytes - 4], err_msg=f"codes, step {step}")
+        np.testing.assert_array_equal(host(r_gpu), r_ref, err_msg=f"residual, step {step}")
+
+
+def test_threshold_feedback_rejects_a_short_residual(ops):
+    from hipress_amd.compll.runtime import GeneratedOpError
+
+    g = torch.zeros(1000, device="cuda")
+    with pytest.raises(GeneratedOpError, match="too small"):
+        ops.ThresholdFeedbackEncode(g, torch.zeros(999, device="cuda"), torch.zeros(400, dtype=torch.uint8, device="cuda"), 0.05)
+
+
 @pytest.mark.parametrize("n", [1, 100, 4096, 4097, 1000003])
 def test_mean_and_spread(ops, n):
     g = np.random.default_rng(n).normal(0.5, 1.0, n).astype(F)
