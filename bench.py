@@ -272,6 +272,42 @@ class CompllWorkload:
         self.g = self.u = self.pay = self.out = None
 
 
+class GeneratedTbqWorkload:
+    """The error-feedback threshold quantiser generated from its CompLL program (one fused
+    sweep for codes and residual) and its decoder, or the hand-written TBQ operator through
+    the same per-tensor entry points, on the largest VGG19 tensor."""
+
+    def __init__(self, name, n, generated):
+        self.name, self.sizes, self.elements, self.generated = name, [n], n, generated
+        self.enc_bytes, self.dec_bytes = 12.25, 4.25
+        self.dominant_kernel, self.dominant_bytes = ("map_fused_kernel" if generated else "tbq_encode_kernel"), 12.25
+
+    def setup(self, dev):
+        import torch
+
+        import hipress_amd as hp
+        from hipress_amd import workloads as W
+        from hipress_amd.compll import runtime
+
+        self.hp, self.gen = hp, runtime.load()
+        self.g = W.normal_set(self.sizes, dev, 0, sigma=0.02)[0]
+        self.r = torch.zeros(self.elements, device=dev)
+        nbytes = hp.tbq_payload_bytes(self.elements) if not self.generated else 4 + (2 * self.elements + 7) // 8
+        self.pay = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+        self.out = torch.empty(self.elements, device=dev)
+
+    def step(self, ev=None):
+        if self.generated:
+            self.gen.ThresholdFeedbackEncode(self.g, self.r, self.pay, 0.05)
+            self.gen.ThresholdTernaryDecode(self.pay, self.out)
+        else:
+            self.hp.tbq_encode(self.g, self.r, self.pay, 0.05)
+            self.hp.tbq_decode(self.pay, self.out)
+
+    def close(self):
+        self.g = self.r = self.pay = self.out = None
+
+
 def make_workload(name):
     from hipress_amd import workloads as W
 
@@ -308,6 +344,10 @@ def make_workload(name):
         return CompllWorkload(name, max(vgg))
     if name == "compll_generated_b2_fc6":
         return CompllWorkload(name, max(vgg), generated=True)
+    if name == "tbq_fc6":
+        return GeneratedTbqWorkload(name, max(vgg), generated=False)
+    if name == "tbq_generated_fc6":
+        return GeneratedTbqWorkload(name, max(vgg), generated=True)
     if name == "merge_tbq_vgg19":
         return MergeWorkload(name, "tbq", W.chunk_sizes(vgg))
     if name == "merge_dgc_vgg19":
@@ -318,7 +358,7 @@ def make_workload(name):
 ALL_WORKLOADS = [
     "onebit_vgg19", "onebit_deferred_vgg19", "tbq_vgg19", "terngrad_vgg19", "dgc_vgg19", "graddrop_vgg19", "tbq_262144", "tbq_262144_x512",
     "terngrad_resnet50", "dgc_bert_large", "graddrop_bert_large", "merge_tbq_vgg19", "merge_dgc_vgg19", "compll_b2_fc6",
-    "compll_generated_b2_fc6",
+    "compll_generated_b2_fc6", "tbq_fc6", "tbq_generated_fc6",
 ]
 
 
