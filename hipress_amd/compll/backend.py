@@ -871,6 +871,10 @@ class FunctionGen:
         o.append(f"    return 256 + 4 * {K} * ((max_elements + cl::kTile - 1) / cl::kTile + 1);")
         o.append("}")
         o.append("")
+        o.append(f"// {name}: vectors with their lengths in elements, then the scalar parameters" +
+                 (", then `uniform`: one uniform[0,1) float per element of the longest mapped range" if self.needs_uniform else "") +
+                 f"; workspace of at least {name}_workspace_bytes(longest float vector) bytes, 16-byte aligned;")
+        o.append("// returns 0, -1 null pointer, -2 a buffer too small, -3 misaligned workspace, -4 bad parameter, -5 HIP error, -6 workspace.")
         o.append(f'extern "C" int {name}({", ".join(t + " " + n for t, n in sig)}) {{')
         o.append(f"    using namespace {self.ns};")
         o.append("    Args a;")
