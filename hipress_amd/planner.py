@@ -10,7 +10,7 @@ fitting the encode / decode coefficients from measurements of this library's own
 kernels on the GPU at hand.
 
     python -m hipress_amd.planner --input input.txt --output SeCoPaPlan.txt --topology PS --nnodes 4
-    python -m hipress_amd.planner --calibrate tbq ...     # encode/decode models measured on cuda:0
+    python -m hipress_amd.planner --calibrate tbq ...     # encode/decode/merge models measured on cuda:0
 """
 import argparse
 import json
@@ -58,6 +58,11 @@ class Planner:
     ring_send: CostModel = REFERENCE_RING_SEND
     gather: CostModel = field(default=None)
     broadcast: CostModel = field(default=None)
+    # This library's aggregator decodes the peers' payloads, sums them and re-encodes the sum
+    # in one launch sequence.  With a model of that step (a function of the uncompressed
+    # partition size, for nodes - 1 peers) the PS cost counts it once in place of the
+    # reference's nodes - 1 decodes, nodes - 1 aggregations and one encode at the server.
+    merge: CostModel = field(default=None)
 
     def __post_init__(self):
         if self.gather is None or self.broadcast is None:
@@ -86,7 +91,11 @@ class Planner:
         for k in range(1, n + 1):
             part, cpart = size / k, size * r / k
             agg = (n - 1) * self.aggregate.cost(part)
-            if topology == "PS":  # SeCoPa.py:75-88
+            if topology == "PS" and self.merge is not None:
+                enc = (min(k + 1, n) - 1) * self.encode.cost(part)
+                dec = (min(n - 1 + k, 2 * (n - 1)) - (n - 1)) * self.decode.cost(cpart)
+                out.append(self.gather.cost(cpart) + self.broadcast.cost(cpart) + enc + dec + self.merge.cost(part))
+            elif topology == "PS":  # SeCoPa.py:75-88
                 enc = min(k + 1, n) * self.encode.cost(part)
                 dec = min(n - 1 + k, 2 * (n - 1)) * self.decode.cost(cpart)
                 out.append(self.gather.cost(cpart) + self.broadcast.cost(cpart) + enc + dec + agg)
@@ -189,6 +198,45 @@ def calibrate(alg="tbq", sizes=None, reps=20, comp_ratio=None):
             "encode": fit_cost_model(sizes, enc_t), "decode": fit_cost_model([n * ratio for n in sizes], dec_t)}
 
 
+def calibrate_merge(alg="tbq", npeers=3, sizes=None, reps=20):
+    """Measures decode-and-merge of `npeers` payloads with the fused re-encode on cuda:0 over a
+    range of partition sizes and fits the model (milliseconds as a function of the
+    uncompressed partition size in elements).  alg: tbq, dgc or graddrop."""
+    import torch
+
+    import hipress_amd as hp
+
+    sizes = sizes or [1 << k for k in range(10, 28, 2)]
+    times = []
+    for n in sizes:
+        if alg == "tbq":
+            nb, kw = hp.tbq_payload_bytes(n), {"threshold": 0.05}
+            enc = lambda g, pay: hp.tbq_encode(g, torch.zeros_like(g), pay, 0.05)
+        else:
+            ratio = 0.01 if alg == "graddrop" else 0.001
+            nb, kw = hp.sparse_payload_bytes(n, ratio), {"ratio": ratio}
+            enc = lambda g, pay: hp.graddrop_encode(g, torch.zeros_like(g), pay, ratio)
+        pays = []
+        for p in range(npeers):
+            pay = torch.zeros(nb, dtype=torch.uint8, device="cuda")
+            enc(torch.randn(n, device="cuda") * 1e-2, pay)
+            pays.append(pay)
+        chunk = {"compressed": pays, "aggregate": torch.empty(n, device="cuda"), "state": torch.zeros(n, device="cuda"),
+                 "out_compressed": torch.zeros(nb, dtype=torch.uint8, device="cuda")}
+        mb = hp.MergeBatch("tbq" if alg == "tbq" else "dgc", [chunk], **kw)
+        for _ in range(3):
+            mb.run()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            mb.run()
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1) / reps)
+        mb.close()
+    return {"alg": alg, "npeers": npeers, "unit": "ms", "sizes": sizes, "merge_ms": times, "merge": fit_cost_model(sizes, times)}
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description="SeCoPa: selective compression and partitioning plan")
     ap.add_argument("--input", default="input.txt", help="lines of name,size (fp32 elements)")
@@ -204,6 +252,10 @@ def main(argv=None):
         cal = calibrate(args.calibrate)
         kw = {"encode": cal["encode"], "decode": cal["decode"], "comp_ratio": cal["comp_ratio"]}
         print(json.dumps({k: (v.__dict__ if isinstance(v, CostModel) else v) for k, v in cal.items()}))
+        if args.calibrate in ("tbq", "dgc", "graddrop") and args.topology == "PS":
+            mer = calibrate_merge(args.calibrate, npeers=args.nnodes - 1)
+            kw["merge"] = mer["merge"]
+            print(json.dumps({k: (v.__dict__ if isinstance(v, CostModel) else v) for k, v in mer.items()}))
     planner = Planner(nodes=args.nnodes, **kw)
     with open(args.output, "w") as f:
         for line in planner.plan(read_gradients(args.input), args.topology):

@@ -84,3 +84,21 @@ def test_fit_recovers_a_piecewise_line():
     assert fit.overhead == 0.05
     assert abs(fit.weight - true.weight) / true.weight < 1e-6
     assert abs(fit.bias - true.bias) < 1e-6
+
+
+def test_fused_merge_model_replaces_the_server_side_terms():
+    """With a model of this library's decode-and-merge the PS cost counts that step once
+    instead of nodes - 1 decodes, nodes - 1 aggregations and the server's encode."""
+    from hipress_amd.planner import CostModel, Planner
+
+    enc, dec = CostModel(2e-9, 0.0, 0.0), CostModel(1e-9, 0.0, 0.0)
+    flat = CostModel(0.0, 0.0, 0.0)
+    base = Planner(nodes=4, encode=enc, decode=dec, gather=flat, broadcast=flat)
+    size, r = 1 << 20, base.comp_ratio
+    # k = 1: reference terms are 2 encodes and 4 decodes (SeCoPa.py:83-84)
+    assert base.compressed_costs(size)[0] == pytest.approx(2 * 2e-9 * size + 4 * 1e-9 * size * r)
+    merge = CostModel(5e-10, 0.0, 0.0)
+    fused = Planner(nodes=4, encode=enc, decode=dec, gather=flat, broadcast=flat, merge=merge)
+    assert fused.compressed_costs(size)[0] == pytest.approx(1 * 2e-9 * size + 1 * 1e-9 * size * r + 5e-10 * size)
+    # the ring formula has no server and is unchanged
+    assert fused.compressed_costs(size, "RING") == base.compressed_costs(size, "RING")
