@@ -56,6 +56,30 @@ def test_onebit_vgg19_full_set(hp):
     b.close()
 
 
+def test_tbq_vgg19_full_set_three_steps(hp):
+    """TBQ (threshold 0.05) over the 38 VGG19 tensors, three steps with the residual carried,
+    every tensor against the oracle."""
+    from hipress_amd import workloads as W
+
+    sizes = W.vgg19_sizes()
+    dev = torch.device("cuda:0")
+    ts = [{"gradient": torch.empty(n, device=dev), "residual": torch.zeros(n, device=dev), "out": torch.empty(n, device=dev),
+           "compressed": torch.full((hp.tbq_payload_bytes(n),), 0xAB, dtype=torch.uint8, device=dev)} for n in sizes]
+    b = hp.Batch("tbq", ts, threshold=0.05)
+    refs = [np.zeros(n, F) for n in sizes]
+    for step in range(3):
+        for t, g in zip(ts, W.normal_set(sizes, dev, 200 + step, sigma=0.02)):
+            t["gradient"].copy_(g)
+        b.encode()
+        b.decode()
+        for i, (t, n) in enumerate(zip(ts, sizes)):
+            want, refs[i] = oracle.tbq_encode(host(t["gradient"]), refs[i], 0.05)
+            np.testing.assert_array_equal(host(t["compressed"]), want, err_msg=f"payload, step {step} tensor {i}")
+            np.testing.assert_array_equal(host(t["residual"]), refs[i], err_msg=f"residual, step {step} tensor {i}")
+            np.testing.assert_array_equal(host(t["out"]), oracle.tbq_decode(want, n), err_msg=f"decode, step {step} tensor {i}")
+    b.close()
+
+
 def test_terngrad_resnet50_full_set(hp):
     """configs[2]: bucket 512, heavy-tailed gradients, explicit uniform tensor."""
     from hipress_amd import workloads as W
