@@ -16,6 +16,7 @@ terngrad, dgc, graddrop; /root/reference/README.md:9,45,160,276), with
 CompLL-style aliases (``TernGradEncode`` ...: TernGradEncode.cc:10) kept in
 ``ALIASES``.  All of them are also registered as ``torch.ops.hipress.<name>``.
 """
+import contextlib
 import ctypes
 
 import torch
@@ -93,6 +94,15 @@ def _same_numel(a, b, na, nb):
         raise ValueError(f"{na} has {a.numel()} elements, {nb} has {b.numel()}")
 
 
+_NO_SWITCH = contextlib.nullcontext()
+
+
+def _on(device):
+    """Makes `device` current for a call; costs nothing when it already is (the usual case,
+    and the one where a few microseconds per call matter: small tensors are launch-bound)."""
+    return _NO_SWITCH if torch.cuda.current_device() == device.index else torch.cuda.device(device)
+
+
 def _stream(t):
     return torch.cuda.current_stream(t.device).cuda_stream
 
@@ -119,14 +129,14 @@ def tbq_encode(gradient, residual, compressed, threshold):
     """Threshold two-bit quantisation with error feedback; residual is updated in place."""
     _f32(gradient, "gradient"); _f32(residual, "residual", gradient); _u8(compressed, "compressed", gradient)
     _same_numel(gradient, residual, "gradient", "residual")
-    with torch.cuda.device(gradient.device):
+    with _on(gradient.device):
         check(_lib.lib().hipress_tbq_encode(_p(gradient), _p(residual), gradient.numel(), _p(compressed),
                                             compressed.numel(), float(threshold), _stream(gradient)), "tbq_encode")
 
 
 def tbq_decode(compressed, gradient):
     _u8(compressed, "compressed"); _f32(gradient, "gradient", compressed)
-    with torch.cuda.device(gradient.device):
+    with _on(gradient.device):
         check(_lib.lib().hipress_tbq_decode(_p(compressed), compressed.numel(), _p(gradient), gradient.numel(),
                                             _stream(gradient)), "tbq_decode")
 
@@ -138,7 +148,7 @@ def onebit_encode(gradient, residual, compressed):
     _same_numel(gradient, residual, "gradient", "residual")
     L = _lib.lib()
     n = gradient.numel()
-    with torch.cuda.device(gradient.device):
+    with _on(gradient.device):
         need = size(L.hipress_onebit_workspace_bytes(n), "onebit_workspace_bytes")
         ws = _workspace(gradient, need)
         check(L.hipress_onebit_encode(_p(gradient), _p(residual), n, _p(compressed), compressed.numel(),
@@ -156,7 +166,7 @@ def onebit_encode_deferred(gradient, state, scale_state, compressed):
         raise ValueError("scale_state must hold exactly one float")
     L = _lib.lib()
     n = gradient.numel()
-    with torch.cuda.device(gradient.device):
+    with _on(gradient.device):
         ws = _workspace(gradient, size(L.hipress_onebit_workspace_bytes(n), "onebit_workspace_bytes"))
         check(L.hipress_onebit_encode_deferred(_p(gradient), _p(state), _p(scale_state), n, _p(compressed),
                                                compressed.numel(), _p(ws), ws.numel(), _stream(gradient)),
@@ -167,14 +177,14 @@ def onebit_residual(state, scale_state, residual):
     """residual = the error-feedback residual onebit_encode would hold after the same steps."""
     _f32(state, "state"); _f32(scale_state, "scale_state", state); _f32(residual, "residual", state)
     _same_numel(state, residual, "state", "residual")
-    with torch.cuda.device(state.device):
+    with _on(state.device):
         check(_lib.lib().hipress_onebit_residual(_p(state), _p(scale_state), state.numel(), _p(residual),
                                                  _stream(state)), "onebit_residual")
 
 
 def onebit_decode(compressed, gradient):
     _u8(compressed, "compressed"); _f32(gradient, "gradient", compressed)
-    with torch.cuda.device(gradient.device):
+    with _on(gradient.device):
         check(_lib.lib().hipress_onebit_decode(_p(compressed), compressed.numel(), _p(gradient), gradient.numel(),
                                                _stream(gradient)), "onebit_decode")
 
@@ -184,14 +194,14 @@ def terngrad_encode(gradient, uniform, compressed, bucket=512):
     """Stochastic ternarisation; `uniform` holds one U[0,1) draw per element."""
     _f32(gradient, "gradient"); _f32(uniform, "uniform", gradient); _u8(compressed, "compressed", gradient)
     _same_numel(gradient, uniform, "gradient", "uniform")
-    with torch.cuda.device(gradient.device):
+    with _on(gradient.device):
         check(_lib.lib().hipress_terngrad_encode(_p(gradient), _p(uniform), gradient.numel(), _p(compressed),
                                                  compressed.numel(), int(bucket), _stream(gradient)), "terngrad_encode")
 
 
 def terngrad_decode(compressed, gradient):
     _u8(compressed, "compressed"); _f32(gradient, "gradient", compressed)
-    with torch.cuda.device(gradient.device):
+    with _on(gradient.device):
         check(_lib.lib().hipress_terngrad_decode(_p(compressed), compressed.numel(), _p(gradient), gradient.numel(),
                                                  _stream(gradient)), "terngrad_decode")
 
@@ -208,7 +218,7 @@ def compll_terngrad_encode(gradient, uniform, compressed, bitwidth=2):
     _same_numel(gradient, uniform, "gradient", "uniform")
     L = _lib.lib()
     n = gradient.numel()
-    with torch.cuda.device(gradient.device):
+    with _on(gradient.device):
         ws = _workspace(gradient, size(L.hipress_compll_workspace_bytes(n), "compll_workspace_bytes"))
         check(L.hipress_compll_encode(_p(gradient), _p(uniform), n, _p(compressed), compressed.numel(), int(bitwidth),
                                       _p(ws), ws.numel(), _stream(gradient)), "compll_encode")
@@ -217,7 +227,7 @@ def compll_terngrad_encode(gradient, uniform, compressed, bitwidth=2):
 def compll_terngrad_decode(compressed, gradient):
     """Decode of that format; the element count comes from the payload length and its tail byte."""
     _u8(compressed, "compressed"); _f32(gradient, "gradient", compressed)
-    with torch.cuda.device(gradient.device):
+    with _on(gradient.device):
         check(_lib.lib().hipress_compll_decode(_p(compressed), compressed.numel(), _p(gradient), gradient.numel(),
                                                _stream(gradient)), "compll_decode")
 
@@ -231,7 +241,7 @@ def dgc_encode(gradient, momentum, accumulator, compressed, momentum_factor=0.9,
     _same_numel(gradient, momentum, "gradient", "momentum"); _same_numel(gradient, accumulator, "gradient", "accumulator")
     L = _lib.lib()
     n = gradient.numel()
-    with torch.cuda.device(gradient.device):
+    with _on(gradient.device):
         need = size(L.hipress_sparse_workspace_bytes(n, float(ratio)), "sparse_workspace_bytes")
         ws = _workspace(gradient, need)
         check(L.hipress_dgc_encode(_p(gradient), _p(momentum), _p(accumulator), n, _p(compressed), compressed.numel(),
@@ -244,7 +254,7 @@ def graddrop_encode(gradient, accumulator, compressed, ratio=0.01):
     _same_numel(gradient, accumulator, "gradient", "accumulator")
     L = _lib.lib()
     n = gradient.numel()
-    with torch.cuda.device(gradient.device):
+    with _on(gradient.device):
         need = size(L.hipress_sparse_workspace_bytes(n, float(ratio)), "sparse_workspace_bytes")
         ws = _workspace(gradient, need)
         check(L.hipress_graddrop_encode(_p(gradient), _p(accumulator), n, _p(compressed), compressed.numel(),
@@ -253,7 +263,7 @@ def graddrop_encode(gradient, accumulator, compressed, ratio=0.01):
 
 def dgc_decode(compressed, gradient):
     _u8(compressed, "compressed"); _f32(gradient, "gradient", compressed)
-    with torch.cuda.device(gradient.device):
+    with _on(gradient.device):
         check(_lib.lib().hipress_sparse_decode(_p(compressed), compressed.numel(), _p(gradient), gradient.numel(),
                                                _stream(gradient)), "sparse_decode")
 
@@ -281,7 +291,7 @@ def tbq_decode_merge(compressed_list, aggregate, residual=None, out_compressed=N
     if residual is not None:
         _f32(residual, "residual", aggregate); _u8(out_compressed, "out_compressed", aggregate)
         _same_numel(aggregate, residual, "aggregate", "residual")
-    with torch.cuda.device(aggregate.device):
+    with _on(aggregate.device):
         check(_lib.lib().hipress_tbq_decode_merge(
             ptrs, lens, P, _p(aggregate), aggregate.numel(), _p(residual), _p(out_compressed),
             out_compressed.numel() if out_compressed is not None else 0, float(threshold), _stream(aggregate)),
@@ -291,7 +301,7 @@ def tbq_decode_merge(compressed_list, aggregate, residual=None, out_compressed=N
 def onebit_decode_merge(compressed_list, aggregate):
     _f32(aggregate, "aggregate")
     ptrs, lens, P = _peers(compressed_list, aggregate)
-    with torch.cuda.device(aggregate.device):
+    with _on(aggregate.device):
         check(_lib.lib().hipress_onebit_decode_merge(ptrs, lens, P, _p(aggregate), aggregate.numel(),
                                                      _stream(aggregate)), "onebit_decode_merge")
 
@@ -299,7 +309,7 @@ def onebit_decode_merge(compressed_list, aggregate):
 def terngrad_decode_merge(compressed_list, aggregate):
     _f32(aggregate, "aggregate")
     ptrs, lens, P = _peers(compressed_list, aggregate)
-    with torch.cuda.device(aggregate.device):
+    with _on(aggregate.device):
         check(_lib.lib().hipress_terngrad_decode_merge(ptrs, lens, P, _p(aggregate), aggregate.numel(),
                                                        _stream(aggregate)), "terngrad_decode_merge")
 
@@ -315,7 +325,7 @@ def dgc_decode_merge(compressed_list, aggregate, accumulator=None, out_compresse
     if accumulator is not None:
         _f32(accumulator, "accumulator", aggregate); _u8(out_compressed, "out_compressed", aggregate)
         _same_numel(aggregate, accumulator, "aggregate", "accumulator")
-    with torch.cuda.device(aggregate.device):
+    with _on(aggregate.device):
         ws = _workspace(aggregate, size(L.hipress_sparse_merge_workspace_bytes(n, P, float(ratio), int(accumulator is not None)),
                                         "sparse_merge_workspace_bytes"))
         check(L.hipress_sparse_decode_merge(
@@ -366,21 +376,21 @@ class Batch:
         self.device = dev
         pr = Params(float(threshold), int(bucket), float(momentum_factor), 0.0, float(ratio))
         h = ctypes.c_void_p()
-        with torch.cuda.device(dev):
+        with _on(dev):
             check(_lib.lib().hipress_batch_create(ctypes.byref(h), alg_id, arr, len(tensors), ctypes.byref(pr)), "batch_create")
         self._h = h
 
     def encode(self):
-        with torch.cuda.device(self.device):
+        with _on(self.device):
             check(_lib.lib().hipress_batch_encode(self._h, torch.cuda.current_stream(self.device).cuda_stream), "batch_encode")
 
     def encode_phase(self, phase):
         """One launch of the encode sequence (measurement aid)."""
-        with torch.cuda.device(self.device):
+        with _on(self.device):
             check(_lib.lib().hipress_batch_encode_phase(self._h, int(phase), torch.cuda.current_stream(self.device).cuda_stream), "batch_encode_phase")
 
     def decode(self):
-        with torch.cuda.device(self.device):
+        with _on(self.device):
             check(_lib.lib().hipress_batch_decode(self._h, torch.cuda.current_stream(self.device).cuda_stream), "batch_decode")
 
     def close(self):
@@ -424,18 +434,18 @@ class MergeBatch:
         self.device = dev
         pr = Params(float(threshold), int(bucket), 0.0, 0.0, float(ratio))
         h = ctypes.c_void_p()
-        with torch.cuda.device(dev):
+        with _on(dev):
             check(_lib.lib().hipress_merge_batch_create(ctypes.byref(h), ALG_IDS[alg], arr, len(chunks), npeers,
                                                         ctypes.byref(pr)), "merge_batch_create")
         self._h = h
 
     def run(self):
-        with torch.cuda.device(self.device):
+        with _on(self.device):
             check(_lib.lib().hipress_merge_batch_run(self._h, torch.cuda.current_stream(self.device).cuda_stream), "merge_batch_run")
 
     def run_phase(self, phase):
         """One part of the launch sequence (measurement aid)."""
-        with torch.cuda.device(self.device):
+        with _on(self.device):
             check(_lib.lib().hipress_merge_batch_run_phase(self._h, int(phase), torch.cuda.current_stream(self.device).cuda_stream),
                   "merge_batch_run_phase")
 
