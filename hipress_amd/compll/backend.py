@@ -888,7 +888,8 @@ class FunctionGen:
             if s.is_param:
                 o.append(f"    a.v_{s.name} = {s.name};")
         if self.needs_uniform:
-            o.append("    if (!uniform) return -1;")
+            some = " || ".join(f"{v.name}_size > 0" for v in self.vectors.values() if v.is_param and v.elem == "float") or "true"
+            o.append(f"    if (!uniform && ({some})) return -1;")
             o.append("    a.uniform = uniform;")
         else:
             o.append("    a.uniform = nullptr;")

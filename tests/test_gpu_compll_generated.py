@@ -152,6 +152,28 @@ def test_sign_mean_matches_onebit_without_residual(ops, n):
     np.testing.assert_array_equal(host(out), oracle.onebit_decode(onebit, n))
 
 
+def test_generated_ops_on_empty_and_truncated_inputs(ops):
+    empty = torch.zeros(0, device="cuda")
+    # no element: the header is still written, nothing else
+    pay = torch.full((12,), 0xAB, dtype=torch.uint8, device="cuda")
+    ops.MinMaxQuantEncode(empty, pay[:10], 2, uniform=empty)
+    got = host(pay)
+    want = oracle.compll_encode(np.zeros(0, F), np.zeros(0, F), 2)
+    np.testing.assert_array_equal(got[:10], want)
+    assert (got[10:] == 0xAB).all()
+    pay = torch.full((8,), 0xAB, dtype=torch.uint8, device="cuda")
+    ops.ThresholdTernaryEncode(empty, pay[:4], 0.25)
+    assert host(pay)[:4].view(F)[0] == F(0.25) and (host(pay)[4:] == 0xAB).all()
+    ops.SignMeanEncode(empty, pay[:4])  # the mean of nothing: 0 / 0
+    assert np.isnan(host(pay)[:4].view(F)[0])
+    # a payload cut off inside its header decodes to nothing
+    out = torch.full((16,), 7.0, device="cuda")
+    ops.MinMaxQuantDecode(torch.tensor([2, 0, 0, 0, 0], dtype=torch.uint8, device="cuda"), out)
+    assert (host(out) == 7.0).all()
+    ops.MinMaxQuantDecode(pay[:0], out)
+    assert (host(out) == 7.0).all()
+
+
 def test_generated_ops_report_errors(ops):
     from hipress_amd.compll.runtime import GeneratedOpError
 
