@@ -87,11 +87,13 @@ class Operators:
             key = (device, stream, name)  # scratch is per stream: calls on one stream are ordered, others are not
             ws = self._workspaces.get(key)
             if ws is None or ws.numel() < need:
-                with torch.cuda.device(device):
-                    ws = self._workspaces[key] = torch.empty(need, dtype=torch.uint8, device=device)
+                ws = self._workspaces[key] = torch.empty(need, dtype=torch.uint8, device=device)
             cargs += [ws.data_ptr(), ws.numel(), stream]
-            with torch.cuda.device(device):
+            if torch.cuda.current_device() == device.index:
                 rc = fn(*cargs)
+            else:
+                with torch.cuda.device(device):
+                    rc = fn(*cargs)
             if rc != 0:
                 raise GeneratedOpError(f"{name}: {_ERRORS.get(rc, rc)}")
 
