@@ -398,7 +398,12 @@ class Batch:
             _lib.lib().hipress_batch_destroy(self._h)
             self._h = None
 
-    __del__ = close
+    def __del__(self):
+        # at interpreter shutdown the library module may already be gone
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class MergeBatch:
@@ -454,7 +459,12 @@ class MergeBatch:
             _lib.lib().hipress_merge_batch_destroy(self._h)
             self._h = None
 
-    __del__ = close
+    def __del__(self):
+        # at interpreter shutdown the library module may already be gone
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 # ---------------------------------------------------------------- aliases + torch.ops registration
