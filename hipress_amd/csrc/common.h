@@ -63,12 +63,17 @@ struct MergeSeg {
     unsigned long long tp0;  // sparse: first tile pointer of this chunk
 };
 
+// where(k) = {tensor index, tile index inside the tensor} of tile k of the launch;
+// seg(i) = descriptor of tensor i, whose id is i and whose tiles are the launch's
+// tiles tile0 .. tile0 + ntiles - 1, so k = tile0 + tile index.
 struct SingleSrc {
     Seg seg;
     __device__ __forceinline__ const Seg& get(unsigned& tile, unsigned blk) const {
         tile = blk;
         return seg;
     }
+    __device__ __forceinline__ uint2 where(unsigned blk) const { return make_uint2(0u, blk); }
+    __device__ __forceinline__ const Seg& at(unsigned) const { return seg; }
 };
 
 struct BatchSrc {
@@ -79,6 +84,8 @@ struct BatchSrc {
         tile = m.y;
         return segs[m.x];
     }
+    __device__ __forceinline__ uint2 where(unsigned blk) const { return map[blk]; }
+    __device__ __forceinline__ const Seg& at(unsigned i) const { return segs[i]; }
 };
 
 // Per-tensor (not per-tile) launches: workgroup i works on tensor i.
@@ -204,10 +211,21 @@ __device__ __forceinline__ float wave_max(float x) {
     }
     return x;
 }
-__device__ __forceinline__ unsigned wave_sum_u(unsigned x) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) x += (unsigned)__shfl_xor((int)x, m, 64);
+// Inclusive prefix sum over the 64 lanes in six data-parallel-primitive steps:
+// four shifts inside every row of 16 lanes, then lane 15 of rows 0 and 2 is added
+// to the row after it, then lane 31 to the upper two rows.
+__device__ __forceinline__ unsigned wave_incl_scan_u(unsigned x) {
+    x += (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x111, 0xf, 0xf, true);   // row_shr:1
+    x += (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x112, 0xf, 0xf, true);   // row_shr:2
+    x += (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x114, 0xf, 0xf, true);   // row_shr:4
+    x += (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x118, 0xf, 0xf, true);   // row_shr:8
+    x += (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1, 3
+    x += (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2, 3
     return x;
+}
+// Sum over the 64 lanes, the same value (wavefront-uniform) in every lane.
+__device__ __forceinline__ unsigned wave_sum_u(unsigned x) {
+    return (unsigned)__builtin_amdgcn_readlane((int)wave_incl_scan_u(x), 63);
 }
 #endif  // __HIPCC__
 

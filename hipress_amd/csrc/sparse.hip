@@ -196,14 +196,18 @@ __global__ __launch_bounds__(kBlock) void sparse_select_kernel(Src src, SparseWs
     const unsigned k = pass ? ctl[kCtlK] : s.ks;  // read before the barriers; the owner below rewrites it
     for (unsigned i = threadIdx.x; i < nb; i += kBlock) lh[i] = 0;
     __syncthreads();
+    // all sixteen keys of a thread are requested before the first one is looked at
     const unsigned long long lo = (unsigned long long)stile * kSampleTile;
-#pragma unroll 4
+    unsigned key[kSampleTile / kBlock];
+#pragma unroll
     for (int j = 0; j < kSampleTile / kBlock; ++j) {
-        unsigned long long i = lo + j * kBlock + threadIdx.x;
-        if (i < s.ns) {
-            unsigned key = keys[i];
-            if ((key & above) == prefix) atomicAdd(&lh[(key >> shift) & (nb - 1)], 1u);
-        }
+        const unsigned long long i = lo + j * kBlock + threadIdx.x;
+        key[j] = i < s.ns ? keys[i] : 0u;
+    }
+#pragma unroll
+    for (int j = 0; j < kSampleTile / kBlock; ++j) {
+        const unsigned long long i = lo + j * kBlock + threadIdx.x;
+        if (i < s.ns && (key[j] & above) == prefix) atomicAdd(&lh[(key[j] >> shift) & (nb - 1)], 1u);
     }
     __syncthreads();
     unsigned was[kBins / kBlock];  // what the adds return; all are issued before any is waited for
@@ -240,12 +244,7 @@ __global__ __launch_bounds__(kBlock) void sparse_select_kernel(Src src, SparseWs
     // exclusive prefix of the chunk sums, from the top: wavefront scan, then the
     // four wavefront totals through LDS
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    unsigned incl = mine;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        unsigned y = (unsigned)__shfl_up((int)incl, d, 64);
-        if ((int)lane >= d) incl += y;
-    }
+    const unsigned incl = wave_incl_scan_u(mine);
     if (lane == 63) chunk[wave] = incl;
     __syncthreads();
     unsigned before = incl - mine;
@@ -292,12 +291,12 @@ __device__ __forceinline__ unsigned pick_row(unsigned row, unsigned a, unsigned 
 // to thr; lane l looks at the record of 64-element group l and only groups that
 // may hold more than one such key are read, eight per round, the next round's
 // loads in flight while this round is counted.  Wavefront-uniform result.
-__device__ __forceinline__ void count_tile(const Seg& s, const SparseWs& ws, unsigned tile, unsigned thr,
-                                           unsigned lane, unsigned& gt, unsigned& eq) {
+__device__ __forceinline__ void count_tile(const Seg& s, uint2 rec, unsigned tile, unsigned thr, unsigned lane,
+                                           unsigned& gt, unsigned& eq) {
     const long long n = (long long)s.n;
     const bool aligned = s.aligned != 0;
     const float* acc = s.s1;
-    const GroupView gv = view_group(ws.grec[(unsigned long long)(s.tile0 + tile) * 64 + lane], thr);
+    const GroupView gv = view_group(rec, thr);
     unsigned long long mask = __ballot(gv.multi);
     const unsigned row = lane >> 4;
     const long long base = (long long)tile * kTile + (lane & 15u) * 4;
@@ -344,49 +343,49 @@ __global__ __launch_bounds__(kBlock) void sparse_count_kernel(Src src, SparseWs 
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const unsigned gt_idx = blockIdx.x * 4 + wave;
     if (gt_idx >= total_tiles) return;
-    unsigned tile;
-    const Seg s = src.get(tile, gt_idx);
-    const unsigned thr = ws.thr[2 * s.id];
+    // the record needs nothing but the tile's place in the launch, the threshold only
+    // the tensor's index: neither waits for the descriptor
+    const uint2 rec = ws.grec[(unsigned long long)gt_idx * 64 + lane];
+    const uint2 m = src.where(gt_idx);
+    const unsigned thr = ws.thr[2 * m.x];
+    const Seg s = src.at(m.x);
     unsigned gt, eq;
-    count_tile(s, ws, tile, thr, lane, gt, eq);
-    if (lane == 0) {
-        unsigned long long c = (unsigned long long)(s.tile0 + tile) * 2;
-        ws.counts[c] = gt;
-        ws.counts[c + 1] = eq;
-    }
+    count_tile(s, rec, m.y, thr, lane, gt, eq);
+    if (lane == 0) *reinterpret_cast<uint2*>(ws.counts + (unsigned long long)gt_idx * 2) = make_uint2(gt, eq);
 }
 
 // ---- 5. scan ----------------------------------------------------------------------
 
 // In-place exclusive scan of nw {above, equal} pairs by one workgroup of
 // kScanBlock threads; returns the totals to every thread.  Each wavefront owns a
-// contiguous span: one coalesced sweep for the span totals, a second one that
-// scans 256 pairs at a time.
+// contiguous span.  The first sweep adds the span up, sixteen loads in flight per
+// lane, and leaves the pairs in LDS as 16 + 16 bits (a tile holds at most 4096 of
+// either kind); the second sweep scans 256 pairs at a time from there, so only its
+// stores touch memory.  Tensors beyond kScanStage tiles read memory twice.
 constexpr int kScanBlock = 1024;
 constexpr int kScanWaves = kScanBlock / 64;
-
-__device__ __forceinline__ unsigned wave_incl_scan(unsigned x, unsigned lane) {
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        unsigned y = (unsigned)__shfl_up((int)x, d, 64);
-        if ((int)lane >= d) x += y;
-    }
-    return x;
-}
+constexpr unsigned kScanStage = 32768;  // pairs that stay in LDS between the sweeps: 128 KiB
+constexpr int kScanBatch = 16;          // loads in flight per lane in the first sweep
 
 __device__ __forceinline__ void block_scan_pairs(uint32_t* c, unsigned nw, unsigned (&sh)[2][kScanWaves],
-                                                 unsigned& tot_gt, unsigned& tot_eq) {
+                                                 uint32_t* stage, unsigned& tot_gt, unsigned& tot_eq) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     uint2* c2 = reinterpret_cast<uint2*>(c);
+    const bool staged = nw <= kScanStage;
     const unsigned span = ((nw + kScanWaves - 1) / kScanWaves + 63u) & ~63u;
     const unsigned lo = wave * span < nw ? wave * span : nw;
     const unsigned hi = lo + span < nw ? lo + span : nw;
     unsigned sg = 0, se = 0;
-#pragma unroll 4
-    for (unsigned i = lo + lane; i < hi; i += 64) {
-        uint2 v = c2[i];
-        sg += v.x;
-        se += v.y;
+    for (unsigned i0 = lo + lane; i0 < hi; i0 += kScanBatch * 64) {
+        uint2 v[kScanBatch];
+#pragma unroll
+        for (int r = 0; r < kScanBatch; ++r) v[r] = i0 + r * 64 < hi ? c2[i0 + r * 64] : make_uint2(0u, 0u);
+#pragma unroll
+        for (int r = 0; r < kScanBatch; ++r) {
+            sg += v[r].x;
+            se += v[r].y;
+            if (staged && i0 + r * 64 < hi) stage[i0 + r * 64] = v[r].x | (v[r].y << 16);
+        }
     }
     sg = wave_sum_u(sg);
     se = wave_sum_u(se);
@@ -409,24 +408,37 @@ __device__ __forceinline__ void block_scan_pairs(uint32_t* c, unsigned nw, unsig
         tot_gt += g;
         tot_eq += e;
     }
-    // 256 pairs per trip: every lane owns four consecutive pairs, adds them up on its
-    // own, and one wavefront scan of the lane sums places them
+    // 256 pairs per trip as four rows of 64, lane l the l-th pair of every row: the
+    // eight wavefront scans of a trip are independent of each other and every store
+    // is one contiguous 512 bytes.  A wavefront reads back only what it staged itself.
     for (unsigned i0 = lo; i0 < hi; i0 += 256) {
-        const unsigned i = i0 + lane * 4;
         uint2 v[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = i + r < hi ? c2[i + r] : make_uint2(0u, 0u);
-        const unsigned lg = v[0].x + v[1].x + v[2].x + v[3].x, le = v[0].y + v[1].y + v[2].y + v[3].y;
-        const unsigned ig = wave_incl_scan(lg, lane), ie = wave_incl_scan(le, lane);
-        unsigned xg = bg + ig - lg, xe = be + ie - le;
+        unsigned ig[4], ie[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            if (i + r < hi) c2[i + r] = make_uint2(xg, xe);
-            xg += v[r].x;
-            xe += v[r].y;
+            const unsigned i = i0 + r * 64 + lane;
+            v[r] = make_uint2(0u, 0u);
+            if (i < hi) {
+                if (staged) {
+                    const unsigned w = stage[i];
+                    v[r] = make_uint2(w & 0xffffu, w >> 16);
+                } else {
+                    v[r] = c2[i];
+                }
+            }
         }
-        bg += (unsigned)__builtin_amdgcn_readlane((int)ig, 63);
-        be += (unsigned)__builtin_amdgcn_readlane((int)ie, 63);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            ig[r] = wave_incl_scan_u(v[r].x);
+            ie[r] = wave_incl_scan_u(v[r].y);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const unsigned i = i0 + r * 64 + lane;
+            if (i < hi) c2[i] = make_uint2(bg + ig[r] - v[r].x, be + ie[r] - v[r].y);
+            bg += (unsigned)__builtin_amdgcn_readlane((int)ig[r], 63);
+            be += (unsigned)__builtin_amdgcn_readlane((int)ie[r], 63);
+        }
     }
     __syncthreads();
 }
@@ -482,6 +494,7 @@ template <class SegSrc>
 __global__ __launch_bounds__(kScanBlock) void sparse_scan_kernel(SegSrc src, SparseWs ws) {
     __shared__ unsigned sh[2][kScanWaves];
     __shared__ RadixScratch sc;
+    __shared__ uint32_t stage[kScanStage];
     const Seg s = src.at(blockIdx.x);
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const unsigned nw = s.ntiles;
@@ -489,7 +502,7 @@ __global__ __launch_bounds__(kScanBlock) void sparse_scan_kernel(SegSrc src, Spa
     unsigned thr = ws.thr[2 * s.id];
     unsigned quota = kNoQuota;
     unsigned tot_gt, tot_eq;
-    block_scan_pairs(c, nw, sh, tot_gt, tot_eq);
+    block_scan_pairs(c, nw, sh, stage, tot_gt, tot_eq);
     unsigned long long total = (unsigned long long)tot_gt + tot_eq;
     if (total > s.cap) {
         // More candidates than slots: the threshold becomes the capacity-th largest
@@ -512,14 +525,14 @@ __global__ __launch_bounds__(kScanBlock) void sparse_scan_kernel(SegSrc src, Spa
         });
         for (unsigned t = wave; t < nw; t += kScanWaves) {
             unsigned gt, eq;
-            count_tile(s, ws, t, thr, lane, gt, eq);
+            count_tile(s, grec[(unsigned long long)t * 64 + lane], t, thr, lane, gt, eq);
             if (lane == 0) {
                 c[2 * t] = gt;
                 c[2 * t + 1] = eq;
             }
         }
         __syncthreads();
-        block_scan_pairs(c, nw, sh, tot_gt, tot_eq);
+        block_scan_pairs(c, nw, sh, stage, tot_gt, tot_eq);
         quota = s.cap - tot_gt;
         total = s.cap;
     }
@@ -550,16 +563,19 @@ __global__ __launch_bounds__(kBlock) void sparse_emit_kernel(Src src, SparseWs w
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const unsigned gt_idx = blockIdx.x * 4 + wave;
     if (gt_idx >= total_tiles) return;
-    unsigned tile;
-    const Seg s = src.get(tile, gt_idx);
+    // record and offsets need nothing but the tile's place in the launch, threshold and
+    // quota only the tensor's index: none of them waits for the descriptor
+    const uint2 rec = ws.grec[(unsigned long long)gt_idx * 64 + lane];
+    const uint2 before = *reinterpret_cast<const uint2*>(ws.counts + (unsigned long long)gt_idx * 2);
+    const uint2 m = src.where(gt_idx);
+    const uint2 tq = *reinterpret_cast<const uint2*>(ws.thr + 2 * m.x);
+    const Seg s = src.at(m.x);
+    const unsigned tile = m.y, thr = tq.x, quota = tq.y;
     const long long n = (long long)s.n;
-    const unsigned thr = ws.thr[2 * s.id], quota = ws.thr[2 * s.id + 1];
-    const unsigned long long ci = (unsigned long long)(s.tile0 + tile) * 2;
-    const unsigned G = ws.counts[ci], E = ws.counts[ci + 1];
+    const unsigned G = before.x, E = before.y;
     unsigned pos = G + (E < quota ? E : quota);  // pairs written by earlier tiles
     int32_t* idx = reinterpret_cast<int32_t*>(s.pay + kHeaderBytes);
     float* val = reinterpret_cast<float*>(s.pay + kHeaderBytes + 4ull * s.cap);
-    const uint2 rec = ws.grec[(unsigned long long)(s.tile0 + tile) * 64 + lane];
     const GroupView gv = view_group(rec, thr);
     if (quota == kNoQuota) {
         // Usual case: everything at or above the threshold is taken.  Lane l speaks for
@@ -733,7 +749,8 @@ __global__ __launch_bounds__(kBlock) void sparse_scatter_kernel(Src src) {
 // of order (their tiles were only cleared); workgroups of other tensors leave at once.
 __global__ __launch_bounds__(kBlock) void sparse_scatter_if_disordered_kernel(BatchSrc src, const uint32_t* disorder,
                                                                               unsigned epoch) {
-    if (disorder[src.map[blockIdx.x].x] != epoch) return;
+    if (disorder[0] != epoch) return;  // no payload of this call was out of order
+    if (disorder[1 + src.map[blockIdx.x].x] != epoch) return;
     unsigned ct;
     const Seg s = src.get(ct, blockIdx.x);
     scatter_slots(s, ct);
@@ -799,7 +816,10 @@ __global__ __launch_bounds__(kBlock) void sparse_decode_index_kernel(Src src, ui
         }
     }
     if (ct == 0 && threadIdx.x == 0 && nnz == 0 && nt) start(0, nt, 0u);
-    if (bad) disorder[s.id] = epoch;  // every writer stores the same value
+    if (bad) {  // every writer stores the same value; word 0 speaks for the whole table
+        disorder[1 + s.id] = epoch;
+        disorder[0] = epoch;
+    }
     __syncthreads();
     const unsigned ng = ngaps;
     for (unsigned g = 0; g < ng; ++g)
@@ -819,7 +839,7 @@ __global__ __launch_bounds__(kBlock) void sparse_decode_tile_kernel(Src src, con
     const float* val;
     const unsigned nnz = sparse_header(s.pay, s.cap, idx, val);
     unsigned lo = 0, hi = 0;  // a payload out of order: the tile is cleared here and filled by the scatter that follows
-    if (disorder[s.id] != epoch) {
+    if (disorder[1 + s.id] != epoch) {
         lo = tptr[s.tile0 + tile];
         hi = tile + 1 < s.ntiles ? tptr[s.tile0 + tile + 1] : nnz;
         if (hi > nnz) hi = nnz;
@@ -1044,7 +1064,8 @@ hipError_t launch_sparse_decode(const Launch& L, hipStream_t st) {
 }
 
 // Decode of a tensor table through tile pointers: tptr has one word per tile of the
-// launch, disorder one word per tensor; epoch must differ from call to call.
+// launch, disorder one word for the table and then one per tensor; epoch must differ
+// from call to call.
 // few_pairs: most tiles receive no or a handful of pairs, so the tile kernel is a plain
 // stream of stores and runs with the occupancy cap of one; with tens of pairs per tile
 // every workgroup waits on a chain of loads first and the cap would cost throughput.
