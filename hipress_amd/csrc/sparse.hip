@@ -372,6 +372,7 @@ __device__ __forceinline__ void block_scan_pairs(uint32_t* c, unsigned nw, unsig
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     uint2* c2 = reinterpret_cast<uint2*>(c);
     const bool staged = nw <= kScanStage;
+    const bool wide = (reinterpret_cast<unsigned long long>(c) & 15ull) == 0;  // a tensor may start at an odd tile
     const unsigned span = ((nw + kScanWaves - 1) / kScanWaves + 63u) & ~63u;
     const unsigned lo = wave * span < nw ? wave * span : nw;
     const unsigned hi = lo + span < nw ? lo + span : nw;
@@ -408,37 +409,38 @@ __device__ __forceinline__ void block_scan_pairs(uint32_t* c, unsigned nw, unsig
         tot_gt += g;
         tot_eq += e;
     }
-    // 256 pairs per trip as four rows of 64, lane l the l-th pair of every row: the
-    // eight wavefront scans of a trip are independent of each other and every store
-    // is one contiguous 512 bytes.  A wavefront reads back only what it staged itself.
+    // 256 pairs per trip: every lane owns four consecutive pairs, adds them up on its
+    // own, and one wavefront scan per kind of the lane sums places them (the scan's
+    // instructions, not memory, bound this kernel: one compute unit works through the
+    // largest tensor).  A wavefront reads back only what it staged itself.
     for (unsigned i0 = lo; i0 < hi; i0 += 256) {
+        const unsigned i = i0 + lane * 4;
         uint2 v[4];
-        unsigned ig[4], ie[4];
+        if (staged) {
+            const uint4 p = *reinterpret_cast<const uint4*>(&stage[i]);  // lo is a multiple of 64
+            const unsigned w[4] = {p.x, p.y, p.z, p.w};
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const unsigned i = i0 + r * 64 + lane;
-            v[r] = make_uint2(0u, 0u);
-            if (i < hi) {
-                if (staged) {
-                    const unsigned w = stage[i];
-                    v[r] = make_uint2(w & 0xffffu, w >> 16);
-                } else {
-                    v[r] = c2[i];
-                }
-            }
-        }
+            for (int r = 0; r < 4; ++r) v[r] = i + r < hi ? make_uint2(w[r] & 0xffffu, w[r] >> 16) : make_uint2(0u, 0u);
+        } else {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            ig[r] = wave_incl_scan_u(v[r].x);
-            ie[r] = wave_incl_scan_u(v[r].y);
+            for (int r = 0; r < 4; ++r) v[r] = i + r < hi ? c2[i + r] : make_uint2(0u, 0u);
         }
+        const unsigned lg = v[0].x + v[1].x + v[2].x + v[3].x, le = v[0].y + v[1].y + v[2].y + v[3].y;
+        const unsigned ig = wave_incl_scan_u(lg), ie = wave_incl_scan_u(le);
+        uint2 x[4];
+        x[0] = make_uint2(bg + ig - lg, be + ie - le);
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const unsigned i = i0 + r * 64 + lane;
-            if (i < hi) c2[i] = make_uint2(bg + ig[r] - v[r].x, be + ie[r] - v[r].y);
-            bg += (unsigned)__builtin_amdgcn_readlane((int)ig[r], 63);
-            be += (unsigned)__builtin_amdgcn_readlane((int)ie[r], 63);
+        for (int r = 1; r < 4; ++r) x[r] = make_uint2(x[r - 1].x + v[r - 1].x, x[r - 1].y + v[r - 1].y);
+        if (i + 3 < hi && wide) {  // two 16-byte stores
+            *reinterpret_cast<uint4*>(&c2[i]) = make_uint4(x[0].x, x[0].y, x[1].x, x[1].y);
+            *reinterpret_cast<uint4*>(&c2[i + 2]) = make_uint4(x[2].x, x[2].y, x[3].x, x[3].y);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (i + r < hi) c2[i + r] = x[r];
         }
+        bg += (unsigned)__builtin_amdgcn_readlane((int)ig, 63);
+        be += (unsigned)__builtin_amdgcn_readlane((int)ie, 63);
     }
     __syncthreads();
 }
@@ -494,7 +496,7 @@ template <class SegSrc>
 __global__ __launch_bounds__(kScanBlock) void sparse_scan_kernel(SegSrc src, SparseWs ws) {
     __shared__ unsigned sh[2][kScanWaves];
     __shared__ RadixScratch sc;
-    __shared__ uint32_t stage[kScanStage];
+    __shared__ __attribute__((aligned(16))) uint32_t stage[kScanStage + 256];  // a trip may read past the last pair
     const Seg s = src.at(blockIdx.x);
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const unsigned nw = s.ntiles;
