@@ -317,7 +317,7 @@ struct hipress_batch {
     uint2* d_smap = nullptr;  // sparse: sample tiles
     uint2* d_cmap = nullptr;  // sparse decode: payload-slot tiles
     uint32_t* d_tptr = nullptr;      // sparse decode: first payload slot of every tile
-    uint32_t* d_disorder = nullptr;  // sparse decode: the epoch in which a payload was last seen out of order, [0] any, [1 + i] tensor i
+    uint32_t* d_disorder = nullptr;  // sparse decode: per tensor, the epoch in which its payload was last seen out of order
     unsigned epoch = 0;
     unsigned ntiles = 0, nstiles = 0, nctiles = 0;
     void* ws = nullptr;  // onebit: one float per tile; sparse: SparseWsLayout
@@ -772,7 +772,7 @@ int hipress_batch_create(hipress_batch** out, int32_t alg, const hipress_tensor*
             for (unsigned j = 0; j < b->dec[i].ncblk; ++j) cmap.push_back(make_uint2((unsigned)i, j));
         b->nctiles = (unsigned)cmap.size();
         if ((rc = upload(cmap, &b->d_cmap))) return fail(rc);
-        const size_t tptr_bytes = 4 * (size_t)(b->ntiles ? b->ntiles : 1), flag_bytes = 4 * ((size_t)count + 1);
+        const size_t tptr_bytes = 4 * (size_t)(b->ntiles ? b->ntiles : 1), flag_bytes = 4 * (size_t)(count ? count : 1);
         if (hipMalloc(reinterpret_cast<void**>(&b->d_tptr), tptr_bytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
         if (hipMalloc(reinterpret_cast<void**>(&b->d_disorder), flag_bytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
         if (hipMemset(b->d_disorder, 0, flag_bytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);

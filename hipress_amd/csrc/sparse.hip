@@ -747,24 +747,15 @@ __global__ __launch_bounds__(kBlock) void sparse_scatter_kernel(Src src) {
     scatter_slots(s, ct);
 }
 
-// The same scatter for the tensors of a table whose payload the index kernel found out
-// of order (their tiles were only cleared); workgroups of other tensors leave at once.
-__global__ __launch_bounds__(kBlock) void sparse_scatter_if_disordered_kernel(BatchSrc src, const uint32_t* disorder,
-                                                                              unsigned epoch) {
-    if (disorder[0] != epoch) return;  // no payload of this call was out of order
-    if (disorder[1 + src.map[blockIdx.x].x] != epoch) return;
-    unsigned ct;
-    const Seg s = src.get(ct, blockIdx.x);
-    scatter_slots(s, ct);
-}
-
 // ---- decode with tile pointers (launches over a tensor table) -------------------------
 // A payload in ascending index order holds the pairs of a 4096-element tile as one
 // contiguous run.  The index kernel walks the payload once, records where every
 // tile's run starts and notices disorder; the tile kernel then builds each output
 // tile in LDS (zeros plus the tile's pairs) and writes it once, so no line of the
-// output is written twice.  The tensors whose payload is not in order are only
-// cleared by the tile kernel and then filled by a scatter launch.
+// output is written twice.  For a tensor whose payload is not in order every tile
+// looks through the whole payload instead of a run: correct, and slow in proportion
+// to tiles x pairs (this library's encoders, like the reference's, emit ascending
+// indices; the per-tensor decode scatters and does not care about order).
 
 // One workgroup per 1024 slots.  ptr[t] (t < ntiles) = first slot whose index lies in
 // tile t or later.  Slot j starts every tile after the tile of slot j-1 up to its
@@ -818,10 +809,7 @@ __global__ __launch_bounds__(kBlock) void sparse_decode_index_kernel(Src src, ui
         }
     }
     if (ct == 0 && threadIdx.x == 0 && nnz == 0 && nt) start(0, nt, 0u);
-    if (bad) {  // every writer stores the same value; word 0 speaks for the whole table
-        disorder[1 + s.id] = epoch;
-        disorder[0] = epoch;
-    }
+    if (bad) disorder[s.id] = epoch;  // every writer stores the same value
     __syncthreads();
     const unsigned ng = ngaps;
     for (unsigned g = 0; g < ng; ++g)
@@ -840,8 +828,8 @@ __global__ __launch_bounds__(kBlock) void sparse_decode_tile_kernel(Src src, con
     const int32_t* idx;
     const float* val;
     const unsigned nnz = sparse_header(s.pay, s.cap, idx, val);
-    unsigned lo = 0, hi = 0;  // a payload out of order: the tile is cleared here and filled by the scatter that follows
-    if (disorder[1 + s.id] != epoch) {
+    unsigned lo = 0, hi = nnz;  // a payload out of order: every pair is looked at
+    if (disorder[s.id] != epoch) {
         lo = tptr[s.tile0 + tile];
         hi = tile + 1 < s.ntiles ? tptr[s.tile0 + tile + 1] : nnz;
         if (hi > nnz) hi = nnz;
@@ -1066,8 +1054,7 @@ hipError_t launch_sparse_decode(const Launch& L, hipStream_t st) {
 }
 
 // Decode of a tensor table through tile pointers: tptr has one word per tile of the
-// launch, disorder one word for the table and then one per tensor; epoch must differ
-// from call to call.
+// launch, disorder one word per tensor; epoch must differ from call to call.
 // few_pairs: most tiles receive no or a handful of pairs, so the tile kernel is a plain
 // stream of stores and runs with the occupancy cap of one; with tens of pairs per tile
 // every workgroup waits on a chain of loads first and the cap would cost throughput.
@@ -1081,9 +1068,6 @@ hipError_t launch_sparse_decode_indexed(const Launch& L, uint32_t* tptr, uint32_
     BatchSrc src{L.dsegs, L.dmap};
     hipLaunchKernelGGL((sparse_decode_tile_kernel<BatchSrc>), dim3(L.ntiles), dim3(kBlock),
                        few_pairs ? kLdsFor4 - 4 * kTile : 0u, st, src, tptr, disorder, epoch);
-    if (L.nctiles)
-        hipLaunchKernelGGL(sparse_scatter_if_disordered_kernel, dim3(L.nctiles), dim3(kBlock), 0, st, csrc, disorder,
-                           epoch);
     return hipGetLastError();
 }
 

@@ -184,9 +184,13 @@ int hipress_sparse_decode_merge(const void *const *payloads, const int64_t *payl
  * algorithm does not use may be NULL.  A batch owns scratch memory on the device, so
  * calls on one batch must not overlap (one stream, or ordered by events); distinct
  * batches are independent.  All calls only enqueue kernels: they may be captured in a
- * HIP graph.  The sparse decode passes a per-call counter to its kernels, which a graph
- * freezes: in replays a tensor whose payload was once found out of order keeps taking
- * the slower scatter path (results stay correct). */
+ * HIP graph.  The batched sparse decode expects ascending indices, as this library's and
+ * the reference's encoders emit them; a payload out of order still decodes correctly,
+ * but every tile of that tensor then looks through its whole payload (time grows with
+ * tiles x pairs; hipress_sparse_decode scatters and does not care about order).  The
+ * decode passes a per-call counter to its kernels, which a graph freezes: in replays a
+ * tensor whose payload was once found out of order keeps taking that slow path
+ * (results stay correct). */
 typedef struct hipress_tensor {
     const float *grad;    /* encode input, fp32[n] */
     float *state0;        /* residual (onebit, tbq) | momentum (dgc) | accumulator (graddrop) */

@@ -569,7 +569,7 @@ def test_sparse_batch_decode_handmade_payloads(hp):
     Payloads made by hand: empty, one pair in a large tensor (long stretches of empty
     tiles), all slots used with the capacity a multiple of 1024, indices outside the
     tensor at both ends, a tensor shorter than a tile, and two payloads out of order
-    (decoded by the scatter fall-back) between ordered ones.  Two rounds with the payloads
+    (every tile then looks through the whole payload) between ordered ones.  Two rounds with the payloads
     exchanged between the rounds, since the batch keeps its pointers and flags."""
     rng = np.random.default_rng(123)
 
