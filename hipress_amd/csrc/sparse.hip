@@ -340,7 +340,8 @@ __device__ __forceinline__ void count_tile(const Seg& s, uint2 rec, unsigned til
 // One wavefront per tile, four tiles per workgroup.
 template <class Src>
 __global__ __launch_bounds__(kBlock) void sparse_count_kernel(Src src, SparseWs ws, unsigned total_tiles) {
-    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    // the wavefront's index as a scalar: what is addressed by it is then fetched by scalar loads
+    const unsigned lane = threadIdx.x & 63u, wave = (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const unsigned gt_idx = blockIdx.x * 4 + wave;
     if (gt_idx >= total_tiles) return;
     // the record needs nothing but the tile's place in the launch, the threshold only
@@ -562,7 +563,8 @@ __device__ __forceinline__ unsigned row_scan16(unsigned x) {
 
 template <class Src>
 __global__ __launch_bounds__(kBlock) void sparse_emit_kernel(Src src, SparseWs ws, unsigned total_tiles) {
-    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    // the wavefront's index as a scalar: what is addressed by it is then fetched by scalar loads
+    const unsigned lane = threadIdx.x & 63u, wave = (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const unsigned gt_idx = blockIdx.x * 4 + wave;
     if (gt_idx >= total_tiles) return;
     // record and offsets need nothing but the tile's place in the launch, threshold and
