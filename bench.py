@@ -31,14 +31,14 @@ MEASURED_TRAFFIC = {
     "onebit_deferred_vgg19": 1748885811,  # onebit_deferred_kernel
     "tbq_vgg19": 1765707366,              # tbq_encode_kernel
     "terngrad_vgg19": 1193284403,         # terngrad_encode_kernel
-    "dgc_vgg19": 2904915558,              # sparse_accum_kernel
-    "graddrop_vgg19": 1755467264,         # sparse_accum_kernel
+    "dgc_vgg19": 2904932454,              # sparse_accum_kernel
+    "graddrop_vgg19": 1755469209,         # sparse_accum_kernel
     "tbq_262144_x512": 1650560614,        # tbq_encode_kernel
     "terngrad_resnet50": 212500377,       # terngrad_encode_kernel
-    "dgc_bert_large": 6782786764,         # sparse_accum_kernel
-    "graddrop_bert_large": 4101440716,    # sparse_accum_kernel
+    "dgc_bert_large": 6782823833,         # sparse_accum_kernel
+    "graddrop_bert_large": 4101445222,    # sparse_accum_kernel
     "merge_tbq_vgg19": 2090605363,        # dense_merge_kernel
-    "merge_dgc_vgg19": 1780951961,        # sparse_merge_kernel
+    "merge_dgc_vgg19": 1780978995,        # sparse_merge_kernel
     "compll_b2_fc6": 848749465,           # compll_quant_kernel
     "compll_generated_b2_fc6": 848736665, # map_packed_kernel of the generated operator
 }
