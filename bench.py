@@ -37,7 +37,7 @@ MEASURED_TRAFFIC = {
     "terngrad_resnet50": 212500377,       # terngrad_encode_kernel
     "dgc_bert_large": 6782823833,         # sparse_accum_kernel
     "graddrop_bert_large": 4101445222,    # sparse_accum_kernel
-    "merge_tbq_vgg19": 2090605363,        # dense_merge_kernel
+    "merge_tbq_vgg19": 2090826240,        # dense_merge_kernel
     "merge_dgc_vgg19": 1780978995,        # sparse_merge_kernel
     "compll_b2_fc6": 848749465,           # compll_quant_kernel
     "compll_generated_b2_fc6": 848736665, # map_packed_kernel of the generated operator

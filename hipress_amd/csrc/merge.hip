@@ -33,61 +33,90 @@ __device__ __forceinline__ void merge_tile(const MergeSeg& m, unsigned tile, int
     const Seg s = m.s;
     const long long n = (long long)s.n;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
-    f4 agg[4];
+    f4 agg[4], rpre[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) agg[j] = (f4){0.f, 0.f, 0.f, 0.f};
-    for (int p = 0; p < npeers; ++p) {
-        const uint8_t* pay = m.peer[p];
-        if (ALG == HIPRESS_ONEBIT) {
-            const float sc = *reinterpret_cast<const float*>(pay);
-            const uint32_t* words = reinterpret_cast<const uint32_t*>(pay + kHeaderBytes);
-            const long long nwords = (n + 31) >> 5;
+    for (int j = 0; j < 4; ++j) {
+        agg[j] = (f4){0.f, 0.f, 0.f, 0.f};
+        // the aggregator's residual is requested first: it is in flight while the peers are added
+        if (REENC) rpre[j] = load4<FAST>(s.s0, base + j * 256 + lane * 4, n);
+    }
+    // Up to eight peers at a time.  First everything that comes from memory is requested:
+    // per peer one word per lane (the 1024 elements of the wavefront are 64 two-bit or 32
+    // one-bit words) and the scalar of its header.  Then the peers are added one after the
+    // other, each lane taking the word it needs from the lane that loaded it.
+    constexpr int kPeerChunk = 8;
+    for (int p0 = 0; p0 < npeers; p0 += kPeerChunk) {
+        uint32_t wq[kPeerChunk];
+        float sc[kPeerChunk];                // onebit: scale, tbq: threshold
+        const float* scales[kPeerChunk];     // terngrad
+        long long bucket[kPeerChunk];
+        bool use[kPeerChunk];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                long long widx = (base >> 5) + j * 8 + (lane >> 3);
-                uint32_t w = (FAST || widx < nwords) ? words[widx] : 0u;
-                unsigned nib = (w >> (4 * (lane & 7u))) & 0xfu;
-                f4 d;
-                d.x = (nib & 1u) ? sc : -sc;
-                d.y = (nib & 2u) ? sc : -sc;
-                d.z = (nib & 4u) ? sc : -sc;
-                d.w = (nib & 8u) ? sc : -sc;
-                agg[j] = agg[j] + d;
-            }
-        } else {
+        for (int q = 0; q < kPeerChunk; ++q) {
+            wq[q] = 0u;
+            sc[q] = 0.f;
+            scales[q] = nullptr;
+            bucket[q] = 1;
+            use[q] = p0 + q < npeers;
+            if (!use[q]) continue;
+            const uint8_t* pay = m.peer[p0 + q];
             const uint32_t* h = reinterpret_cast<const uint32_t*>(pay);
-            const long long nwords = (n + 15) >> 4;
-            const uint32_t* words;
-            const float* scales = nullptr;
-            float tau = 0.f;
-            long long B = 1;
-            if (ALG == HIPRESS_TBQ) {
-                tau = __uint_as_float(h[0]);
-                words = reinterpret_cast<const uint32_t*>(pay + kHeaderBytes);
+            if (ALG == HIPRESS_ONEBIT) {
+                sc[q] = __uint_as_float(h[0]);
+                const uint32_t* words = reinterpret_cast<const uint32_t*>(pay + kHeaderBytes);
+                const long long widx = (base >> 5) + lane;
+                if (lane < 32u && (FAST || widx < ((n + 31) >> 5))) wq[q] = words[widx];
             } else {
-                // bucket size from the header; a header that does not fit the buffer adds nothing
-                B = h[1];
-                unsigned long long nb = B >= 1 ? ((unsigned long long)n + B - 1) / B : 0;
-                unsigned long long off = kHeaderBytes + ((4 * nb + 15) & ~15ull);
-                if (B < 1 || off + 4 * (unsigned long long)nwords > m.peer_bytes[p]) continue;
-                scales = reinterpret_cast<const float*>(pay + kHeaderBytes);
-                words = reinterpret_cast<const uint32_t*>(pay + off);
+                const long long nwords = (n + 15) >> 4;
+                const uint32_t* words;
+                if (ALG == HIPRESS_TBQ) {
+                    sc[q] = __uint_as_float(h[0]);
+                    words = reinterpret_cast<const uint32_t*>(pay + kHeaderBytes);
+                } else {
+                    // bucket size from the header; a header that does not fit the buffer adds nothing
+                    const long long B = h[1];
+                    const unsigned long long nb = B >= 1 ? ((unsigned long long)n + B - 1) / B : 0;
+                    const unsigned long long off = kHeaderBytes + ((4 * nb + 15) & ~15ull);
+                    if (B < 1 || off + 4 * (unsigned long long)nwords > m.peer_bytes[p0 + q]) {
+                        use[q] = false;
+                        continue;
+                    }
+                    bucket[q] = B;
+                    scales[q] = reinterpret_cast<const float*>(pay + kHeaderBytes);
+                    words = reinterpret_cast<const uint32_t*>(pay + off);
+                }
+                const long long widx = (base >> 4) + lane;
+                if (FAST || widx < nwords) wq[q] = words[widx];
             }
+        }
+#pragma unroll
+        for (int q = 0; q < kPeerChunk; ++q) {
+            if (!use[q]) continue;  // wavefront-uniform
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                long long widx = (base >> 4) + j * 16 + (lane >> 2);
-                uint32_t w = (FAST || widx < nwords) ? words[widx] : 0u;
-                unsigned byte = (w >> (8 * (lane & 3u))) & 0xffu;
-                if (ALG == HIPRESS_TBQ) {
-                    agg[j] = agg[j] + expand_codes(byte, tau);
-                } else {
-                    long long e = base + j * 256 + lane * 4;
+                if (ALG == HIPRESS_ONEBIT) {
+                    const uint32_t w = (uint32_t)__shfl((int)wq[q], j * 8 + (int)(lane >> 3), 64);
+                    const unsigned nib = (w >> (4 * (lane & 7u))) & 0xfu;
                     f4 d;
-                    d.x = e < n ? code_val(byte & 3u, scales[e / B]) : 0.f;
-                    d.y = e + 1 < n ? code_val((byte >> 2) & 3u, scales[(e + 1) / B]) : 0.f;
-                    d.z = e + 2 < n ? code_val((byte >> 4) & 3u, scales[(e + 2) / B]) : 0.f;
-                    d.w = e + 3 < n ? code_val((byte >> 6) & 3u, scales[(e + 3) / B]) : 0.f;
+                    d.x = (nib & 1u) ? sc[q] : -sc[q];
+                    d.y = (nib & 2u) ? sc[q] : -sc[q];
+                    d.z = (nib & 4u) ? sc[q] : -sc[q];
+                    d.w = (nib & 8u) ? sc[q] : -sc[q];
                     agg[j] = agg[j] + d;
+                } else {
+                    const uint32_t w = (uint32_t)__shfl((int)wq[q], j * 16 + (int)(lane >> 2), 64);
+                    const unsigned byte = (w >> (8 * (lane & 3u))) & 0xffu;
+                    if (ALG == HIPRESS_TBQ) {
+                        agg[j] = agg[j] + expand_codes(byte, sc[q]);
+                    } else {
+                        const long long e = base + j * 256 + lane * 4, B = bucket[q];
+                        f4 d;
+                        d.x = e < n ? code_val(byte & 3u, scales[q][e / B]) : 0.f;
+                        d.y = e + 1 < n ? code_val((byte >> 2) & 3u, scales[q][(e + 1) / B]) : 0.f;
+                        d.z = e + 2 < n ? code_val((byte >> 4) & 3u, scales[q][(e + 2) / B]) : 0.f;
+                        d.w = e + 3 < n ? code_val((byte >> 6) & 3u, scales[q][(e + 3) / B]) : 0.f;
+                        agg[j] = agg[j] + d;
+                    }
                 }
             }
         }
@@ -101,8 +130,7 @@ __device__ __forceinline__ void merge_tile(const MergeSeg& m, unsigned tile, int
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             long long e = base + j * 256 + lane * 4;
-            f4 r = load4<FAST>(s.s0, e, n);
-            f4 v = r + agg[j];
+            f4 v = rpre[j] + agg[j];
             f4 keep;
             float k;
             unsigned byte = 0, c;
