@@ -304,7 +304,7 @@ def test_sparse_all_zero(hp):
 
 # ---------------------------------------------------------------- decode-and-merge
 @pytest.mark.parametrize("n", [1, 4097, 1048576])
-@pytest.mark.parametrize("npeers", [1, 8])
+@pytest.mark.parametrize("npeers", [1, 8, 9, 16])
 def test_tbq_decode_merge(hp, n, npeers):
     rng = np.random.default_rng(n + npeers)
     tau = 0.05
@@ -325,9 +325,10 @@ def test_tbq_decode_merge(hp, n, npeers):
     np.testing.assert_array_equal(host(r), want_r)
 
 
-def test_onebit_and_terngrad_decode_merge(hp):
-    n, P = 70001, 5
-    rng = np.random.default_rng(9)
+@pytest.mark.parametrize("P", [5, 13])
+def test_onebit_and_terngrad_decode_merge(hp, P):
+    n = 70001
+    rng = np.random.default_rng(9 + P)
     ob = [oracle.onebit_encode(rng.normal(0, 1, n).astype(F), np.zeros(n, F))[0] for _ in range(P)]
     agg = torch.empty(n, device="cuda")
     hp.onebit_decode_merge([dev(p) for p in ob], agg)
@@ -336,6 +337,22 @@ def test_onebit_and_terngrad_decode_merge(hp):
         tg = [oracle.terngrad_encode(rng.normal(0, 1, n).astype(F), rng.random(n, dtype=F), bucket) for _ in range(P)]
         hp.terngrad_decode_merge([dev(p) for p in tg], agg)
         np.testing.assert_array_equal(host(agg), oracle.terngrad_decode_merge(tg, n))
+
+
+def test_terngrad_decode_merge_skips_a_peer_whose_header_does_not_fit(hp):
+    """A peer whose header names a bucket size of zero, or one whose scales and words
+    would not fit its buffer, adds nothing; the other peers are summed as usual."""
+    n, bucket = 20000, 512
+    rng = np.random.default_rng(31)
+    tg = [oracle.terngrad_encode(rng.normal(0, 1, n).astype(F), rng.random(n, dtype=F), bucket) for _ in range(3)]
+    zero_bucket = tg[1].copy()
+    zero_bucket[4:8] = 0          # header word 1 = bucket size
+    tiny_bucket = tg[1].copy()
+    tiny_bucket[4:8] = np.frombuffer(np.uint32(1).tobytes(), np.uint8)  # n scales would not fit the buffer
+    agg = torch.empty(n, device="cuda")
+    for bad in (zero_bucket, tiny_bucket):
+        hp.terngrad_decode_merge([dev(tg[0]), dev(bad), dev(tg[2])], agg)
+        np.testing.assert_array_equal(host(agg), oracle.terngrad_decode_merge([tg[0], tg[2]], n))
 
 
 @pytest.mark.parametrize("n", [1000, 1048576])
