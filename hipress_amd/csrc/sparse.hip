@@ -1058,8 +1058,12 @@ hipError_t launch_sparse_decode(const Launch& L, hipStream_t st) {
 // Decode of a tensor table through tile pointers: tptr has one word per tile of the
 // launch, disorder one word per tensor; epoch must differ from call to call.
 // few_pairs: most tiles receive no or a handful of pairs, so the tile kernel is a plain
-// stream of stores and runs with the occupancy cap of one; with tens of pairs per tile
-// every workgroup waits on a chain of loads first and the cap would cost throughput.
+// stream of stores and runs with the occupancy cap of one.  With tens of pairs per tile
+// every workgroup waits on a chain of loads first; five workgroups per CU still move
+// more bytes then (6-13 %) as long as the launch writes less than about 1 GiB, and fewer
+// beyond (5-9 % at 1.3-1.6 GiB, measured on MI355X: the crossover is at 65,536 tiles), so
+// the cap is applied below 57,344 tiles only.
+constexpr unsigned kTileCapTiles = 57344;
 hipError_t launch_sparse_decode_indexed(const Launch& L, uint32_t* tptr, uint32_t* disorder, unsigned epoch,
                                         bool few_pairs, hipStream_t st) {
     if (L.ntiles == 0 || L.single) return hipSuccess;
@@ -1069,7 +1073,8 @@ hipError_t launch_sparse_decode_indexed(const Launch& L, uint32_t* tptr, uint32_
                            disorder, epoch);
     BatchSrc src{L.dsegs, L.dmap};
     hipLaunchKernelGGL((sparse_decode_tile_kernel<BatchSrc>), dim3(L.ntiles), dim3(kBlock),
-                       few_pairs ? kLdsFor4 - 4 * kTile : 0u, st, src, tptr, disorder, epoch);
+                       few_pairs ? kLdsFor4 - 4 * kTile : (L.ntiles <= kTileCapTiles ? kLdsFor5 - 4 * kTile : 0u), st, src, tptr,
+                       disorder, epoch);
     return hipGetLastError();
 }
 
