@@ -632,13 +632,24 @@ __global__ __launch_bounds__(kBlock) void terngrad_decode_kernel(Src src) {
         return hipGetLastError();                                                             \
     } while (0)
 
+// The decoders' cap pays while the payload they read (per_tile bytes for every 4096
+// elements) still fits the 256 MiB memory-side cache, where the encoder left it; once it
+// no longer does, the decoders run at about 5 instead of 6.5 TB/s and the cap costs
+// another 15 % (measured on sets of 0.8 to 1.6 G elements: the step in tbq decode lies
+// between 268 and 302 MB of payload, in onebit decode beyond 200 MB).
+static unsigned decode_cap(const Launch& L, unsigned per_tile) {
+    return (unsigned long long)L.ntiles * per_tile <= (192ull << 20) ? kLdsFor5 : 0u;
+}
+
 hipError_t launch_tbq_encode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_encode_kernel, kLdsFor5, L, st); }
-hipError_t launch_tbq_decode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_decode_kernel, kLdsFor5, L, st); }
-hipError_t launch_onebit_decode(const Launch& L, hipStream_t st) { HP_LAUNCH(onebit_decode_kernel, kLdsFor5, L, st); }
+hipError_t launch_tbq_decode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_decode_kernel, decode_cap(L, kTile / 4), L, st); }
+hipError_t launch_onebit_decode(const Launch& L, hipStream_t st) {
+    HP_LAUNCH(onebit_decode_kernel, decode_cap(L, kTile / 8), L, st);
+}
 // A single-tensor call learns the bucket size from the header on the device, a chain of
 // dependent loads that wants full occupancy; a table launch carries it in the descriptors.
 hipError_t launch_terngrad_decode(const Launch& L, hipStream_t st) {
-    HP_LAUNCH(terngrad_decode_kernel, (L.single ? 0u : kLdsFor5), L, st);
+    HP_LAUNCH(terngrad_decode_kernel, (L.single ? 0u : decode_cap(L, kTile / 4)), L, st);
 }
 
 static hipError_t onebit_abs(const Launch& L, float* partial, hipStream_t st) {

@@ -1062,8 +1062,10 @@ hipError_t launch_sparse_decode(const Launch& L, hipStream_t st) {
 // every workgroup waits on a chain of loads first; five workgroups per CU still move
 // more bytes then (6-13 %) as long as the launch writes less than about 1 GiB, and fewer
 // beyond (5-9 % at 1.3-1.6 GiB, measured on MI355X: the crossover is at 65,536 tiles), so
-// the cap is applied below 57,344 tiles only.
-constexpr unsigned kTileCapTiles = 57344;
+// the cap is applied below 57,344 tiles only.  The cap of the few-pairs case pays up to
+// 262,144 tiles (4 GiB written: +10 % at 98,304 tiles, +1.5 % at 262,144) and costs 9 % at
+// 393,216.
+constexpr unsigned kTileCapTiles = 57344, kFewPairsCapTiles = 262144;
 hipError_t launch_sparse_decode_indexed(const Launch& L, uint32_t* tptr, uint32_t* disorder, unsigned epoch,
                                         bool few_pairs, hipStream_t st) {
     if (L.ntiles == 0 || L.single) return hipSuccess;
@@ -1073,8 +1075,9 @@ hipError_t launch_sparse_decode_indexed(const Launch& L, uint32_t* tptr, uint32_
                            disorder, epoch);
     BatchSrc src{L.dsegs, L.dmap};
     hipLaunchKernelGGL((sparse_decode_tile_kernel<BatchSrc>), dim3(L.ntiles), dim3(kBlock),
-                       few_pairs ? kLdsFor4 - 4 * kTile : (L.ntiles <= kTileCapTiles ? kLdsFor5 - 4 * kTile : 0u), st, src, tptr,
-                       disorder, epoch);
+                       few_pairs ? (L.ntiles <= kFewPairsCapTiles ? kLdsFor4 - 4 * kTile : 0u)
+                                 : (L.ntiles <= kTileCapTiles ? kLdsFor5 - 4 * kTile : 0u),
+                       st, src, tptr, disorder, epoch);
     return hipGetLastError();
 }
 
