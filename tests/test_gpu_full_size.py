@@ -370,3 +370,88 @@ def test_hip_graph_replay_of_a_sparse_batch(hp):
             np.testing.assert_array_equal(host(t["accumulator"]), acc, err_msg=f"accumulator, replay {step}")
             np.testing.assert_array_equal(host(t["out"]), out, err_msg=f"decode, replay {step}")
     b.close()
+
+
+# ---------------------------------------------------------------- beyond the benchmark's sizes
+# Above certain launch sizes the batched decoders are started with a different
+# occupancy (the caps stop paying there).  The oracle would take minutes at these sizes:
+# the batched decode is compared with the per-tensor entry point, which takes other
+# launch paths (single-tensor kernels; zero fill + scatter for the sparse formats), and
+# the encode with properties that hold at any size.
+
+def _uniform_set(count, n, sigma, seed):
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    return [torch.randn(n, generator=gen, device="cuda") * sigma for _ in range(count)]
+
+
+def test_graddrop_batch_decode_of_a_large_launch_matches_the_per_tensor_decode(hp):
+    """~240 M elements at one per cent: more tiles than the sparse tile decode's cap covers."""
+    sizes = [64 << 20, 64 << 20, 64 << 20, (48 << 20) + 1]
+    ratio = 0.01
+    ts = []
+    for i, n in enumerate(sizes):
+        g = _uniform_set(1, n, 1e-3, 40 + i)[0]
+        ts.append({"gradient": g, "accumulator": torch.zeros_like(g), "out": torch.full_like(g, 7.0),
+                   "compressed": torch.zeros(hp.graddrop_payload_bytes(n, ratio), dtype=torch.uint8, device="cuda")})
+    b = hp.Batch("graddrop", ts, ratio=ratio)
+    assert sum((n + 4095) // 4096 for n in sizes) > 57344
+    b.encode()
+    b.decode()
+    for t in ts:
+        n = t["gradient"].numel()
+        single = torch.full_like(t["out"], -3.0)
+        hp.graddrop_decode(t["compressed"], single)
+        assert torch.equal(t["out"], single)
+        nnz = int(t["compressed"][:4].view(torch.int32).item())
+        assert 0.5 * ratio * n < nnz < 2.0 * ratio * n
+        assert int((t["out"] != 0).sum().item()) == nnz
+        # what was sent plus what stays is the gradient (first step: accumulator started at zero)
+        assert torch.equal(t["out"] + t["accumulator"], t["gradient"])
+    b.close()
+
+
+def test_tbq_batch_decode_with_a_payload_beyond_the_cache_matches_the_per_tensor_decode(hp):
+    """~870 M elements: 218 MB of packed words, more than the decoders' cap covers."""
+    n, count, tau = 64 << 20, 13, 0.05
+    ts = []
+    for i in range(count):
+        g = _uniform_set(1, n, 0.04, 60 + i)[0]
+        ts.append({"gradient": g, "residual": torch.zeros_like(g), "out": torch.empty_like(g),
+                   "compressed": torch.zeros(hp.tbq_payload_bytes(n), dtype=torch.uint8, device="cuda")})
+    assert count * (n // 4) > (192 << 20)
+    b = hp.Batch("tbq", ts, threshold=tau)
+    b.encode()
+    b.decode()
+    single = torch.empty(n, device="cuda")
+    for t in ts:
+        hp.tbq_decode(t["compressed"], single)
+        assert torch.equal(t["out"], single)
+        g, out = t["gradient"], t["out"]
+        want = torch.where(g >= tau, torch.full_like(g, tau), torch.where(g <= -tau, torch.full_like(g, -tau), torch.zeros_like(g)))
+        assert torch.equal(out, want)
+        assert torch.equal(t["residual"], g - out)
+    b.close()
+
+
+def test_dgc_batch_decode_of_a_very_large_launch_matches_the_per_tensor_decode(hp):
+    """~1.14 G elements at 0.1 per cent: more tiles than the few-pairs cap covers."""
+    n, count, ratio = 64 << 20, 17, 0.001
+    ts = []
+    for i in range(count):
+        g = _uniform_set(1, n, 1e-3, 80 + i)[0]
+        ts.append({"gradient": g, "momentum": torch.zeros_like(g), "accumulator": torch.zeros_like(g),
+                   "out": torch.full_like(g, 7.0),
+                   "compressed": torch.zeros(hp.dgc_payload_bytes(n, ratio), dtype=torch.uint8, device="cuda")})
+    assert count * (n // 4096) > 262144
+    b = hp.Batch("dgc", ts, momentum_factor=0.9, ratio=ratio)
+    b.encode()
+    b.decode()
+    single = torch.empty(n, device="cuda")
+    for t in ts:
+        hp.dgc_decode(t["compressed"], single)
+        assert torch.equal(t["out"], single)
+        nnz = int(t["compressed"][:4].view(torch.int32).item())
+        assert 0.5 * ratio * n < nnz < 2.0 * ratio * n
+        assert int((t["out"] != 0).sum().item()) == nnz
+        assert torch.equal(t["out"] + t["accumulator"], t["gradient"])
+    b.close()
