@@ -213,7 +213,9 @@ __device__ __forceinline__ float wave_max(float x) {
 }
 // Inclusive prefix sum over the 64 lanes in six data-parallel-primitive steps:
 // four shifts inside every row of 16 lanes, then lane 15 of rows 0 and 2 is added
-// to the row after it, then lane 31 to the upper two rows.
+// to the row after it, then lane 31 to the upper two rows.  All 64 lanes must be active
+// where it is called (a lane that is switched off would be read as garbage by its
+// neighbours).
 __device__ __forceinline__ unsigned wave_incl_scan_u(unsigned x) {
     x += (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x111, 0xf, 0xf, true);   // row_shr:1
     x += (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x112, 0xf, 0xf, true);   // row_shr:2
