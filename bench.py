@@ -163,8 +163,9 @@ class MergeWorkload:
     """Decode-and-merge of 8 peer payloads per 4 MB chunk of the VGG19 set, with the
     fused re-encode for the next hop."""
 
-    def __init__(self, name, alg, sizes, npeers=8):
+    def __init__(self, name, alg, sizes, npeers=8, aggregate=True):
         self.name, self.alg, self.sizes, self.npeers = name, alg, sizes, npeers
+        self.aggregate = aggregate  # False: only the re-encoded payload is produced (no fp32 sum written)
         self.elements = sum(sizes)
         self.dominant_phase = 0
         self.nphases = 1
@@ -182,7 +183,8 @@ class MergeWorkload:
         for n in self.sizes:
             nb = hp.tbq_payload_bytes(n) if self.alg == "tbq" else hp.dgc_payload_bytes(n, ratio)
             chunks.append({"compressed": [torch.zeros(nb, dtype=torch.uint8, device=dev) for _ in range(self.npeers)],
-                           "aggregate": torch.empty(n, device=dev), "state": torch.zeros(n, device=dev),
+                           "aggregate": torch.empty(n, device=dev) if self.aggregate else None,
+                           "state": torch.zeros(n, device=dev),
                            "out_compressed": torch.zeros(nb, dtype=torch.uint8, device=dev)})
         # peer p's payloads come from that peer's own gradients (seed p) through the encoders
         for p in range(self.npeers):
@@ -202,12 +204,13 @@ class MergeWorkload:
             del grads, ts
         self.chunks = chunks
         self.mb = hp.MergeBatch(self.alg, chunks, threshold=tau, ratio=ratio)
+        agg_bytes = 4.0 if self.aggregate else 0.0
         if self.alg == "tbq":
-            self.enc_bytes, self.dec_bytes = 0.25 * self.npeers + 4 + 8.25, 0.0
+            self.enc_bytes, self.dec_bytes = 0.25 * self.npeers + agg_bytes + 8.25, 0.0
             self.dominant_kernel, self.dominant_bytes = "dense_merge_kernel", self.enc_bytes
         else:
-            self.enc_bytes, self.dec_bytes = 12.0, 0.0  # + 8*(P*rho + rho'), added after the run
-            self.dominant_kernel, self.dominant_bytes = "sparse_merge_kernel", 12.0
+            self.enc_bytes, self.dec_bytes = 8.0 + agg_bytes, 0.0  # + 8*(P*rho + rho'), added after the run
+            self.dominant_kernel, self.dominant_bytes = "sparse_merge_kernel", 8.0 + agg_bytes
 
     def step(self, ev=None):
         if ev is not None and self.alg == "tbq":
@@ -352,13 +355,17 @@ def make_workload(name):
         return MergeWorkload(name, "tbq", W.chunk_sizes(vgg))
     if name == "merge_dgc_vgg19":
         return MergeWorkload(name, "dgc", W.chunk_sizes(vgg))
+    if name == "merge_tbq_vgg19_payload_only":
+        return MergeWorkload(name, "tbq", W.chunk_sizes(vgg), aggregate=False)
+    if name == "merge_dgc_vgg19_payload_only":
+        return MergeWorkload(name, "dgc", W.chunk_sizes(vgg), aggregate=False)
     raise SystemExit(f"unknown workload {name}")
 
 
 ALL_WORKLOADS = [
     "onebit_vgg19", "onebit_deferred_vgg19", "tbq_vgg19", "terngrad_vgg19", "dgc_vgg19", "graddrop_vgg19", "tbq_262144", "tbq_262144_x512",
     "terngrad_resnet50", "dgc_bert_large", "graddrop_bert_large", "merge_tbq_vgg19", "merge_dgc_vgg19", "compll_b2_fc6",
-    "compll_generated_b2_fc6", "tbq_fc6", "tbq_generated_fc6",
+    "compll_generated_b2_fc6", "tbq_fc6", "tbq_generated_fc6", "merge_tbq_vgg19_payload_only", "merge_dgc_vgg19_payload_only",
 ]
 
 

@@ -575,12 +575,13 @@ int hipress_sparse_decode(const void* payload, int64_t payload_bytes, float* out
 
 // ---- decode-and-merge ------------------------------------------------------------------
 
+// reencode: the call also re-encodes the sum; only then may the aggregate be left out.
 static int build_merge_seg(int alg, const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
-                           float* aggregate, int64_t n, MergeSeg* m) {
+                           float* aggregate, int64_t n, bool reencode, MergeSeg* m) {
     std::memset(m, 0, sizeof(MergeSeg));
     if (bad_n(n)) return HIPRESS_ERR_SIZE;
     if (npeers < 1 || npeers > HIPRESS_MAX_PEERS) return HIPRESS_ERR_PARAM;
-    if (!payloads || !payload_bytes || (n > 0 && !aggregate)) return HIPRESS_ERR_NULL;
+    if (!payloads || !payload_bytes || (n > 0 && !aggregate && !reencode)) return HIPRESS_ERR_NULL;
     if (mis(aggregate, 4)) return HIPRESS_ERR_ALIGN;
     for (int p = 0; p < npeers; ++p) {
         if (!payloads[p]) return HIPRESS_ERR_NULL;
@@ -629,7 +630,7 @@ int hipress_tbq_decode_merge(const void* const* payloads, const int64_t* payload
                              float* aggregate, int64_t n, float* residual, void* out_payload,
                              int64_t out_payload_bytes, float threshold, void* stream) {
     MergeSeg m;
-    int rc = build_merge_seg(HIPRESS_TBQ, payloads, payload_bytes, npeers, aggregate, n, &m);
+    int rc = build_merge_seg(HIPRESS_TBQ, payloads, payload_bytes, npeers, aggregate, n, residual != nullptr, &m);
     if (rc) return rc;
     if (residual && (rc = add_tbq_reencode(&m, residual, out_payload, out_payload_bytes, threshold))) return rc;
     return hiperr(launch_dense_merge(single_merge_launch(m, npeers, residual != nullptr), HIPRESS_TBQ,
@@ -639,7 +640,7 @@ int hipress_tbq_decode_merge(const void* const* payloads, const int64_t* payload
 int hipress_onebit_decode_merge(const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
                                 float* aggregate, int64_t n, void* stream) {
     MergeSeg m;
-    int rc = build_merge_seg(HIPRESS_ONEBIT, payloads, payload_bytes, npeers, aggregate, n, &m);
+    int rc = build_merge_seg(HIPRESS_ONEBIT, payloads, payload_bytes, npeers, aggregate, n, false, &m);
     if (rc) return rc;
     return hiperr(launch_dense_merge(single_merge_launch(m, npeers, false), HIPRESS_ONEBIT,
                                      static_cast<hipStream_t>(stream)));
@@ -648,7 +649,7 @@ int hipress_onebit_decode_merge(const void* const* payloads, const int64_t* payl
 int hipress_terngrad_decode_merge(const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
                                   float* aggregate, int64_t n, void* stream) {
     MergeSeg m;
-    int rc = build_merge_seg(HIPRESS_TERNGRAD, payloads, payload_bytes, npeers, aggregate, n, &m);
+    int rc = build_merge_seg(HIPRESS_TERNGRAD, payloads, payload_bytes, npeers, aggregate, n, false, &m);
     if (rc) return rc;
     return hiperr(launch_dense_merge(single_merge_launch(m, npeers, false), HIPRESS_TERNGRAD,
                                      static_cast<hipStream_t>(stream)));
@@ -670,14 +671,15 @@ int hipress_sparse_decode_merge(const void* const* payloads, const int64_t* payl
                                 int64_t out_payload_bytes, double ratio, void* workspace,
                                 int64_t workspace_bytes, void* stream) {
     MergeSeg m;
-    int rc = build_merge_seg(HIPRESS_DGC, payloads, payload_bytes, npeers, aggregate, n, &m);
+    int rc = build_merge_seg(HIPRESS_DGC, payloads, payload_bytes, npeers, aggregate, n, accumulator != nullptr, &m);
     if (rc) return rc;
     SparseWsLayout l{};
     const int64_t tp_words = (int64_t)npeers * (m.s.ntiles + 1);
     const int64_t ibytes = merge_index_bytes(tp_words, 1, npeers);
     int64_t need = ibytes;
     if (accumulator) {
-        hipress_tensor t{aggregate, accumulator, nullptr, nullptr, out_payload, nullptr, n, out_payload_bytes};
+        // the gradient of this descriptor is never read (the merge kernel takes the sum from LDS): any valid pointer passes its checks
+        hipress_tensor t{aggregate ? aggregate : accumulator, accumulator, nullptr, nullptr, out_payload, nullptr, n, out_payload_bytes};
         hipress_params pr{};
         pr.ratio = ratio;
         if ((rc = build_encode_seg(HIPRESS_GRADDROP, t, pr, &m.r))) return rc;
@@ -892,12 +894,12 @@ int hipress_merge_batch_create(hipress_merge_batch** out, int32_t alg, const hip
     for (int i = 0; i < count; ++i) {
         const hipress_merge_chunk& c = chunks[i];
         MergeSeg m;
-        if ((rc = build_merge_seg(alg, c.payloads, c.payload_bytes, npeers, c.aggregate, c.n, &m))) return fail(rc);
+        if ((rc = build_merge_seg(alg, c.payloads, c.payload_bytes, npeers, c.aggregate, c.n, b->reencode, &m))) return fail(rc);
         if (b->reencode && alg == HIPRESS_TBQ) {
             if ((rc = add_tbq_reencode(&m, c.state, c.out_payload, c.out_payload_bytes, params->threshold))) return fail(rc);
         }
         if (b->reencode && sparse) {
-            hipress_tensor t{c.aggregate, c.state, nullptr, nullptr, c.out_payload, nullptr, c.n, c.out_payload_bytes};
+            hipress_tensor t{c.aggregate ? c.aggregate : c.state, c.state, nullptr, nullptr, c.out_payload, nullptr, c.n, c.out_payload_bytes};
             Seg s;
             if ((rc = build_encode_seg(HIPRESS_GRADDROP, t, *params, &s))) return fail(rc);
             b->renc.push_back(s);

@@ -122,7 +122,8 @@ __device__ __forceinline__ void merge_tile(const MergeSeg& m, unsigned tile, int
         }
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) store4<FAST>(s.out, base + j * 256 + lane * 4, n, agg[j]);
+    for (int j = 0; j < 4; ++j)
+        if (s.out) store4<FAST>(s.out, base + j * 256 + lane * 4, n, agg[j]);  // a re-encoding call may leave the aggregate out
     if (REENC) {
         const float tau = s.f0;
         uint32_t* owords = reinterpret_cast<uint32_t*>(s.pay + kHeaderBytes);

@@ -990,11 +990,13 @@ __global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs
     }
     __syncthreads();
     auto from_lds = [&](int j, long long) { return *reinterpret_cast<const f4*>(&lds[wave * kWaveTile + j * 256 + lane * 4]); };
+    if (s.out) {  // a re-encoding call may leave the aggregate out
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        long long e = t_lo + wave * kWaveTile + j * 256 + lane * 4;
-        if (fast) st4(s.out + e, from_lds(j, e));
-        else st4_guard(s.out, e, n, from_lds(j, e));
+        for (int j = 0; j < 4; ++j) {
+            long long e = t_lo + wave * kWaveTile + j * 256 + lane * 4;
+            if (fast) st4(s.out + e, from_lds(j, e));
+            else st4_guard(s.out, e, n, from_lds(j, e));
+        }
     }
     if (REENC) {
         if (tile == 0) sparse_reset_select(r, ws);

@@ -285,16 +285,21 @@ def _peers(compressed_list, like):
 
 def tbq_decode_merge(compressed_list, aggregate, residual=None, out_compressed=None, threshold=0.0):
     """aggregate = sum of the decoded peers; with `residual` given the aggregate is
-    re-encoded into `out_compressed` with the aggregator's own residual."""
-    _f32(aggregate, "aggregate")
-    ptrs, lens, P = _peers(compressed_list, aggregate)
+    re-encoded into `out_compressed` with the aggregator's own residual, and `aggregate`
+    may then be None (only the re-encoded payload is produced)."""
+    like = aggregate if aggregate is not None else residual
+    if like is None:
+        raise TypeError("aggregate may only be None when residual and out_compressed are given")
+    if aggregate is not None:
+        _f32(aggregate, "aggregate")
+    ptrs, lens, P = _peers(compressed_list, like)
     if residual is not None:
-        _f32(residual, "residual", aggregate); _u8(out_compressed, "out_compressed", aggregate)
-        _same_numel(aggregate, residual, "aggregate", "residual")
-    with _on(aggregate.device):
+        _f32(residual, "residual", like); _u8(out_compressed, "out_compressed", like)
+        _same_numel(like, residual, "aggregate", "residual")
+    with _on(like.device):
         check(_lib.lib().hipress_tbq_decode_merge(
-            ptrs, lens, P, _p(aggregate), aggregate.numel(), _p(residual), _p(out_compressed),
-            out_compressed.numel() if out_compressed is not None else 0, float(threshold), _stream(aggregate)),
+            ptrs, lens, P, _p(aggregate), like.numel(), _p(residual), _p(out_compressed),
+            out_compressed.numel() if out_compressed is not None else 0, float(threshold), _stream(like)),
             "tbq_decode_merge")
 
 
@@ -316,22 +321,27 @@ def terngrad_decode_merge(compressed_list, aggregate):
 
 def dgc_decode_merge(compressed_list, aggregate, accumulator=None, out_compressed=None, ratio=0.001):
     """Scatter-add of the peers' (index, value) pairs; with `accumulator` given the
-    aggregate is re-sparsified into `out_compressed` (accumulator = aggregator residual)."""
-    _f32(aggregate, "aggregate")
-    ptrs, lens, P = _peers(compressed_list, aggregate)
+    aggregate is re-sparsified into `out_compressed` (accumulator = aggregator residual),
+    and `aggregate` may then be None (only the re-encoded payload is produced)."""
+    like = aggregate if aggregate is not None else accumulator
+    if like is None:
+        raise TypeError("aggregate may only be None when accumulator and out_compressed are given")
+    if aggregate is not None:
+        _f32(aggregate, "aggregate")
+    ptrs, lens, P = _peers(compressed_list, like)
     L = _lib.lib()
-    n = aggregate.numel()
+    n = like.numel()
     ws = None
     if accumulator is not None:
-        _f32(accumulator, "accumulator", aggregate); _u8(out_compressed, "out_compressed", aggregate)
-        _same_numel(aggregate, accumulator, "aggregate", "accumulator")
-    with _on(aggregate.device):
-        ws = _workspace(aggregate, size(L.hipress_sparse_merge_workspace_bytes(n, P, float(ratio), int(accumulator is not None)),
-                                        "sparse_merge_workspace_bytes"))
+        _f32(accumulator, "accumulator", like); _u8(out_compressed, "out_compressed", like)
+        _same_numel(like, accumulator, "aggregate", "accumulator")
+    with _on(like.device):
+        ws = _workspace(like, size(L.hipress_sparse_merge_workspace_bytes(n, P, float(ratio), int(accumulator is not None)),
+                                   "sparse_merge_workspace_bytes"))
         check(L.hipress_sparse_decode_merge(
             ptrs, lens, P, _p(aggregate), n, _p(accumulator), _p(out_compressed),
             out_compressed.numel() if out_compressed is not None else 0, float(ratio),
-            _p(ws), ws.numel() if ws is not None else 0, _stream(aggregate)), "sparse_decode_merge")
+            _p(ws), ws.numel() if ws is not None else 0, _stream(like)), "sparse_decode_merge")
 
 
 graddrop_decode_merge = dgc_decode_merge
@@ -412,6 +422,8 @@ class MergeBatch:
     ``chunks``: list of dicts with ``compressed`` (list of peer payload tensors),
     ``aggregate``, and optionally ``state`` + ``out_compressed`` for the fused
     re-encode (tbq: aggregator residual; dgc/graddrop: aggregator accumulator).
+    With the re-encode a chunk's ``aggregate`` may be None: the sum is then not
+    written as fp32, only the re-encoded payload and the state are produced.
     """
 
     def __init__(self, alg, chunks, threshold=0.0, bucket=512, ratio=0.001):
@@ -420,21 +432,26 @@ class MergeBatch:
         arr = (MergeChunk * max(len(chunks), 1))()
         dev = None
         for i, c in enumerate(chunks):
-            agg = _f32(c["aggregate"], "aggregate")
-            dev = dev or agg.device
+            st, oc = c.get("state"), c.get("out_compressed")
+            agg = c.get("aggregate")
+            like = agg if agg is not None else st
+            if like is None:
+                raise TypeError("a chunk needs an aggregate, or a state and out_compressed to re-encode into")
+            if agg is not None:
+                _f32(agg, "aggregate")
+            dev = dev or like.device
             if len(c["compressed"]) != npeers:
                 raise ValueError("every chunk must have the same number of peers")
             mc = MergeChunk()
             for p, pay in enumerate(c["compressed"]):
-                _u8(pay, "compressed", agg)
+                _u8(pay, "compressed", like)
                 mc.payloads[p] = pay.data_ptr()
                 mc.payload_bytes[p] = pay.numel()
-            mc.aggregate = agg.data_ptr()
-            st, oc = c.get("state"), c.get("out_compressed")
+            mc.aggregate = agg.data_ptr() if agg is not None else None
             if st is not None:
-                _f32(st, "state", agg); _u8(oc, "out_compressed", agg)
+                _f32(st, "state", like); _u8(oc, "out_compressed", like)
                 mc.state, mc.out_payload, mc.out_payload_bytes = st.data_ptr(), oc.data_ptr(), oc.numel()
-            mc.n = agg.numel()
+            mc.n = like.numel()
             arr[i] = mc
         self.device = dev
         pr = Params(float(threshold), int(bucket), 0.0, 0.0, float(ratio))

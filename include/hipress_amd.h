@@ -159,7 +159,11 @@ int hipress_sparse_decode(const void *payload, int64_t payload_bytes, float *out
 /* payloads / payload_bytes are HOST arrays of npeers entries (device pointers
  * and sizes).  aggregate[n] receives the sum of the decoded peers.  With a
  * non-NULL residual (tbq) or accumulator (sparse) the aggregate is re-encoded
- * for the next hop into out_payload in the same pass. */
+ * for the next hop into out_payload in the same pass; such a call may pass
+ * aggregate = NULL when only the re-encoded payload is wanted (an aggregator that
+ * forwards the sum and applies no update itself): the sum is then never written
+ * as fp32, which saves 4 of the step's bytes per element.  Payload and state come
+ * out the same either way. */
 int hipress_tbq_decode_merge(const void *const *payloads, const int64_t *payload_bytes,
                              int32_t npeers, float *aggregate, int64_t n, float *residual,
                              void *out_payload, int64_t out_payload_bytes, float threshold,

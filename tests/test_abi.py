@@ -83,3 +83,9 @@ def test_null_and_range_checks_need_no_gpu(lib):
     assert L.hipress_tbq_decode(None, 100, None, 10, None) == -1
     assert L.hipress_batch_encode(None, None) == -1
     assert L.hipress_merge_batch_run(None, None) == -1
+    # a merge without the re-encode needs its aggregate
+    import ctypes
+    pay = (ctypes.c_void_p * 1)(64)
+    nb = (ctypes.c_int64 * 1)(1 << 20)
+    assert L.hipress_tbq_decode_merge(pay, nb, 1, None, 16, None, None, 0, 0.05, None) == -1
+    assert L.hipress_onebit_decode_merge(pay, nb, 1, None, 16, None) == -1

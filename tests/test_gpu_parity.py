@@ -629,6 +629,56 @@ def test_sparse_batch_decode_handmade_payloads(hp):
 
 
 @pytest.mark.parametrize("alg", ["tbq", "dgc"])
+def test_merge_that_only_re_encodes_leaves_the_same_payload_and_state(hp, alg):
+    """A re-encoding merge may be called without an aggregate buffer (only the
+    re-encoded payload is wanted): payload and state equal those of the call that also
+    writes the aggregate, per tensor and through a batch; without the re-encode a
+    missing aggregate is refused."""
+    rng = np.random.default_rng(5)
+    P, tau, ratio = 8, 0.05, 0.001
+    sizes = [300001, 4097, 1048576]
+    chunks_a, chunks_b = [], []
+    for n in sizes:
+        if alg == "tbq":
+            pays = [oracle.tbq_encode(rng.normal(0, 0.04, n).astype(F), np.zeros(n, F), tau)[0] for _ in range(P)]
+            nb = hp.tbq_payload_bytes(n)
+        else:
+            pays = [oracle.dgc_encode(rng.normal(0, 1e-3, n).astype(F), np.zeros(n, F), np.zeros(n, F), 0.9, ratio)[0] for _ in range(P)]
+            nb = hp.dgc_payload_bytes(n, ratio)
+        st = rng.normal(0, 1e-3, n).astype(F)
+        dp = [dev(p) for p in pays]
+        chunks_a.append({"compressed": dp, "aggregate": torch.empty(n, device="cuda"), "state": dev(st), "out_compressed": payload(nb)})
+        chunks_b.append({"compressed": dp, "aggregate": None, "state": dev(st), "out_compressed": payload(nb)})
+        # per tensor
+        sa, sb, oa, ob = dev(st), dev(st), payload(nb), payload(nb)
+        if alg == "tbq":
+            hp.tbq_decode_merge(dp, torch.empty(n, device="cuda"), sa, oa, tau)
+            hp.tbq_decode_merge(dp, None, sb, ob, tau)
+        else:
+            hp.dgc_decode_merge(dp, torch.empty(n, device="cuda"), sa, oa, ratio)
+            hp.dgc_decode_merge(dp, None, sb, ob, ratio)
+        if alg == "tbq":
+            np.testing.assert_array_equal(host(ob), host(oa))
+        else:
+            check_sparse(host(ob), host(oa))
+        np.testing.assert_array_equal(host(sb), host(sa))
+    ba = hp.MergeBatch(alg, chunks_a, threshold=tau, ratio=ratio)
+    bb = hp.MergeBatch(alg, chunks_b, threshold=tau, ratio=ratio)
+    ba.run()
+    bb.run()
+    for ca, cb in zip(chunks_a, chunks_b):
+        if alg == "tbq":
+            np.testing.assert_array_equal(host(cb["out_compressed"]), host(ca["out_compressed"]))
+        else:
+            check_sparse(host(cb["out_compressed"]), host(ca["out_compressed"]))
+        np.testing.assert_array_equal(host(cb["state"]), host(ca["state"]))
+    ba.close()
+    bb.close()
+    with pytest.raises(TypeError):
+        (hp.tbq_decode_merge if alg == "tbq" else hp.dgc_decode_merge)(chunks_a[0]["compressed"], None)
+
+
+@pytest.mark.parametrize("alg", ["tbq", "dgc"])
 def test_merge_batch_matches_oracle(hp, alg):
     rng = np.random.default_rng(77)
     P, tau, ratio = 8, 0.05, 0.001
