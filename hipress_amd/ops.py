@@ -103,8 +103,20 @@ def _on(device):
     return _NO_SWITCH if torch.cuda.current_device() == device.index else torch.cuda.device(device)
 
 
+# torch's own extensions read the current stream's handle through this accessor; it skips
+# the Stream object that torch.cuda.current_stream builds (about 2 microseconds a call,
+# which shows on launch-bound tensors)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _device_stream(device):
+    if _raw_stream is not None:
+        return _raw_stream(device.index)
+    return torch.cuda.current_stream(device).cuda_stream
+
+
 def _stream(t):
-    return torch.cuda.current_stream(t.device).cuda_stream
+    return _device_stream(t.device)
 
 
 _workspaces = {}
@@ -392,16 +404,16 @@ class Batch:
 
     def encode(self):
         with _on(self.device):
-            check(_lib.lib().hipress_batch_encode(self._h, torch.cuda.current_stream(self.device).cuda_stream), "batch_encode")
+            check(_lib.lib().hipress_batch_encode(self._h, _device_stream(self.device)), "batch_encode")
 
     def encode_phase(self, phase):
         """One launch of the encode sequence (measurement aid)."""
         with _on(self.device):
-            check(_lib.lib().hipress_batch_encode_phase(self._h, int(phase), torch.cuda.current_stream(self.device).cuda_stream), "batch_encode_phase")
+            check(_lib.lib().hipress_batch_encode_phase(self._h, int(phase), _device_stream(self.device)), "batch_encode_phase")
 
     def decode(self):
         with _on(self.device):
-            check(_lib.lib().hipress_batch_decode(self._h, torch.cuda.current_stream(self.device).cuda_stream), "batch_decode")
+            check(_lib.lib().hipress_batch_decode(self._h, _device_stream(self.device)), "batch_decode")
 
     def close(self):
         if getattr(self, "_h", None):
@@ -463,12 +475,12 @@ class MergeBatch:
 
     def run(self):
         with _on(self.device):
-            check(_lib.lib().hipress_merge_batch_run(self._h, torch.cuda.current_stream(self.device).cuda_stream), "merge_batch_run")
+            check(_lib.lib().hipress_merge_batch_run(self._h, _device_stream(self.device)), "merge_batch_run")
 
     def run_phase(self, phase):
         """One part of the launch sequence (measurement aid)."""
         with _on(self.device):
-            check(_lib.lib().hipress_merge_batch_run_phase(self._h, int(phase), torch.cuda.current_stream(self.device).cuda_stream),
+            check(_lib.lib().hipress_merge_batch_run_phase(self._h, int(phase), _device_stream(self.device)),
                   "merge_batch_run_phase")
 
     def close(self):
