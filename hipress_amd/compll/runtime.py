@@ -46,6 +46,7 @@ class Operators:
     def _bind(self, name, m, fn, ws_bytes):
         import torch
 
+        _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)  # the handle without building a Stream object
         vectors = [p for p in m["params"] if p["kind"].endswith("*")]
         scalars = [p for p in m["params"] if not p["kind"].endswith("*")]
 
@@ -83,7 +84,7 @@ class Operators:
                     raise ValueError(f"{name}: uniform= is shorter than the float vectors")
                 cargs.append(uniform.data_ptr())
             need = ws_bytes(biggest)
-            stream = torch.cuda.current_stream(device).cuda_stream
+            stream = _raw_stream(device.index) if _raw_stream is not None else torch.cuda.current_stream(device).cuda_stream
             key = (device, stream, name)  # scratch is per stream: calls on one stream are ordered, others are not
             ws = self._workspaces.get(key)
             if ws is None or ws.numel() < need:
