@@ -203,13 +203,23 @@ __device__ __forceinline__ float wave_sum(float x) {
     for (int m = 32; m >= 1; m >>= 1) x += __shfl_xor(x, m, 64);
     return x;
 }
+// Maximum over the 64 lanes, the same value in every lane: data-parallel-primitive steps
+// inside every row of 16 lanes, then across the rows (a maximum does not depend on the
+// order it is taken in).  All 64 lanes must be active.
 __device__ __forceinline__ float wave_max(float x) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) {
-        float y = __shfl_xor(x, m, 64);
-        x = y > x ? y : x;
+#define HP_MAX_STEP(CTRL, ROWS)                                                                                   \
+    {                                                                                                             \
+        const float y = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(x), __float_as_int(x), CTRL, ROWS, 0xf, false)); \
+        x = y > x ? y : x;                                                                                        \
     }
-    return x;
+    HP_MAX_STEP(0xB1, 0xf)   // quad_perm [1,0,3,2]
+    HP_MAX_STEP(0x4E, 0xf)   // quad_perm [2,3,0,1]
+    HP_MAX_STEP(0x141, 0xf)  // row_half_mirror
+    HP_MAX_STEP(0x140, 0xf)  // row_mirror
+    HP_MAX_STEP(0x142, 0xa)  // row_bcast:15 into rows 1, 3
+    HP_MAX_STEP(0x143, 0xc)  // row_bcast:31 into rows 2, 3
+#undef HP_MAX_STEP
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 63));
 }
 // Inclusive prefix sum over the 64 lanes in six data-parallel-primitive steps:
 // four shifts inside every row of 16 lanes, then lane 15 of rows 0 and 2 is added
