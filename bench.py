@@ -41,6 +41,8 @@ MEASURED_TRAFFIC = {
     "merge_dgc_vgg19": 1780978995,        # sparse_merge_kernel
     "compll_b2_fc6": 848749465,           # compll_quant_kernel
     "compll_generated_b2_fc6": 848736665, # map_packed_kernel of the generated operator
+    "merge_tbq_vgg19_payload_only": 1516136345,  # dense_merge_kernel
+    "merge_dgc_vgg19_payload_only": 1206018662,  # sparse_merge_kernel
 }
 
 
