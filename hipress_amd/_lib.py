@@ -57,6 +57,7 @@ SIGNATURES = {
     "hipress_tbq_encode": (ctypes.c_int, [_vp, _vp, _i64, _vp, _i64, _f32, _vp]),
     "hipress_tbq_decode": (ctypes.c_int, [_vp, _i64, _vp, _i64, _vp]),
     "hipress_onebit_encode": (ctypes.c_int, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
+    "hipress_onebit_encode_static": (ctypes.c_int, [_vp, _vp, _i64, _vp, _i64, _vp]),
     "hipress_onebit_decode": (ctypes.c_int, [_vp, _i64, _vp, _i64, _vp]),
     "hipress_onebit_encode_deferred": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "hipress_onebit_residual": (ctypes.c_int, [_vp, _vp, _i64, _vp, _vp]),

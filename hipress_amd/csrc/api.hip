@@ -2,6 +2,7 @@
 // launch objects.  Kernels live in dense.hip, sparse.hip and merge.hip.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstring>
 #include <new>
@@ -422,6 +423,44 @@ int hipress_onebit_encode(const float* grad, float* residual, int64_t n, void* p
     if (!workspace || workspace_bytes < hipress_onebit_workspace_bytes(n)) return HIPRESS_ERR_WORKSPACE;
     if (mis(workspace, 16)) return HIPRESS_ERR_ALIGN;
     return hiperr(launch_onebit_encode(single_launch(s), static_cast<float*>(workspace), -1, static_cast<hipStream_t>(stream)));
+}
+
+// hipress_onebit_encode without a workspace argument: the per-tile partial sums go to
+// a file-scope device array, so the call needs no memory beyond inputs and outputs.
+// Every GPU holds its own copy of the array at its own address; that address is asked
+// for once per device (the first call on it) and kept.  The array's name is a
+// host-side stand-in, not a device address, so only the looked-up pointer is handed to
+// kernels.  The magnitude-sum launch writes partial[0, tiles) before the scale launch
+// reads them, so whatever an earlier call left there is never seen and nothing has to
+// be cleared.
+constexpr int kStaticMaxDevices = 64;
+constexpr int64_t kStaticTiles = HIPRESS_ONEBIT_STATIC_MAX_N / kTile;
+static __device__ __align__(256) float scratch[kStaticTiles];
+static std::atomic<float*> scratch_ptr[kStaticMaxDevices];
+
+static int static_scratch(float** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kStaticMaxDevices) return HIPRESS_ERR_HIP;
+    float* p = scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        if (hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch)) != hipSuccess || !p) return HIPRESS_ERR_HIP;
+        scratch_ptr[dev].store(p, std::memory_order_release);  // threads that race here look up the same address
+    }
+    *out = p;
+    return HIPRESS_OK;
+}
+
+int hipress_onebit_encode_static(const float* grad, float* residual, int64_t n, void* payload, int64_t payload_bytes,
+                                 void* stream) {
+    if (n > HIPRESS_ONEBIT_STATIC_MAX_N) return HIPRESS_ERR_SIZE;
+    hipress_tensor t{grad, residual, nullptr, nullptr, payload, nullptr, n, payload_bytes};
+    hipress_params pr{};
+    Seg s;
+    int rc = build_encode_seg(HIPRESS_ONEBIT, t, pr, &s);
+    if (rc) return rc;
+    float* partial = nullptr;
+    if ((rc = static_scratch(&partial))) return rc;
+    return hiperr(launch_onebit_encode(single_launch(s), partial, -1, static_cast<hipStream_t>(stream)));
 }
 
 int hipress_onebit_decode(const void* payload, int64_t payload_bytes, float* out, int64_t n, void* stream) {

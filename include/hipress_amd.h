@@ -100,6 +100,20 @@ int hipress_onebit_encode(const float *grad, float *residual, int64_t n, void *p
 int hipress_onebit_decode(const void *payload, int64_t payload_bytes, float *out, int64_t n,
                           void *stream);
 
+/* hipress_onebit_encode for callers that cannot allocate device memory (code under
+ * HIP-graph capture, tight serving loops, harnesses that forbid hipMalloc): same
+ * arguments without the workspace, same payload and residual bit for bit.  The
+ * per-tile partial sums live in a device array inside the library (256 KiB per GPU,
+ * held until the process ends), which limits n to HIPRESS_ONEBIT_STATIC_MAX_N
+ * (larger n: HIPRESS_ERR_SIZE).  The call allocates and frees nothing; the first call
+ * on a device looks up that device's copy of the array (hipGetSymbolAddress), so make
+ * it once before a capture begins.  All calls on one GPU share the array: calls that
+ * overlap there (different streams without ordering) race; calls on one stream, or
+ * ordered by events, are safe.  No counterpart in the reference. */
+#define HIPRESS_ONEBIT_STATIC_MAX_N 268435456LL /* 2^28 elements = 65,536 tiles of 4096 */
+int hipress_onebit_encode_static(const float *grad, float *residual, int64_t n, void *payload,
+                                 int64_t payload_bytes, void *stream);
+
 /* onebit with a deferred residual: one pass per step instead of two.  `state`
  * holds v = r + g of the LAST step (initially the residual itself) and
  * `scale_state` (one float, initially 0) that step's scale; each call first forms

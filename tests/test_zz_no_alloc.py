@@ -1,0 +1,89 @@
+"""hipress_onebit_encode_static: the onebit encoder for callers that cannot allocate.
+
+Called through the C ABI and compared bit for bit with hipress_onebit_encode (which takes
+its workspace from the caller) on the same inputs, twice in a row on one GPU, the second
+time with a smaller tensor, so that what the first call left in the library's static
+scratch array lies behind the part the second call uses."""
+import ctypes
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+STATIC_MAX_N = 1 << 28
+
+
+def _run_pair(L, torch, n, seed, steps=2):
+    """Runs `steps` consecutive steps of both entry points on identical inputs; returns
+    the two (payload, residual) histories."""
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    nbytes = int(L.hipress_onebit_payload_bytes(n))
+    ws = torch.empty(int(L.hipress_onebit_workspace_bytes(n)), dtype=torch.uint8, device="cuda")
+    r_ref, r_new = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    p_ref = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    p_new = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    out = []
+    for _ in range(steps):
+        g = torch.randn(n, generator=gen, device="cuda") * 0.01
+        rc = L.hipress_onebit_encode(g.data_ptr(), r_ref.data_ptr(), n, p_ref.data_ptr(), nbytes, ws.data_ptr(),
+                                     ws.numel(), stream)
+        assert rc == 0
+        rc = L.hipress_onebit_encode_static(g.data_ptr(), r_new.data_ptr(), n, p_new.data_ptr(), nbytes, stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        out.append((p_ref.cpu().numpy().copy(), r_ref.cpu().numpy().copy(), p_new.cpu().numpy().copy(),
+                    r_new.cpu().numpy().copy()))
+    return out
+
+
+def test_static_scratch_encode_equals_the_workspace_encode_on_two_calls_in_a_row():
+    import torch
+
+    from hipress_amd import _lib
+
+    L = _lib.lib()
+    # first a tensor of 2,359,296 + 37 elements (577 tiles, the last one partial), then a
+    # smaller one (24 tiles + a partial one): the second call reuses the front of the array
+    for n, seed in ((2359296 + 37, 1), (100003, 2)):
+        for step, (p_ref, r_ref, p_new, r_new) in enumerate(_run_pair(L, torch, n, seed)):
+            assert np.array_equal(p_ref, p_new), f"payload differs, n={n}, step {step}"
+            assert np.array_equal(r_ref.view(np.uint32), r_new.view(np.uint32)), f"residual differs, n={n}, step {step}"
+            assert float(p_new[:4].view(np.float32)[0]) > 0.0
+            assert int(p_new[4:8].view(np.uint32)[0]) == n
+
+
+def test_static_scratch_encode_matches_the_oracle():
+    import torch
+
+    import oracle
+    from hipress_amd import _lib
+
+    L = _lib.lib()
+    n = 70001
+    g = np.random.default_rng(5).normal(0, 0.02, n).astype(np.float32)
+    gd = torch.from_numpy(g).cuda()
+    r = torch.zeros(n, device="cuda")
+    pay = torch.zeros(int(L.hipress_onebit_payload_bytes(n)), dtype=torch.uint8, device="cuda")
+    assert L.hipress_onebit_encode_static(gd.data_ptr(), r.data_ptr(), n, pay.data_ptr(), pay.numel(), None) == 0
+    torch.cuda.synchronize()
+    got = pay.cpu().numpy()
+    s = got[:4].view(np.float32)[0]
+    s_ref = oracle.onebit_scale(g, np.zeros(n, np.float32))
+    assert abs(float(s) - float(s_ref)) <= 1e-5 * float(s_ref)
+    want_pay, want_r = oracle.onebit_encode(g, np.zeros(n, np.float32), scale=s)
+    assert np.array_equal(got, want_pay)
+    assert np.array_equal(r.cpu().numpy(), want_r)
+
+
+def test_static_scratch_encode_rejects_what_its_array_cannot_hold():
+    from hipress_amd import _lib
+
+    L = _lib.lib()
+    # validated on the host before any launch: the pointers are never touched
+    fake = ctypes.c_void_p(1 << 20)
+    big = STATIC_MAX_N + 1
+    assert L.hipress_onebit_encode_static(fake, fake, big, fake, 16 + 4 * ((big + 31) // 32), None) == -2
+    assert _lib.strerror(-2).startswith("element count")
+    assert L.hipress_onebit_encode_static(None, None, 16, None, 100, None) == -1
