@@ -2,48 +2,60 @@
 """Throughput of the gradient-compression hot path on one MI355X.
 
 A step is one pass of encode followed by decode over a whole synthetic gradient
-set that is already resident in HBM.  The headline line is onebit over the
-VGG19 gradient set; `--workload` selects another, and `others` in the JSON line
-carries a shorter measurement of every other compressor / configuration.
+set that is already resident in HBM, through the calls a user of the library
+makes (`Batch.encode()`, `Batch.decode()`, `MergeBatch.run()`).  The headline
+line is TBQ over the VGG19 gradient set; `--workload` selects another, and
+`others` in the JSON line carries a shorter measurement of every other
+compressor / configuration (DGC over the same set first).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others] [--no-cpu]
 
-Prints ONE JSON line.  value = 4 * elements * steps / elapsed, in GB/s of fp32
-gradient through encode+decode.  `roofline` describes the dominant kernel:
+Prints ONE JSON line.  value = 4 * elements * steps / elapsed over exactly K
+steps bracketed by device synchronisation, in GB/s of fp32 gradient through
+encode+decode; `median_ms_per_step` is the median of the same steps timed one by
+one with events in a second run.  `roofline` describes the dominant kernel:
 algorithmic bytes per launch over its mean duration, measured with events on the
-launch stream inside the timed steps, against the 8 TB/s HBM peak.
+launch stream in a third run that issues the encode sequence launch by launch,
+against the 8 TB/s HBM peak.  Every entry carries `cpu_baseline`: the scalar CPU
+oracle (one thread, the execution model of the reference's registered CPU
+operator) on a bounded sample of the same tensors, and the same source built with
+OpenMP on all host cores beside it.
 """
 import argparse
 import ctypes
 import json
 import os
+import re
+import statistics
+import subprocess
 import sys
 import time
 
 HBM_PEAK_GBS = 8000.0
+ROOT = os.path.dirname(os.path.abspath(__file__))
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs (summaries under profiles/), keyed by workload; absent = not
-# measured.  (FETCH_SIZE KiB * 2.0 + WRITE_SIZE KiB * 1.0) * 1024, the factors
-# being what the same counters read for a plain 1 GiB copy.
-MEASURED_TRAFFIC = {
-    "onebit_vgg19": 1747750092,           # onebit_quant_kernel
-    "onebit_deferred_vgg19": 1748885811,  # onebit_deferred_kernel
-    "tbq_vgg19": 1765707366,              # tbq_encode_kernel
-    "terngrad_vgg19": 1193284403,         # terngrad_encode_kernel
-    "dgc_vgg19": 2904932454,              # sparse_accum_kernel
-    "graddrop_vgg19": 1755469209,         # sparse_accum_kernel
-    "tbq_262144_x512": 1650560614,        # tbq_encode_kernel
-    "terngrad_resnet50": 212500377,       # terngrad_encode_kernel
-    "dgc_bert_large": 6782823833,         # sparse_accum_kernel
-    "graddrop_bert_large": 4101445222,    # sparse_accum_kernel
-    "merge_tbq_vgg19": 2090826240,        # dense_merge_kernel
-    "merge_dgc_vgg19": 1780978995,        # sparse_merge_kernel
-    "compll_b2_fc6": 848749465,           # compll_quant_kernel
-    "compll_generated_b2_fc6": 848736665, # map_packed_kernel of the generated operator
-    "merge_tbq_vgg19_payload_only": 1516136345,  # dense_merge_kernel
-    "merge_dgc_vgg19_payload_only": 1206018662,  # sparse_merge_kernel
-}
+
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` as the rocprofv3 summary of this workload holds them
+    (profiles/<workload>.md, table "HBM traffic per dispatch": (2.0 x FETCH_SIZE + 1.0 x
+    WRITE_SIZE) x 1024, the factors being what the same counters read for a plain 1 GiB
+    copy), or None when no summary with counters exists.  -> (bytes, source path)"""
+    path = os.path.join(ROOT, "profiles", workload + ".md")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, None
+    sect = text.split("HBM traffic per dispatch", 1)
+    if len(sect) < 2:
+        return None, None
+    for line in sect[1].splitlines():
+        cells = [c.strip() for c in line.split("|")]
+        if len(cells) >= 6 and kernel in cells[1]:
+            try:
+                return int(cells[5].replace(",", "")), os.path.relpath(path, ROOT)
+            except ValueError:
+                return None, None
+    return None, None
 
 
 def _events(n):
@@ -52,12 +64,41 @@ def _events(n):
     return [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
 
 
+CPU_TENSOR_CAP = 4 << 20    # elements taken from the front of any one tensor for the CPU sample
+CPU_SAMPLE_CAP = 24 << 20   # elements per CPU pass
+
+
+def _vp(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+class CpuJob:
+    """One pass of a workload's CPU restatement over a bounded sample; run(L) executes it
+    with oracle build L (scalar or OpenMP) and carries state from pass to pass."""
+
+    def __init__(self, elements, sample, run):
+        self.elements, self.sample, self.run = elements, sample, run
+
+
+def _sample_front(sizes):
+    """The front of each tensor (at most CPU_TENSOR_CAP elements), tensors taken in order
+    until CPU_SAMPLE_CAP elements are reached: [(tensor index, elements)]."""
+    picks, total = [], 0
+    for i, n in enumerate(sizes):
+        if total >= CPU_SAMPLE_CAP:
+            break
+        k = min(n, CPU_TENSOR_CAP, CPU_SAMPLE_CAP - total)
+        if k > 0:
+            picks.append((i, k))
+            total += k
+    return picks, total
+
+
 class SetWorkload:
     """encode+decode of one compressor over a list of tensor sizes through a Batch."""
 
     def __init__(self, name, alg, sizes, data, params, enc_bytes, dec_bytes, dominant_phase, dominant_kernel,
-                 dominant_bytes, rotate=1, nphases=1, graph=False):
-        self.graph = graph  # replay encode+decode from a captured HIP graph (one launch per step)
+                 dominant_bytes, rotate=1, nphases=1):
         self.name, self.alg, self.sizes, self.data, self.params = name, alg, sizes, data, params
         self.enc_bytes, self.dec_bytes = enc_bytes, dec_bytes  # algorithmic bytes per element
         self.dominant_phase, self.dominant_kernel, self.dominant_bytes = dominant_phase, dominant_kernel, dominant_bytes
@@ -113,24 +154,8 @@ class SetWorkload:
             self.tensors.append(ts)
             self.batches.append(hp.Batch(self.alg, ts, **self.params))
         self.k = 0
-        self.captured = None
-        if self.graph:
-            side = torch.cuda.Stream()
-            b = self.batches[0]
-            with torch.cuda.stream(side):
-                b.encode()
-                b.decode()
-                side.synchronize()
-                self.captured = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(self.captured, stream=side):
-                    b.encode()
-                    b.decode()
-            torch.cuda.synchronize()
 
     def step(self, ev=None):
-        if self.captured is not None:
-            self.captured.replay()
-            return
         b = self.batches[self.k % self.rotate]
         self.k += 1
         if ev is None:
@@ -145,6 +170,51 @@ class SetWorkload:
                     b.encode_phase(ph)
         b.decode()
 
+    def cpu_job(self):
+        """The same compressor in the CPU oracle over the front of this set's tensors (the
+        values the GPU run used, copied from the device)."""
+        import numpy as np
+
+        import oracle
+
+        picks, total = _sample_front(self.sizes)
+        ts = self.tensors[0]
+        g = [ts[i]["gradient"][:k].cpu().numpy() for i, k in picks]
+        u = [ts[i]["uniform"][:k].cpu().numpy() for i, k in picks] if self.alg == "terngrad" else None
+        zeros = lambda: [np.zeros(k, np.float32) for _, k in picks]
+        s0, s1 = zeros(), zeros()
+        out = [np.empty(k, np.float32) for _, k in picks]
+        alg, pr = self.alg, self.params
+        ratio = pr.get("ratio", 0.001)
+        nbytes = {"tbq": oracle.tbq_payload_bytes, "onebit": oracle.onebit_payload_bytes,
+                  "onebit_deferred": oracle.onebit_payload_bytes,
+                  "terngrad": lambda n: oracle.terngrad_payload_bytes(n, pr.get("bucket", 512)),
+                  "dgc": lambda n: oracle.sparse_payload_bytes(n, ratio),
+                  "graddrop": lambda n: oracle.sparse_payload_bytes(n, ratio)}[alg]
+        pay = [np.zeros(nbytes(k), np.uint8) for _, k in picks]
+
+        def run(L):
+            for j, (_, k) in enumerate(picks):
+                if alg == "tbq":
+                    L.hpo_tbq_encode(_vp(g[j]), _vp(s0[j]), k, _vp(pay[j]), pr["threshold"])
+                    L.hpo_tbq_decode(_vp(pay[j]), _vp(out[j]), k)
+                elif alg in ("onebit", "onebit_deferred"):
+                    L.hpo_onebit_encode(_vp(g[j]), _vp(s0[j]), k, _vp(pay[j]))
+                    L.hpo_onebit_decode(_vp(pay[j]), _vp(out[j]), k)
+                elif alg == "terngrad":
+                    L.hpo_terngrad_encode(_vp(g[j]), _vp(u[j]), k, _vp(pay[j]), pr.get("bucket", 512))
+                    L.hpo_terngrad_decode(_vp(pay[j]), _vp(out[j]), k)
+                elif alg == "dgc":
+                    L.hpo_dgc_encode(_vp(g[j]), _vp(s0[j]), _vp(s1[j]), k, _vp(pay[j]), pr["momentum_factor"], ratio)
+                    L.hpo_sparse_decode(_vp(pay[j]), _vp(out[j]), k)
+                else:
+                    L.hpo_graddrop_encode(_vp(g[j]), _vp(s1[j]), k, _vp(pay[j]), ratio)
+                    L.hpo_sparse_decode(_vp(pay[j]), _vp(out[j]), k)
+
+        what = (f"{alg} encode+decode over the first <= {CPU_TENSOR_CAP:,} elements of "
+                f"{len(picks)} of the set's {len(self.sizes)} tensors ({total:,} elements per pass)")
+        return CpuJob(total, what, run)
+
     def density(self):
         """Measured fraction of elements kept (sparse compressors)."""
         import torch
@@ -155,7 +225,6 @@ class SetWorkload:
         return nnz / self.elements
 
     def close(self):
-        self.captured = None
         for b in self.batches:
             b.close()
         self.batches, self.tensors = [], []
@@ -172,6 +241,13 @@ class MergeWorkload:
         self.dominant_phase = 0
         self.nphases = 1
         self.rotate = 1
+        agg_bytes = 4.0 if aggregate else 0.0
+        if alg == "tbq":
+            self.enc_bytes, self.dec_bytes = 0.25 * npeers + agg_bytes + 8.25, 0.0
+            self.dominant_kernel, self.dominant_bytes = "dense_merge_kernel", self.enc_bytes
+        else:
+            self.enc_bytes, self.dec_bytes = 8.0 + agg_bytes, 0.0  # + 8*(P*rho + rho'), added after the run
+            self.dominant_kernel, self.dominant_bytes = "sparse_merge_kernel", 8.0 + agg_bytes
 
     def setup(self, dev):
         import torch
@@ -206,13 +282,6 @@ class MergeWorkload:
             del grads, ts
         self.chunks = chunks
         self.mb = hp.MergeBatch(self.alg, chunks, threshold=tau, ratio=ratio)
-        agg_bytes = 4.0 if self.aggregate else 0.0
-        if self.alg == "tbq":
-            self.enc_bytes, self.dec_bytes = 0.25 * self.npeers + agg_bytes + 8.25, 0.0
-            self.dominant_kernel, self.dominant_bytes = "dense_merge_kernel", self.enc_bytes
-        else:
-            self.enc_bytes, self.dec_bytes = 8.0 + agg_bytes, 0.0  # + 8*(P*rho + rho'), added after the run
-            self.dominant_kernel, self.dominant_bytes = "sparse_merge_kernel", 8.0 + agg_bytes
 
     def step(self, ev=None):
         if ev is not None and self.alg == "tbq":
@@ -227,6 +296,35 @@ class MergeWorkload:
             self.mb.run_phase(2)
         else:
             self.mb.run()
+
+    def cpu_job(self):
+        """decode-and-merge + re-encode of the first chunks in the CPU oracle, on the very
+        peer payloads the GPU run merges."""
+        import numpy as np
+
+        picks, total = _sample_front(self.sizes)
+        picks = picks[:4]
+        total = sum(k for _, k in picks)
+        P, alg, ratio = self.npeers, self.alg, self.ratio
+        jobs = []
+        for i, k in picks:
+            n = self.sizes[i]
+            pays = [p.cpu().numpy() for p in self.chunks[i]["compressed"]]
+            arr = (ctypes.c_void_p * P)(*[p.ctypes.data for p in pays])
+            jobs.append((n, pays, arr, np.empty(n, np.float32), np.zeros(n, np.float32),
+                         np.zeros(self.chunks[i]["out_compressed"].numel(), np.uint8)))
+        total = sum(j[0] for j in jobs)
+
+        def run(L):
+            for n, _, arr, agg, state, outp in jobs:
+                if alg == "tbq":
+                    L.hpo_tbq_decode_merge(arr, P, _vp(agg), n, _vp(state), _vp(outp), 0.05)
+                else:
+                    L.hpo_sparse_decode_merge(arr, P, _vp(agg), n, _vp(state), _vp(outp), ratio)
+
+        what = (f"{alg} decode-and-merge of {P} peers + re-encode over the first {len(jobs)} of "
+                f"{len(self.sizes)} chunks ({total:,} elements per pass)")
+        return CpuJob(total, what, run)
 
     def density(self):
         import torch
@@ -247,7 +345,8 @@ class CompllWorkload:
     def __init__(self, name, n, bitwidth=2, generated=False):
         self.name, self.sizes, self.elements, self.b, self.generated = name, [n], n, bitwidth, generated
         self.enc_bytes, self.dec_bytes = 8.0 + bitwidth / 8.0, 4.0 + bitwidth / 8.0
-        self.dominant_kernel, self.dominant_bytes = "compll_quant_kernel", 8.0 + bitwidth / 8.0
+        self.dominant_kernel = "map_packed_kernel" if generated else "compll_quant_kernel"
+        self.dominant_bytes = 8.0 + bitwidth / 8.0
 
     def setup(self, dev):
         import torch
@@ -272,6 +371,21 @@ class CompllWorkload:
         else:
             self.hp.compll_terngrad_encode(self.g, self.u, self.pay, self.b)
             self.hp.compll_terngrad_decode(self.pay, self.out)
+
+    def cpu_job(self):
+        import numpy as np
+
+        k = min(self.elements, 4 * CPU_TENSOR_CAP)
+        g, u = self.g[:k].cpu().numpy(), self.u[:k].cpu().numpy()
+        pay = np.zeros(10 + (k * self.b + 7) // 8, np.uint8)
+        out = np.empty(k, np.float32)
+        b = self.b
+
+        def run(L):
+            L.hpo_compll_encode(_vp(g), _vp(u), k, _vp(pay), b)
+            L.hpo_compll_decode(_vp(pay), pay.size, _vp(out), k)
+
+        return CpuJob(k, f"min/max {b}-bit quantiser encode+decode over the first {k:,} elements of the tensor", run)
 
     def close(self):
         self.g = self.u = self.pay = self.out = None
@@ -309,6 +423,21 @@ class GeneratedTbqWorkload:
             self.hp.tbq_encode(self.g, self.r, self.pay, 0.05)
             self.hp.tbq_decode(self.pay, self.out)
 
+    def cpu_job(self):
+        import numpy as np
+
+        import oracle
+
+        k = min(self.elements, 4 * CPU_TENSOR_CAP)
+        g, r = self.g[:k].cpu().numpy(), np.zeros(k, np.float32)
+        pay, out = np.zeros(oracle.tbq_payload_bytes(k), np.uint8), np.empty(k, np.float32)
+
+        def run(L):
+            L.hpo_tbq_encode(_vp(g), _vp(r), k, _vp(pay), 0.05)
+            L.hpo_tbq_decode(_vp(pay), _vp(out), k)
+
+        return CpuJob(k, f"tbq encode+decode over the first {k:,} elements of the tensor", run)
+
     def close(self):
         self.g = self.r = self.pay = self.out = None
 
@@ -332,9 +461,6 @@ def make_workload(name):
         return SetWorkload(name, "graddrop", vgg, "vgg", {"ratio": 0.01}, 12.0, 4.0, 0, "sparse_accum_kernel", 12.0, nphases=7)
     if name == "tbq_262144":
         return SetWorkload(name, "tbq", [262144], "n0.02", {"threshold": 0.05}, 12.25, 4.25, 0, "tbq_encode_kernel", 12.25)
-    if name == "tbq_262144_graph":
-        return SetWorkload(name, "tbq", [262144], "n0.02", {"threshold": 0.05}, 12.25, 4.25, 0, "tbq_encode_kernel", 12.25,
-                           graph=True)
     if name == "tbq_262144_x512":
         return SetWorkload(name, "tbq", [262144] * 512, "n0.02", {"threshold": 0.05}, 12.25, 4.25, 0, "tbq_encode_kernel", 12.25)
     if name == "terngrad_resnet50":
@@ -364,28 +490,106 @@ def make_workload(name):
     raise SystemExit(f"unknown workload {name}")
 
 
+# the metric's configurations first (VGG19: TBQ, then DGC), then every other compressor / configuration
 ALL_WORKLOADS = [
-    "onebit_vgg19", "onebit_deferred_vgg19", "tbq_vgg19", "terngrad_vgg19", "dgc_vgg19", "graddrop_vgg19", "tbq_262144", "tbq_262144_x512",
-    "terngrad_resnet50", "dgc_bert_large", "graddrop_bert_large", "merge_tbq_vgg19", "merge_dgc_vgg19", "compll_b2_fc6",
-    "compll_generated_b2_fc6", "tbq_fc6", "tbq_generated_fc6", "merge_tbq_vgg19_payload_only", "merge_dgc_vgg19_payload_only",
+    "tbq_vgg19", "dgc_vgg19", "onebit_vgg19", "terngrad_vgg19", "graddrop_vgg19", "onebit_deferred_vgg19",
+    "tbq_262144", "tbq_262144_x512", "terngrad_resnet50", "dgc_bert_large", "graddrop_bert_large",
+    "merge_tbq_vgg19", "merge_dgc_vgg19", "compll_b2_fc6", "compll_generated_b2_fc6", "tbq_fc6", "tbq_generated_fc6",
+    "merge_tbq_vgg19_payload_only", "merge_dgc_vgg19_payload_only",
 ]
+# any workload with the suffix _graph: the same step captured once into a HIP graph and replayed
+EXTRA_WORKLOADS = [w + "_graph" for w in ALL_WORKLOADS]
 
 
-def measure(name, steps, warmup):
+def cpu_baseline(job, budget_s):
+    """Times `job` (a CpuJob) with the scalar oracle for about budget_s seconds (at least one
+    pass), then with the OpenMP build of the same source for about half of that."""
+    import oracle
+
+    def run(L, budget, max_passes=1000):
+        passes, t0 = 0, time.perf_counter()
+        while True:
+            job.run(L)
+            passes += 1
+            el = time.perf_counter() - t0
+            if el >= budget or passes >= max_passes:
+                return passes, el
+
+    passes, el = run(oracle.lib(), budget_s)
+    out = {"value": 4.0 * job.elements * passes / el / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+           "sample": f"{job.sample}, {passes} passes, {el:.1f} s, scalar C oracle (gcc -O3, one thread)"}
+    try:
+        Lo = oracle.omp_lib()
+        threads = int(Lo.hpo_threads())
+        run(Lo, 0.0, 1)  # thread start-up
+        p2, e2 = run(Lo, budget_s / 2)
+        out["all_cores"] = {"value": 4.0 * job.elements * p2 / e2 / 1e9, "unit": "GB/s", "cores": threads,
+                            "sample": f"same sample, same source built with -fopenmp, {p2} passes, {e2:.1f} s"}
+    except Exception as exc:  # the OpenMP build is optional
+        out["all_cores"] = {"error": str(exc)}
+    return out
+
+
+def c_level_latency():
+    """encode+decode of one 262,144-element tensor timed by a small C program straight on the
+    C ABI (no Python, no torch between the launches): separates the library's latency from
+    the binding's.  Returns the program's JSON or an error note."""
+    exe = os.path.join(ROOT, "hipress_amd", "hipress_latency")
+    if not os.path.exists(exe):
+        return {"error": "hipress_amd/hipress_latency is not built (python -m hipress_amd.build)"}
+    try:
+        r = subprocess.run([exe, "262144", "2000"], capture_output=True, text=True, timeout=120)
+        return json.loads(r.stdout.strip().splitlines()[-1])
+    except Exception as exc:
+        return {"error": str(exc)}
+
+
+def measure(name, steps, warmup, cpu_budget_s=0.0):
     import torch
 
     dev = torch.device("cuda:0")
-    w = make_workload(name)
+    graph = name.endswith("_graph")
+    w = make_workload(name[: -len("_graph")] if graph else name)
     w.setup(dev)
     for _ in range(warmup):
         w.step()
-    evs = _events(steps)
+    captured = None
+    if graph:  # one step captured on a side stream; every later step is one graph launch
+        side = torch.cuda.Stream()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            captured = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(captured, stream=side):
+                w.step()
+        torch.cuda.synchronize()
+        eager_step = w.step
+        w.step = lambda ev=None: captured.replay()
+        for _ in range(warmup):
+            w.step()
+    # 1. exactly `steps` steps of the product calls between two synchronisations
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(steps):
-        w.step(evs[i])
+    for _ in range(steps):
+        w.step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    # 2. the same steps one by one between events: the median step
+    evs = _events(steps)
+    for a, b in evs:
+        a.record()
+        w.step()
+        b.record()
+    torch.cuda.synchronize()
+    median_ms = statistics.median(a.elapsed_time(b) for a, b in evs)
+    # 3. the encode sequence launch by launch, the dominant kernel between events
+    kev = _events(steps)
+    for i in range(steps):
+        w.step(kev[i])
+    torch.cuda.synchronize()
+    try:
+        dom_ms = sum(a.elapsed_time(b) for a, b in kev) / steps
+    except Exception:
+        dom_ms = None  # the events were never recorded (no bracketed kernel for this workload)
     enc_b, dec_b = w.enc_bytes, w.dec_bytes
     dom_b = w.dominant_bytes
     extra = {}
@@ -398,16 +602,14 @@ def measure(name, steps, warmup):
         rin, rout = w.density()
         enc_b += 8 * (rin + rout)
         extra["density_in"], extra["density_out"] = rin, rout
-    try:
-        dom_ms = sum(a.elapsed_time(b) for a, b in evs) / steps
-    except Exception:
-        dom_ms = None  # the events were never recorded (no bracketed kernel for this workload)
     gbs = 4.0 * w.elements * steps / elapsed / 1e9
     alg_gbs = (enc_b + dec_b) * w.elements * steps / elapsed / 1e9
     res = {
         "workload": name,
         "value": gbs,
         "ms_per_step": elapsed / steps * 1e3,
+        "median_ms_per_step": median_ms,
+        "value_at_median": 4.0 * w.elements / (median_ms * 1e-3) / 1e9,
         "elements": w.elements,
         "tensors": len(w.sizes),
         "algorithmic_bytes_per_element": enc_b + dec_b,
@@ -416,60 +618,24 @@ def measure(name, steps, warmup):
     }
     if dom_ms:
         ach = dom_b * w.elements / (dom_ms * 1e-3) / 1e9
+        traffic, source = measured_traffic(name, w.dominant_kernel)
         res["roofline"] = {"bound": "hbm", "kernel": w.dominant_kernel, "achieved": ach, "peak": HBM_PEAK_GBS,
-                           "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(name),
+                           "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": source,
                            "kernel_ms": dom_ms, "algorithmic_bytes_per_launch": dom_b * w.elements}
+    if name == "tbq_262144":
+        res["c_level"] = c_level_latency()
+    if cpu_budget_s > 0 and hasattr(w, "cpu_job") and not graph:
+        job = w.cpu_job()
+        torch.cuda.synchronize()
+        res["cpu_baseline"] = cpu_baseline(job, cpu_budget_s)
+        del job
+    if graph:
+        w.step = eager_step
+        captured = None
     w.close()
     del w
     torch.cuda.empty_cache()
     return res
-
-
-def cpu_baseline(budget_s=12.0):
-    """The scalar CPU oracle (one thread, the execution model of the reference's
-    registered CPU operator) on the headline workload: onebit encode+decode over the
-    whole VGG19 set, same seeded values, repeated until the budget is used.  The same
-    source built with OpenMP is timed beside it on all host cores (`all_cores`)."""
-    import numpy as np
-    import torch
-
-    import oracle
-    from hipress_amd import workloads as W
-
-    sizes = W.vgg19_sizes()
-    grads = W.normal_set(sizes, torch.device("cuda:0"), 0, log_sigma_range=(-4.0, -2.0))
-    host = [g.cpu().numpy() for g in grads]
-    del grads
-    outs = [np.empty(n, np.float32) for n in sizes]
-    pays = [np.zeros(oracle.onebit_payload_bytes(n), np.uint8) for n in sizes]
-    vp = lambda a: a.ctypes.data_as(ctypes.c_void_p)
-
-    def run(L, budget, max_passes):
-        res = [np.zeros(n, np.float32) for n in sizes]
-        passes, t0 = 0, time.perf_counter()
-        while True:
-            for g, r, p, o in zip(host, res, pays, outs):
-                L.hpo_onebit_encode(vp(g), vp(r), g.size, vp(p))
-                L.hpo_onebit_decode(vp(p), vp(o), g.size)
-            passes += 1
-            el = time.perf_counter() - t0
-            if el >= budget or passes >= max_passes:
-                return passes, el
-
-    passes, el = run(oracle.lib(), budget_s, 20)
-    out = {"value": 4.0 * sum(sizes) * passes / el / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-           "sample": f"onebit encode+decode over the whole VGG19 set ({sum(sizes):,} elements), {passes} passes, "
-                     f"{el:.1f} s, scalar C oracle built with gcc -O2"}
-    try:
-        Lo = oracle.omp_lib()
-        threads = int(Lo.hpo_threads())
-        run(Lo, 0.0, 1)  # first touch / thread start-up
-        p2, e2 = run(Lo, budget_s / 3, 40)
-        out["all_cores"] = {"value": 4.0 * sum(sizes) * p2 / e2 / 1e9, "unit": "GB/s", "cores": threads,
-                            "sample": f"same workload, same source built with -fopenmp, {p2} passes, {e2:.1f} s"}
-    except Exception as exc:  # the OpenMP build is optional
-        out["all_cores"] = {"error": str(exc)}
-    return out
 
 
 def main():
@@ -477,10 +643,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="onebit_vgg19", choices=ALL_WORKLOADS + ["tbq_262144_graph"])
+    ap.add_argument("--workload", default="tbq_vgg19", choices=ALL_WORKLOADS + EXTRA_WORKLOADS)
     ap.add_argument("--no-others", action="store_true", help="measure only --workload")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--others-steps", type=int, default=10)
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="one-thread CPU budget of the headline workload")
+    ap.add_argument("--others-cpu-seconds", type=float, default=2.0, help="one-thread CPU budget of every other workload")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 1 GiB device-to-device copy (a kernel of known traffic: 1 GiB read, "
                          "1 GiB written) so that rocprofv3 FETCH_SIZE / WRITE_SIZE can be scaled against it")
@@ -506,12 +674,12 @@ def main():
                           "launches": args.steps}))
         return
 
-    main_res = measure(args.workload, args.steps, args.warmup)
+    main_res = measure(args.workload, args.steps, args.warmup, 0.0 if args.no_cpu else args.cpu_seconds)
     others = []
     if not args.no_others:
         for name in ALL_WORKLOADS:
             if name != args.workload:
-                others.append(measure(name, args.others_steps, 3))
+                others.append(measure(name, args.others_steps, 3, 0.0 if args.no_cpu else args.others_cpu_seconds))
     line = {
         "metric": "fp32 grad GB/s through encode+decode",
         "value": main_res["value"],
@@ -520,6 +688,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": main_res["ms_per_step"],
+        "median_ms_per_step": main_res["median_ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -530,13 +699,16 @@ def main():
         "pct_of_hbm_roofline": main_res["pct_of_hbm_roofline"],
         "roofline": {k: v for k, v in main_res.get("roofline", {}).items()},
     }
-    if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline()
+    if "cpu_baseline" in main_res:
+        line["cpu_baseline"] = main_res["cpu_baseline"]
+    for k in ("density", "c_level"):
+        if k in main_res:
+            line[k] = main_res[k]
     if others:
         line["others"] = others
     print(json.dumps(line))
 
 
 if __name__ == "__main__":
-    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    sys.path.insert(0, ROOT)
     main()

@@ -65,6 +65,7 @@ SIGNATURES = {
     "hipress_terngrad_decode": (ctypes.c_int, [_vp, _i64, _vp, _i64, _vp]),
     "hipress_compll_payload_bytes": (_i64, [_i64, _i32]),
     "hipress_compll_workspace_bytes": (_i64, [_i64]),
+    "hipress_compll_decoded_count": (_i64, [_i64, _i32]),
     "hipress_compll_encode": (ctypes.c_int, [_vp, _vp, _i64, _vp, _i64, _i32, _vp, _i64, _vp]),
     "hipress_compll_decode": (ctypes.c_int, [_vp, _i64, _vp, _i64, _vp]),
     "hipress_dgc_encode": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp, _i64, _f32, _f64, _vp, _i64, _vp]),

@@ -9,6 +9,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libhipress_amd.so")
+LATENCY_EXE = os.path.join(HERE, "hipress_latency")  # C-level latency probe (csrc/latency_main.cpp)
 SOURCES = ["api.hip", "dense.hip", "sparse.hip", "merge.hip", "compll.hip"]
 FLAGS = [
     "--offload-arch=gfx950",
@@ -46,6 +47,9 @@ def build(verbose=False):
         raise RuntimeError("hipcc failed")
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     subprocess.check_call(cmd)
+    # a plain C++ program over the C ABI; no device code of its own
+    subprocess.check_call([hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", os.path.join(CSRC, "latency_main.cpp"), "-o", LATENCY_EXE,
+                           "-L" + HERE, "-lhipress_amd", "-Wl,-rpath,$ORIGIN"])
     return LIB
 
 

@@ -23,6 +23,9 @@ inline bool al16(const void* p) { return !mis(p, 16); }
 inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 inline unsigned tiles_of(int64_t n) { return n <= 0 ? 1u : (unsigned)((n + kTile - 1) / kTile); }
 inline bool bad_n(int64_t n) { return n < 0 || n > HIPRESS_MAX_N; }
+// sparse payloads carry int32 indices
+inline bool bad_sparse_n(int64_t n) { return n < 0 || n > HIPRESS_SPARSE_MAX_N; }
+inline bool is_sparse(int alg) { return alg == HIPRESS_DGC || alg == HIPRESS_GRADDROP; }
 
 inline int64_t words_bytes(int64_t n, int bits) {
     int per = 32 / bits;
@@ -132,7 +135,7 @@ int check_params(int alg, const hipress_params& pr) {
 // Fills the fields of `s` that do not depend on the tensor's place in a launch.
 int build_encode_seg(int alg, const hipress_tensor& t, const hipress_params& pr, Seg* s) {
     std::memset(s, 0, sizeof(Seg));
-    if (bad_n(t.n)) return HIPRESS_ERR_SIZE;
+    if (bad_n(t.n) || (is_sparse(alg) && bad_sparse_n(t.n))) return HIPRESS_ERR_SIZE;
     int rc = check_params(alg, pr);
     if (rc) return rc;
     if (!t.payload) return HIPRESS_ERR_NULL;
@@ -198,7 +201,7 @@ int build_encode_seg(int alg, const hipress_tensor& t, const hipress_params& pr,
 
 int build_decode_seg(int alg, const void* payload, int64_t payload_bytes, float* out, int64_t n, Seg* s) {
     std::memset(s, 0, sizeof(Seg));
-    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (bad_n(n) || (is_sparse(alg) && bad_sparse_n(n))) return HIPRESS_ERR_SIZE;
     if (!payload || (n > 0 && !out)) return HIPRESS_ERR_NULL;
     if (mis(payload, 16) || mis(out, 4)) return HIPRESS_ERR_ALIGN;
     if (payload_bytes < HIPRESS_HEADER_BYTES) return HIPRESS_ERR_SIZE;
@@ -374,7 +377,7 @@ int64_t hipress_terngrad_payload_bytes(int64_t n, int32_t bucket) {
     return HIPRESS_HEADER_BYTES + tg_scale_bytes(n, bucket) + words_bytes(n, 2);
 }
 int64_t hipress_sparse_capacity(int64_t n, double ratio) {
-    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (bad_sparse_n(n)) return HIPRESS_ERR_SIZE;
     if (bad_ratio(ratio)) return HIPRESS_ERR_PARAM;
     return sparse_plan(n, ratio).cap;
 }
@@ -386,7 +389,7 @@ int64_t hipress_onebit_workspace_bytes(int64_t n) {
     return bad_n(n) ? HIPRESS_ERR_SIZE : round_up(4 * (int64_t)tiles_of(n), 256);
 }
 int64_t hipress_sparse_workspace_bytes(int64_t n, double ratio) {
-    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (bad_sparse_n(n)) return HIPRESS_ERR_SIZE;
     if (bad_ratio(ratio)) return HIPRESS_ERR_PARAM;
     return sparse_ws_layout(sparse_plan(n, ratio).ns, tiles_of(n), 1).bytes;
 }
@@ -529,6 +532,16 @@ int64_t hipress_compll_payload_bytes(int64_t n, int32_t bitwidth) {
     return 10 + (n * bitwidth + 7) / 8;
 }
 
+// What hipress_compll_decode writes for a payload hipress_compll_encode made of n
+// elements: (8 * code bytes) / b - tail with tail = n mod 2^b, never more than n.
+int64_t hipress_compll_decoded_count(int64_t n, int32_t bitwidth) {
+    int64_t bytes = hipress_compll_payload_bytes(n, bitwidth);
+    if (bytes < 0) return bytes;
+    int64_t count = (8 * (bytes - 10)) / bitwidth - (n % (1LL << bitwidth));
+    if (count < 0) count = 0;
+    return count < n ? count : n;
+}
+
 int64_t hipress_compll_workspace_bytes(int64_t n) {
     return bad_n(n) ? HIPRESS_ERR_SIZE : round_up(8 * (int64_t)tiles_of(n), 256);
 }
@@ -618,7 +631,7 @@ int hipress_sparse_decode(const void* payload, int64_t payload_bytes, float* out
 static int build_merge_seg(int alg, const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
                            float* aggregate, int64_t n, bool reencode, MergeSeg* m) {
     std::memset(m, 0, sizeof(MergeSeg));
-    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (bad_n(n) || (is_sparse(alg) && bad_sparse_n(n))) return HIPRESS_ERR_SIZE;
     if (npeers < 1 || npeers > HIPRESS_MAX_PEERS) return HIPRESS_ERR_PARAM;
     if (!payloads || !payload_bytes || (n > 0 && !aggregate && !reencode)) return HIPRESS_ERR_NULL;
     if (mis(aggregate, 4)) return HIPRESS_ERR_ALIGN;
@@ -639,6 +652,12 @@ static int build_merge_seg(int alg, const void* const* payloads, const int64_t* 
     m->s.ntiles = tiles_of(n);
     m->s.aligned = al16(aggregate);
     return HIPRESS_OK;
+}
+
+// The state buffer asks for the re-encode; an empty chunk has no state buffer to point at,
+// so there the output payload does.
+static bool wants_reencode(const float* state, const void* out_payload, int64_t n) {
+    return state != nullptr || (n == 0 && out_payload != nullptr);
 }
 
 static MergeLaunch single_merge_launch(const MergeSeg& m, int npeers, bool reencode) {
@@ -669,10 +688,11 @@ int hipress_tbq_decode_merge(const void* const* payloads, const int64_t* payload
                              float* aggregate, int64_t n, float* residual, void* out_payload,
                              int64_t out_payload_bytes, float threshold, void* stream) {
     MergeSeg m;
-    int rc = build_merge_seg(HIPRESS_TBQ, payloads, payload_bytes, npeers, aggregate, n, residual != nullptr, &m);
+    const bool reenc = wants_reencode(residual, out_payload, n);
+    int rc = build_merge_seg(HIPRESS_TBQ, payloads, payload_bytes, npeers, aggregate, n, reenc, &m);
     if (rc) return rc;
-    if (residual && (rc = add_tbq_reencode(&m, residual, out_payload, out_payload_bytes, threshold))) return rc;
-    return hiperr(launch_dense_merge(single_merge_launch(m, npeers, residual != nullptr), HIPRESS_TBQ,
+    if (reenc && (rc = add_tbq_reencode(&m, residual, out_payload, out_payload_bytes, threshold))) return rc;
+    return hiperr(launch_dense_merge(single_merge_launch(m, npeers, reenc), HIPRESS_TBQ,
                                      static_cast<hipStream_t>(stream)));
 }
 
@@ -695,7 +715,7 @@ int hipress_terngrad_decode_merge(const void* const* payloads, const int64_t* pa
 }
 
 int64_t hipress_sparse_merge_workspace_bytes(int64_t n, int32_t npeers, double ratio, int32_t reencode) {
-    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (bad_sparse_n(n)) return HIPRESS_ERR_SIZE;
     if (npeers < 1 || npeers > HIPRESS_MAX_PEERS) return HIPRESS_ERR_PARAM;
     int64_t bytes = merge_index_bytes((int64_t)npeers * (tiles_of(n) + 1), 1, npeers);
     if (reencode) {
@@ -710,13 +730,14 @@ int hipress_sparse_decode_merge(const void* const* payloads, const int64_t* payl
                                 int64_t out_payload_bytes, double ratio, void* workspace,
                                 int64_t workspace_bytes, void* stream) {
     MergeSeg m;
-    int rc = build_merge_seg(HIPRESS_DGC, payloads, payload_bytes, npeers, aggregate, n, accumulator != nullptr, &m);
+    const bool reenc = wants_reencode(accumulator, out_payload, n);
+    int rc = build_merge_seg(HIPRESS_DGC, payloads, payload_bytes, npeers, aggregate, n, reenc, &m);
     if (rc) return rc;
     SparseWsLayout l{};
     const int64_t tp_words = (int64_t)npeers * (m.s.ntiles + 1);
     const int64_t ibytes = merge_index_bytes(tp_words, 1, npeers);
     int64_t need = ibytes;
-    if (accumulator) {
+    if (reenc) {
         // the gradient of this descriptor is never read (the merge kernel takes the sum from LDS): any valid pointer passes its checks
         hipress_tensor t{aggregate ? aggregate : accumulator, accumulator, nullptr, nullptr, out_payload, nullptr, n, out_payload_bytes};
         hipress_params pr{};
@@ -731,11 +752,11 @@ int hipress_sparse_decode_merge(const void* const* payloads, const int64_t* payl
     uint32_t* tileptr = reinterpret_cast<uint32_t*>(wsb);
     uint32_t* unsorted = reinterpret_cast<uint32_t*>(wsb + round_up(4 * tp_words, 256));
     SparseWs ws{};
-    if (accumulator) ws = sparse_ws_at(wsb + ibytes, l);
+    if (reenc) ws = sparse_ws_at(wsb + ibytes, l);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipError_t e = launch_sparse_merge(single_merge_launch(m, npeers, accumulator != nullptr), ws, tileptr, unsorted, -1, st);
+    hipError_t e = launch_sparse_merge(single_merge_launch(m, npeers, reenc), ws, tileptr, unsorted, -1, st);
     if (e != hipSuccess) return HIPRESS_ERR_HIP;
-    if (accumulator) e = launch_sparse_encode(single_launch(m.r), false, ws, kSparseAfterAccum, st);
+    if (reenc) e = launch_sparse_encode(single_launch(m.r), false, ws, kSparseAfterAccum, st);
     return hiperr(e);
 }
 
@@ -924,7 +945,7 @@ int hipress_merge_batch_create(hipress_merge_batch** out, int32_t alg, const hip
     int rc;
     bool any_state = false, all_state = true;
     for (int i = 0; i < count; ++i) {
-        if (chunks[i].state) any_state = true;
+        if (wants_reencode(chunks[i].state, chunks[i].out_payload, chunks[i].n)) any_state = true;
         else all_state = false;
     }
     if (any_state && !all_state) return fail(HIPRESS_ERR_NULL);  // re-encode is all chunks or none

@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kHeaderBlock) void compll_header_kernel(SegSrc src,
 __device__ __forceinline__ unsigned compll_code(float g, float u, float mn, float gap, float top) {
     if (!(gap > 0.f)) return 0u;
     float f = floorf((g - mn) / gap + u);
-    return f <= 0.f ? 0u : (f >= top ? (unsigned)top : (unsigned)f);
+    return !(f > 0.f) ? 0u : (f >= top ? (unsigned)top : (unsigned)f);  // NaN -> 0
 }
 
 template <class Src, int B>

@@ -29,7 +29,7 @@ __all__ = [
     "sparse_payload_bytes", "dgc_payload_bytes", "graddrop_payload_bytes",
     "onebit_encode", "onebit_decode", "onebit_encode_deferred", "onebit_residual", "tbq_encode", "tbq_decode", "terngrad_encode", "terngrad_decode",
     "dgc_encode", "dgc_decode", "graddrop_encode", "graddrop_decode",
-    "compll_payload_bytes", "compll_terngrad_encode", "compll_terngrad_decode",
+    "compll_payload_bytes", "compll_decoded_count", "compll_terngrad_encode", "compll_terngrad_decode",
     "onebit_decode_merge", "tbq_decode_merge", "terngrad_decode_merge", "dgc_decode_merge",
     "graddrop_decode_merge", "Batch", "MergeBatch", "ALIASES",
 ]
@@ -223,6 +223,13 @@ def compll_payload_bytes(n, bitwidth=2):
     return size(_lib.lib().hipress_compll_payload_bytes(n, int(bitwidth)), "compll_payload_bytes")
 
 
+def compll_decoded_count(n, bitwidth=2):
+    """Elements compll_terngrad_decode writes for a payload encoded from n elements: the
+    reference's count (8 * code bytes / bitwidth - tail, tail = n mod 2**bitwidth), which is
+    smaller than n for some n; the rest of the output buffer is left untouched."""
+    return size(_lib.lib().hipress_compll_decoded_count(n, int(bitwidth)), "compll_decoded_count")
+
+
 def compll_terngrad_encode(gradient, uniform, compressed, bitwidth=2):
     """The operator CompLL generates from pse/TernGradEncode.pse: min/max `bitwidth`-bit
     stochastic quantiser with the 10-byte header; `uniform` replaces random<float>(0,1)."""
@@ -237,7 +244,9 @@ def compll_terngrad_encode(gradient, uniform, compressed, bitwidth=2):
 
 
 def compll_terngrad_decode(compressed, gradient):
-    """Decode of that format; the element count comes from the payload length and its tail byte."""
+    """Decode of that format; the element count comes from the payload length and its tail
+    byte as in the reference and can fall short of gradient.numel() (see compll_decoded_count):
+    elements past it keep what the caller put there, so pass a zeroed buffer if that matters."""
     _u8(compressed, "compressed"); _f32(gradient, "gradient", compressed)
     with _on(gradient.device):
         check(_lib.lib().hipress_compll_decode(_p(compressed), compressed.numel(), _p(gradient), gradient.numel(),
@@ -281,6 +290,27 @@ def dgc_decode(compressed, gradient):
 
 
 graddrop_decode = dgc_decode
+
+
+# ---------------------------------------------------------------- the reference's own operator names
+def TernGradEncode(gradient, compressed, bitwidth=2, uniform=None):
+    """The operator the reference registers under this name
+    (/root/reference/src/CompLL/GCGen/output/TernGradEncode/TernGradEncode.cc:10-24):
+    arguments (gradient, compressed, bitwidth), the min/max `bitwidth`-bit stochastic
+    quantiser with the 10-byte [bitwidth][tail][min][max] header.  The reference draws its
+    rounding noise inside the operator from a clock-seeded generator
+    (TernGradEncode_body.h:49,119); here `uniform` supplies it, and when it is left out one
+    U[0,1) draw per element is taken from torch's generator for the gradient's device."""
+    if uniform is None:
+        _f32(gradient, "gradient")
+        uniform = torch.rand_like(gradient)
+    compll_terngrad_encode(gradient, uniform, compressed, bitwidth)
+
+
+def TernGradDecode(compressed, gradient):
+    """Decode of TernGradEncode's format, arguments as the reference registers them
+    (/root/reference/src/CompLL/GCGen/output/TernGradDecode/TernGradDecode.cc:10-24)."""
+    compll_terngrad_decode(compressed, gradient)
 
 
 # ---------------------------------------------------------------- decode-and-merge
@@ -499,10 +529,15 @@ class MergeBatch:
 # ---------------------------------------------------------------- aliases + torch.ops registration
 # CompLL names its generated operators <Func>Encode / <Func>Decode
 # (TernGradEncode.cc:10); one line per name maps them onto the operators above.
+# TernGradEncode / TernGradDecode are the reference's own registered operator (the
+# min/max quantiser, arguments gradient, compressed, bitwidth); the bucketed max-abs
+# ternariser, which the reference names only as the algorithm token "terngrad", goes by
+# BucketTernGradEncode / BucketTernGradDecode here.
 ALIASES = {
     "OnebitEncode": onebit_encode, "OnebitDecode": onebit_decode,
     "TBQEncode": tbq_encode, "TBQDecode": tbq_decode,
-    "TernGradEncode": terngrad_encode, "TernGradDecode": terngrad_decode,
+    "TernGradEncode": TernGradEncode, "TernGradDecode": TernGradDecode,
+    "BucketTernGradEncode": terngrad_encode, "BucketTernGradDecode": terngrad_decode,
     "DGCEncode": dgc_encode, "DGCDecode": dgc_decode,
     "GradDropEncode": graddrop_encode, "GradDropDecode": graddrop_decode,
 }
@@ -523,6 +558,8 @@ _SCHEMAS = {
     "graddrop_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
     "compll_terngrad_encode": "(Tensor gradient, Tensor uniform, Tensor(a!) compressed, int bitwidth=2) -> ()",
     "compll_terngrad_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
+    "TernGradEncode": "(Tensor gradient, Tensor(a!) compressed, int bitwidth=2, Tensor? uniform=None) -> ()",
+    "TernGradDecode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
     "onebit_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate) -> ()",
     "terngrad_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate) -> ()",
     "tbq_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate, Tensor(b!)? residual=None, "
@@ -534,7 +571,7 @@ _SCHEMAS = {
 }
 _ALIAS_OF = {
     "OnebitEncode": "onebit_encode", "OnebitDecode": "onebit_decode", "TBQEncode": "tbq_encode",
-    "TBQDecode": "tbq_decode", "TernGradEncode": "terngrad_encode", "TernGradDecode": "terngrad_decode",
+    "TBQDecode": "tbq_decode", "BucketTernGradEncode": "terngrad_encode", "BucketTernGradDecode": "terngrad_decode",
     "DGCEncode": "dgc_encode", "DGCDecode": "dgc_decode", "GradDropEncode": "graddrop_encode",
     "GradDropDecode": "graddrop_decode",
 }

@@ -59,6 +59,9 @@ extern "C" {
 #define HIPRESS_HEADER_BYTES 16
 #define HIPRESS_MAX_PEERS 16
 #define HIPRESS_MAX_N 4294967295LL /* n is carried as u32 in payload headers */
+/* DGC, GradDrop, hipress_sparse_decode and hipress_sparse_decode_merge (and batches of
+ * them) carry element indices as int32 in the payload: a larger n is HIPRESS_ERR_SIZE. */
+#define HIPRESS_SPARSE_MAX_N 2147483647LL
 
 enum hipress_alg {
     HIPRESS_ONEBIT = 0,
@@ -147,8 +150,14 @@ int hipress_terngrad_decode(const void *payload, int64_t payload_bytes, float *o
  * (i mod 8/b)*b of byte floor(i*b/8); bitwidth in {1,2,4,8}; no alignment is
  * required of `compressed`.  The rounding noise is an explicit uniform[0,1)
  * tensor.  Decode writes (8*compressed_bytes - 80)/b - tail elements, as the
- * reference does, but never more than n. */
+ * reference does (TernGradDecode_body.h:70-72), but never more than n.  With the
+ * encoder's tail = n mod 2^b (TernGradEncode_body.h:118) that count is SMALLER than n
+ * for some n (b = 2: two short when n mod 4 = 3; b = 4: up to 15; b = 8: n mod 256 short
+ * when n is no multiple of 256): out[count, n) is then left as the caller passed it.
+ * hipress_compll_decoded_count(n, bitwidth) is that count for a payload encoded from n
+ * elements (host arithmetic only). */
 int64_t hipress_compll_payload_bytes(int64_t n, int32_t bitwidth);
+int64_t hipress_compll_decoded_count(int64_t n, int32_t bitwidth);
 int64_t hipress_compll_workspace_bytes(int64_t n);
 int hipress_compll_encode(const float *grad, const float *uniform, int64_t n, void *compressed,
                           int64_t compressed_bytes, int32_t bitwidth, void *workspace,
@@ -177,7 +186,8 @@ int hipress_sparse_decode(const void *payload, int64_t payload_bytes, float *out
  * aggregate = NULL when only the re-encoded payload is wanted (an aggregator that
  * forwards the sum and applies no update itself): the sum is then never written
  * as fp32, which saves 4 of the step's bytes per element.  Payload and state come
- * out the same either way. */
+ * out the same either way.  (An empty chunk, n = 0, has no state buffer to point at:
+ * there a non-NULL out_payload asks for the re-encode, which writes the header.) */
 int hipress_tbq_decode_merge(const void *const *payloads, const int64_t *payload_bytes,
                              int32_t npeers, float *aggregate, int64_t n, float *residual,
                              void *out_payload, int64_t out_payload_bytes, float threshold,

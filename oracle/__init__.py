@@ -31,21 +31,20 @@ def build(force=False):
 
 def omp_lib():
     """The all-cores (OpenMP) build of the same source, for the CPU-baseline timing only:
-    hpo_tbq_* and hpo_onebit_* run their loops on every core."""
-    build()
-    if not os.path.exists(_SO_OMP):
-        subprocess.check_call(["make", "-C", _HERE, "libhipress_oracle_omp.so"], stdout=subprocess.DEVNULL)
-    L = ctypes.CDLL(_SO_OMP)
-    L.hpo_threads.restype = ctypes.c_int
-    L.hpo_onebit_encode.argtypes = [_ptr, _ptr, _i64, _ptr]
-    L.hpo_onebit_decode.argtypes = [_ptr, _ptr, _i64]
-    L.hpo_tbq_encode.argtypes = [_ptr, _ptr, _i64, _ptr, _f32]
-    L.hpo_tbq_decode.argtypes = [_ptr, _ptr, _i64]
-    L.hpo_onebit_scale.restype = _f32
-    L.hpo_onebit_scale.argtypes = [_ptr, _ptr, _i64]
-    return L
+    same entry points, every loop with independent iterations shared between the cores."""
+    global _omp
+    if _omp is None:
+        build()
+        if not os.path.exists(_SO_OMP):
+            subprocess.check_call(["make", "-C", _HERE, "libhipress_oracle_omp.so"], stdout=subprocess.DEVNULL)
+        L = ctypes.CDLL(_SO_OMP)
+        _bind(L)
+        L.hpo_threads.restype = ctypes.c_int
+        _omp = L
+    return _omp
 
 
+_omp = None
 _lib = None
 
 _i64 = ctypes.c_int64
@@ -54,48 +53,54 @@ _f64 = ctypes.c_double
 _ptr = ctypes.c_void_p
 
 
+_SIG = {
+    "hpo_get_code": (ctypes.c_uint32, [_ptr, _i64, ctypes.c_int]),
+    "hpo_put_code": (None, [_ptr, _i64, ctypes.c_int, ctypes.c_uint32]),
+    "hpo_onebit_payload_bytes": (_i64, [_i64]),
+    "hpo_tbq_payload_bytes": (_i64, [_i64]),
+    "hpo_terngrad_scale_bytes": (_i64, [_i64, _i64]),
+    "hpo_terngrad_payload_bytes": (_i64, [_i64, _i64]),
+    "hpo_sparse_capacity": (_i64, [_i64, _f64]),
+    "hpo_sparse_payload_bytes": (_i64, [_i64, _f64]),
+    "hpo_tbq_encode": (None, [_ptr, _ptr, _i64, _ptr, _f32]),
+    "hpo_tbq_decode": (None, [_ptr, _ptr, _i64]),
+    "hpo_onebit_scale": (_f32, [_ptr, _ptr, _i64]),
+    "hpo_onebit_encode_with_scale": (None, [_ptr, _ptr, _i64, _ptr, _f32]),
+    "hpo_onebit_encode": (None, [_ptr, _ptr, _i64, _ptr]),
+    "hpo_onebit_decode": (None, [_ptr, _ptr, _i64]),
+    "hpo_terngrad_encode": (None, [_ptr, _ptr, _i64, _ptr, _i64]),
+    "hpo_terngrad_decode": (None, [_ptr, _ptr, _i64]),
+    "hpo_sparse_sample_stride": (_i64, [_i64]),
+    "hpo_sparse_sample_count": (_i64, [_i64]),
+    "hpo_sparse_sample_k": (_i64, [_i64, _f64]),
+    "hpo_sparse_threshold": (_f32, [_ptr, _i64, _f64]),
+    "hpo_dgc_encode": (None, [_ptr, _ptr, _ptr, _i64, _ptr, _f32, _f64]),
+    "hpo_graddrop_encode": (None, [_ptr, _ptr, _i64, _ptr, _f64]),
+    "hpo_sparse_decode": (None, [_ptr, _ptr, _i64]),
+    "hpo_tbq_decode_merge": (None, [_ptr, ctypes.c_int, _ptr, _i64, _ptr, _ptr, _f32]),
+    "hpo_onebit_decode_merge": (None, [_ptr, ctypes.c_int, _ptr, _i64]),
+    "hpo_terngrad_decode_merge": (None, [_ptr, ctypes.c_int, _ptr, _i64]),
+    "hpo_sparse_decode_merge": (None, [_ptr, ctypes.c_int, _ptr, _i64, _ptr, _ptr, _f64]),
+    "hpo_compll_decode": (_i64, [_ptr, _i64, _ptr, _i64]),
+    "hpo_compll_payload_bytes": (_i64, [_i64, ctypes.c_int]),
+    "hpo_compll_encode": (_i64, [_ptr, _ptr, _i64, _ptr, ctypes.c_int]),
+    "hpo_lcg_uniform": (None, [ctypes.c_uint32, _f32, _f32, _ptr, _i64]),
+}
+
+
+def _bind(L):
+    for name, (res, args) in _SIG.items():
+        fn = getattr(L, name)
+        fn.restype = res
+        fn.argtypes = args
+
+
 def lib():
     global _lib
     if _lib is None:
         build()
         L = ctypes.CDLL(_SO)
-        sig = {
-            "hpo_get_code": (ctypes.c_uint32, [_ptr, _i64, ctypes.c_int]),
-            "hpo_put_code": (None, [_ptr, _i64, ctypes.c_int, ctypes.c_uint32]),
-            "hpo_onebit_payload_bytes": (_i64, [_i64]),
-            "hpo_tbq_payload_bytes": (_i64, [_i64]),
-            "hpo_terngrad_scale_bytes": (_i64, [_i64, _i64]),
-            "hpo_terngrad_payload_bytes": (_i64, [_i64, _i64]),
-            "hpo_sparse_capacity": (_i64, [_i64, _f64]),
-            "hpo_sparse_payload_bytes": (_i64, [_i64, _f64]),
-            "hpo_tbq_encode": (None, [_ptr, _ptr, _i64, _ptr, _f32]),
-            "hpo_tbq_decode": (None, [_ptr, _ptr, _i64]),
-            "hpo_onebit_scale": (_f32, [_ptr, _ptr, _i64]),
-            "hpo_onebit_encode_with_scale": (None, [_ptr, _ptr, _i64, _ptr, _f32]),
-            "hpo_onebit_encode": (None, [_ptr, _ptr, _i64, _ptr]),
-            "hpo_onebit_decode": (None, [_ptr, _ptr, _i64]),
-            "hpo_terngrad_encode": (None, [_ptr, _ptr, _i64, _ptr, _i64]),
-            "hpo_terngrad_decode": (None, [_ptr, _ptr, _i64]),
-            "hpo_sparse_sample_stride": (_i64, [_i64]),
-            "hpo_sparse_sample_count": (_i64, [_i64]),
-            "hpo_sparse_sample_k": (_i64, [_i64, _f64]),
-            "hpo_sparse_threshold": (_f32, [_ptr, _i64, _f64]),
-            "hpo_dgc_encode": (None, [_ptr, _ptr, _ptr, _i64, _ptr, _f32, _f64]),
-            "hpo_graddrop_encode": (None, [_ptr, _ptr, _i64, _ptr, _f64]),
-            "hpo_sparse_decode": (None, [_ptr, _ptr, _i64]),
-            "hpo_tbq_decode_merge": (None, [_ptr, ctypes.c_int, _ptr, _i64, _ptr, _ptr, _f32]),
-            "hpo_onebit_decode_merge": (None, [_ptr, ctypes.c_int, _ptr, _i64]),
-            "hpo_terngrad_decode_merge": (None, [_ptr, ctypes.c_int, _ptr, _i64]),
-            "hpo_sparse_decode_merge": (None, [_ptr, ctypes.c_int, _ptr, _i64, _ptr, _ptr, _f64]),
-            "hpo_compll_decode": (_i64, [_ptr, _i64, _ptr, _i64]),
-            "hpo_compll_payload_bytes": (_i64, [_i64, ctypes.c_int]),
-            "hpo_compll_encode": (_i64, [_ptr, _ptr, _i64, _ptr, ctypes.c_int]),
-            "hpo_lcg_uniform": (None, [ctypes.c_uint32, _f32, _f32, _ptr, _i64]),
-        }
-        for name, (res, args) in sig.items():
-            fn = getattr(L, name)
-            fn.restype = res
-            fn.argtypes = args
+        _bind(L)
         _lib = L
     return _lib
 

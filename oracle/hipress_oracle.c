@@ -41,7 +41,7 @@
  * in-tree operator and is pinned by its header layout, grid-point round trips
  * through hpo_compll_decode and a float64 closed form.
  *
- * Build: gcc -O2 -ffp-contract=off -fno-fast-math (see oracle/Makefile).  All
+ * Build: gcc -O3 -ffp-contract=off -fno-fast-math (see oracle/Makefile).  All
  * arithmetic is IEEE binary32 round-to-nearest with no contraction.
  */
 #include <math.h>
@@ -52,17 +52,25 @@
 #define HPO_HEADER_BYTES 16
 
 /* The same source builds the all-cores variant of the CPU baseline (-fopenmp
- * -DHPO_OMP, libhipress_oracle_omp.so): the TBQ and onebit loops run one packed
- * word per iteration, so iterations never share a word.  Without HPO_OMP the
- * pragmas vanish and every loop is sequential. */
+ * -DHPO_OMP, libhipress_oracle_omp.so).  Loops whose iterations are independent
+ * are shared between the cores: the quantisers run one packed word (or one bucket
+ * of whole words, or one byte) per iteration so that iterations never share a
+ * word, element-wise loops run as they are, counts are reductions.  What depends
+ * on order stays sequential in both builds: the radix selection of a threshold and
+ * the walk that emits the selected pairs in ascending index order.  Without
+ * HPO_OMP the pragmas vanish and every loop is sequential. */
 #ifdef HPO_OMP
 #define HPO_PRAGMA(x) _Pragma(#x)
 #define HPO_PARALLEL_FOR HPO_PRAGMA(omp parallel for schedule(static))
+#define HPO_PARALLEL_FOR_IF(c) HPO_PRAGMA(omp parallel for schedule(static) if (c))
 #define HPO_PARALLEL_SUM(v) HPO_PRAGMA(omp parallel for schedule(static) reduction(+ : v))
+#define HPO_PARALLEL_MINMAX(a, b) HPO_PRAGMA(omp parallel for schedule(static) reduction(max : a) reduction(min : b))
 int hpo_threads(void);
 #else
 #define HPO_PARALLEL_FOR
+#define HPO_PARALLEL_FOR_IF(c)
 #define HPO_PARALLEL_SUM(v)
+#define HPO_PARALLEL_MINMAX(a, b)
 #endif
 
 /* ------------------------------------------------------------------ */
@@ -260,6 +268,8 @@ void hpo_terngrad_encode(const float *g, const float *u, int64_t n, uint8_t *pay
     hdr[3] = 0;
     memset(scale, 0, sb);
     memset(w, 0, 4 * words_for(n, 2));
+    /* buckets of whole words (a multiple of 16 codes) never share a word */
+    HPO_PARALLEL_FOR_IF(bucket % 16 == 0)
     for (int64_t k = 0; k < nb; ++k) {
         int64_t lo = k * bucket, hi = lo + bucket < n ? lo + bucket : n;
         float s = 0.0f;
@@ -284,6 +294,7 @@ void hpo_terngrad_decode(const uint8_t *payload, float *out, int64_t n)
     int64_t bucket = hdr[1];
     const float *scale = (const float *)(payload + HPO_HEADER_BYTES);
     const uint32_t *w = (const uint32_t *)(payload + HPO_HEADER_BYTES + hpo_terngrad_scale_bytes(n, bucket));
+    HPO_PARALLEL_FOR
     for (int64_t i = 0; i < n; ++i) {
         float s = scale[i / bucket];
         out[i] = tbq_value(hpo_get_code(w, i, 2), s);
@@ -384,6 +395,7 @@ static void sparse_select(float *a, float *mom, int64_t n, uint8_t *payload, dou
     uint32_t tk = abs_key(thr);
     int64_t count = 0, eq_quota = INT64_MAX, nnz = 0;
 
+    HPO_PARALLEL_SUM(count)
     for (int64_t i = 0; i < n; ++i) {
         uint32_t k = abs_key(a[i]);
         if (k >= tk && k > 0) count++;
@@ -391,10 +403,12 @@ static void sparse_select(float *a, float *mom, int64_t n, uint8_t *payload, dou
     if (count > cap) {
         uint32_t *keys = (uint32_t *)malloc(sizeof(uint32_t) * (size_t)n);
         int64_t gt = 0;
+        HPO_PARALLEL_FOR
         for (int64_t i = 0; i < n; ++i) keys[i] = abs_key(a[i]);
         tk = kth_largest(keys, n, cap);
         free(keys);
         thr = key_value(tk);
+        HPO_PARALLEL_SUM(gt)
         for (int64_t i = 0; i < n; ++i)
             if (abs_key(a[i]) > tk) gt++;
         eq_quota = cap - gt;
@@ -428,6 +442,7 @@ static void sparse_select(float *a, float *mom, int64_t n, uint8_t *payload, dou
 void hpo_dgc_encode(const float *g, float *mom, float *acc, int64_t n, uint8_t *payload, float m,
                     double ratio)
 {
+    HPO_PARALLEL_FOR
     for (int64_t i = 0; i < n; ++i) {
         float p = m * mom[i]; /* rounded product: the build disables contraction */
         float u = p + g[i];
@@ -441,6 +456,7 @@ void hpo_dgc_encode(const float *g, float *mom, float *acc, int64_t n, uint8_t *
  * (drop ratio 0.99 = ratio 0.01). */
 void hpo_graddrop_encode(const float *g, float *acc, int64_t n, uint8_t *payload, double ratio)
 {
+    HPO_PARALLEL_FOR
     for (int64_t i = 0; i < n; ++i) acc[i] = acc[i] + g[i];
     sparse_select(acc, NULL, n, payload, ratio);
 }
@@ -453,7 +469,8 @@ void hpo_sparse_decode(const uint8_t *payload, float *out, int64_t n)
     const int32_t *idx = (const int32_t *)(payload + HPO_HEADER_BYTES);
     const float *val = (const float *)(payload + HPO_HEADER_BYTES + 4 * cap);
     if (nnz > cap) nnz = cap;
-    memset(out, 0, sizeof(float) * (size_t)n);
+    HPO_PARALLEL_FOR
+    for (int64_t i = 0; i < n; ++i) out[i] = 0.0f;
     for (int64_t j = 0; j < nnz; ++j)
         if (idx[j] >= 0 && idx[j] < n) out[idx[j]] = val[j];
 }
@@ -468,11 +485,13 @@ void hpo_sparse_decode(const uint8_t *payload, float *out, int64_t n)
 void hpo_tbq_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n, float *r,
                           uint8_t *out_payload, float tau)
 {
+    HPO_PARALLEL_FOR
     for (int64_t i = 0; i < n; ++i) agg[i] = 0.0f;
     for (int p = 0; p < npeers; ++p) {
         float t;
         const uint32_t *w = (const uint32_t *)(payloads[p] + HPO_HEADER_BYTES);
         memcpy(&t, payloads[p], 4);
+        HPO_PARALLEL_FOR
         for (int64_t i = 0; i < n; ++i) agg[i] = agg[i] + tbq_value(hpo_get_code(w, i, 2), t);
     }
     if (r) hpo_tbq_encode(agg, r, n, out_payload, tau);
@@ -480,17 +499,20 @@ void hpo_tbq_decode_merge(const uint8_t *const *payloads, int npeers, float *agg
 
 void hpo_onebit_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n)
 {
+    HPO_PARALLEL_FOR
     for (int64_t i = 0; i < n; ++i) agg[i] = 0.0f;
     for (int p = 0; p < npeers; ++p) {
         float s;
         const uint32_t *w = (const uint32_t *)(payloads[p] + HPO_HEADER_BYTES);
         memcpy(&s, payloads[p], 4);
+        HPO_PARALLEL_FOR
         for (int64_t i = 0; i < n; ++i) agg[i] = agg[i] + (hpo_get_code(w, i, 1) ? s : -s);
     }
 }
 
 void hpo_terngrad_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n)
 {
+    HPO_PARALLEL_FOR
     for (int64_t i = 0; i < n; ++i) agg[i] = 0.0f;
     for (int p = 0; p < npeers; ++p) {
         const uint32_t *hdr = (const uint32_t *)payloads[p];
@@ -498,6 +520,7 @@ void hpo_terngrad_decode_merge(const uint8_t *const *payloads, int npeers, float
         const float *scale = (const float *)(payloads[p] + HPO_HEADER_BYTES);
         const uint32_t *w =
             (const uint32_t *)(payloads[p] + HPO_HEADER_BYTES + hpo_terngrad_scale_bytes(n, bucket));
+        HPO_PARALLEL_FOR
         for (int64_t i = 0; i < n; ++i)
             agg[i] = agg[i] + tbq_value(hpo_get_code(w, i, 2), scale[i / bucket]);
     }
@@ -510,7 +533,8 @@ void hpo_terngrad_decode_merge(const uint8_t *const *payloads, int npeers, float
 void hpo_sparse_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n,
                              float *acc, uint8_t *out_payload, double ratio)
 {
-    memset(agg, 0, sizeof(float) * (size_t)n);
+    HPO_PARALLEL_FOR
+    for (int64_t i = 0; i < n; ++i) agg[i] = 0.0f;
     for (int p = 0; p < npeers; ++p) {
         const uint32_t *hdr = (const uint32_t *)payloads[p];
         int64_t nnz = hdr[0], cap = hdr[2];
@@ -544,6 +568,7 @@ int64_t hpo_compll_decode(const uint8_t *compressed, int64_t csz, float *out, in
     gap = (mx - mn) / (float)((1 << b) - 1);
     count = (8 * csz - 80) / b - tail;
     if (count > out_cap) count = out_cap;
+    HPO_PARALLEL_FOR
     for (int64_t i = 0; i < count; ++i) {
         uint32_t code = (Q[i * b / 8] >> ((i % (8 / b)) * b)) & ((1u << b) - 1u);
         out[i] = (float)code * gap + mn;
@@ -559,7 +584,8 @@ int64_t hpo_compll_decode(const uint8_t *compressed, int64_t csz, float *out, in
  *   max = reduce(g, -99999, greater), min = reduce(g, 99999, smaller) in float;
  *   gap = (max - min) / ((1<<b) - 1);  tail = n % (1<<b) kept as uint8;
  *   code_i = floor((g_i - min) / gap + u_i), u_i an explicit uniform[0,1) draw in
- *   place of random<float>(0,1), limited to [0, 2^b - 1]; gap == 0 gives code 0;
+ *   place of random<float>(0,1), limited to [0, 2^b - 1]; gap == 0 gives code 0, and so
+ *   does a value that is no number (a NaN gradient, or Inf/Inf when the range is infinite);
  *   code i is stored where the decoder reads it: bit (i mod 8/b)*b of byte
  *   floor(i*b/8) after the 10-byte header [b][tail][min][max]
  *   (TernGradEncode_body.h:114,120-123; TernGradDecode_body.h:44).
@@ -573,6 +599,8 @@ int64_t hpo_compll_encode(const float *g, const float *u, int64_t n, uint8_t *co
     uint8_t *Q = compressed + 10;
     uint8_t tail = (uint8_t)(n % (1 << b));
     uint32_t top = (1u << b) - 1u;
+    int per = 8 / b;
+    HPO_PARALLEL_MINMAX(mx, mn)
     for (int64_t i = 0; i < n; ++i) {
         if (g[i] > mx) mx = g[i];
         if (g[i] < mn) mn = g[i];
@@ -582,15 +610,21 @@ int64_t hpo_compll_encode(const float *g, const float *u, int64_t n, uint8_t *co
     compressed[1] = tail;
     memcpy(compressed + 2, &mn, 4);
     memcpy(compressed + 6, &mx, 4);
-    memset(Q, 0, (size_t)nbytes);
-    for (int64_t i = 0; i < n; ++i) {
-        uint32_t code = 0;
-        if (gap > 0.0f) {
-            float r = (g[i] - mn) / gap + u[i];
-            float f = floorf(r);
-            code = f <= 0.0f ? 0u : (f >= (float)top ? top : (uint32_t)f);
+    /* one output byte (8/b codes) per iteration, so that iterations never share a byte */
+    HPO_PARALLEL_FOR
+    for (int64_t k = 0; k < nbytes; ++k) {
+        int64_t hi = (k + 1) * per < n ? (k + 1) * per : n;
+        uint8_t q = 0;
+        for (int64_t i = k * per; i < hi; ++i) {
+            uint32_t code = 0;
+            if (gap > 0.0f) {
+                float r = (g[i] - mn) / gap + u[i];
+                float f = floorf(r);
+                code = !(f > 0.0f) ? 0u : (f >= (float)top ? top : (uint32_t)f); /* NaN -> 0 */
+            }
+            q |= (uint8_t)(code << ((i % per) * b));
         }
-        Q[i * b / 8] |= (uint8_t)(code << ((i % (8 / b)) * b));
+        Q[k] = q;
     }
     return 10 + nbytes;
 }

@@ -89,3 +89,73 @@ def test_null_and_range_checks_need_no_gpu(lib):
     nb = (ctypes.c_int64 * 1)(1 << 20)
     assert L.hipress_tbq_decode_merge(pay, nb, 1, None, 16, None, None, 0, 0.05, None) == -1
     assert L.hipress_onebit_decode_merge(pay, nb, 1, None, 16, None) == -1
+
+
+def test_sparse_entry_points_reject_what_int32_indices_cannot_address(lib):
+    """DGC / GradDrop payloads carry int32 indices: n above 2^31 - 1 is refused on the host,
+    before any launch (the pointers below are never touched)."""
+    L = lib.lib()
+    big, ok = (1 << 31), (1 << 31) - 1
+    fake = ctypes.c_void_p(1 << 20)
+    assert L.hipress_sparse_capacity(big, 0.001) == -2
+    assert L.hipress_sparse_payload_bytes(big, 0.001) == -2
+    assert L.hipress_sparse_workspace_bytes(big, 0.001) == -2
+    assert L.hipress_sparse_merge_workspace_bytes(big, 8, 0.001, 1) == -2
+    assert L.hipress_sparse_capacity(ok, 0.001) > 0
+    assert L.hipress_sparse_capacity(ok, 1.0) == 1 << 31  # whole tensor, rounded up to 64: still fits u32
+    nbytes = 1 << 40
+    assert L.hipress_dgc_encode(fake, fake, fake, big, fake, nbytes, 0.9, 0.001, fake, nbytes, None) == -2
+    assert L.hipress_graddrop_encode(fake, fake, big, fake, nbytes, 0.01, fake, nbytes, None) == -2
+    assert L.hipress_sparse_decode(fake, nbytes, fake, big, None) == -2
+    pay = (ctypes.c_void_p * 1)(1 << 20)
+    nb = (ctypes.c_int64 * 1)(nbytes)
+    assert L.hipress_sparse_decode_merge(pay, nb, 1, fake, big, None, None, 0, 0.001, fake, nbytes, None) == -2
+    # batches: the check precedes every allocation
+    t = lib.Tensor(fake.value, fake.value, fake.value, None, fake.value, fake.value, big, nbytes)
+    pr = lib.Params(0.0, 512, 0.9, 0.0, 0.001)
+    h = ctypes.c_void_p()
+    for alg in (lib.DGC, lib.GRADDROP):
+        assert L.hipress_batch_create(ctypes.byref(h), alg, ctypes.byref(t), 1, ctypes.byref(pr)) == -2
+        assert not h.value
+    mc = lib.MergeChunk()
+    mc.payloads[0], mc.payload_bytes[0] = fake.value, nbytes
+    mc.aggregate, mc.n = fake.value, big
+    assert L.hipress_merge_batch_create(ctypes.byref(h), lib.DGC, ctypes.byref(mc), 1, 1, ctypes.byref(pr)) == -2
+    # the dense formats carry no indices and keep the u32 limit
+    assert L.hipress_tbq_payload_bytes(big) > 0
+
+
+@pytest.mark.parametrize("b", [1, 2, 4, 8])
+def test_compll_decoded_count_is_the_reference_formula(lib, b):
+    """count = (8 * code bytes) / b - n mod 2^b (TernGradDecode_body.h:70-72 with the
+    encoder's tail, TernGradEncode_body.h:118), clamped to n; checked against the oracle's
+    decoder, which writes exactly that many elements."""
+    import numpy as np
+
+    L = lib.lib()
+    for n in (0, 1, 3, 4, 5, 7, 255, 256, 257, 1000, 4097):
+        want = min(n, max(0, 8 * ((n * b + 7) // 8) // b - n % (1 << b)))
+        assert L.hipress_compll_decoded_count(n, b) == want
+        pay = oracle.compll_encode(np.linspace(-1, 1, n, dtype=np.float32), np.zeros(n, np.float32), b)
+        assert oracle.compll_decode(pay, n).size == want
+    assert L.hipress_compll_decoded_count(10, 3) == -4
+
+
+def test_reference_operator_names_keep_the_reference_signature():
+    """TernGradEncode(gradient, compressed, bitwidth) / TernGradDecode(compressed, gradient) as
+    registered in the reference (TernGradEncode.cc:16,21-23; TernGradDecode.cc:16)."""
+    import inspect
+
+    import torch
+
+    from hipress_amd import ops
+
+    enc = list(inspect.signature(ops.ALIASES["TernGradEncode"]).parameters)
+    assert enc[:3] == ["gradient", "compressed", "bitwidth"]
+    assert list(inspect.signature(ops.ALIASES["TernGradDecode"]).parameters) == ["compressed", "gradient"]
+    schema = torch.ops.hipress.TernGradEncode.default._schema
+    assert [a.name for a in schema.arguments][:3] == ["gradient", "compressed", "bitwidth"]
+    assert [a.name for a in torch.ops.hipress.TernGradDecode.default._schema.arguments] == ["compressed", "gradient"]
+    assert len(schema.returns) == 0  # in place, zero outputs (TernGradEncode.cc:12-13)
+    # the bucketed ternariser keeps its own name
+    assert ops.ALIASES["BucketTernGradEncode"] is ops.terngrad_encode

@@ -106,3 +106,49 @@ def test_constant_tensor_and_bad_bitwidth(hp):
     out = torch.full((n,), 7.0, device="cuda")
     hp.compll_terngrad_decode(bad, out)
     assert (host(out) == 7.0).all()
+
+
+@pytest.mark.parametrize("b", [2, 4])
+def test_reference_operator_name_is_the_in_tree_operator(hp, b):
+    """TernGradEncode(gradient, compressed, bitwidth) under the reference's own name and
+    argument order produces the in-tree format, byte for byte the oracle's payload."""
+    n = 70001
+    rng = np.random.default_rng(41 + b)
+    g, u = rng.normal(0, 1e-2, n).astype(F), rng.random(n, dtype=F)
+    want = oracle.compll_encode(g, u, b)
+    pay = torch.zeros(want.size, dtype=torch.uint8, device="cuda")
+    hp.TernGradEncode(dev(g), pay, b, uniform=dev(u))
+    np.testing.assert_array_equal(host(pay), want)
+    pay.zero_()
+    torch.ops.hipress.TernGradEncode(dev(g), pay, b, dev(u))
+    np.testing.assert_array_equal(host(pay), want)
+    out = torch.zeros(n, device="cuda")
+    torch.ops.hipress.TernGradDecode(pay, out)
+    ref = oracle.compll_decode(want, n)
+    np.testing.assert_array_equal(host(out)[: ref.size], ref)
+    # without `uniform` the noise is drawn inside the operator, as in the reference: the header
+    # (bit width, tail, min, max) is still the oracle's, the codes stay within one level of it
+    pay2 = torch.zeros(want.size, dtype=torch.uint8, device="cuda")
+    hp.TernGradEncode(dev(g), pay2, b)
+    got = host(pay2)
+    np.testing.assert_array_equal(got[:10], want[:10])
+    lo, hi = oracle.compll_encode(g, np.zeros(n, F), b), oracle.compll_encode(g, np.full(n, np.nextafter(F(1), F(0)), F), b)
+    per = 8 // b
+    codes = lambda p: np.stack([(p[10:] >> (b * k)) & ((1 << b) - 1) for k in range(per)], 1).reshape(-1)[:n]
+    assert (codes(got) >= codes(lo)).all() and (codes(got) <= codes(hi)).all()
+
+
+@pytest.mark.parametrize("n,b", [(1000, 8), (4097 + 250, 8), (70015, 4), (4099, 2)])
+def test_decode_leaves_the_remainder_as_the_caller_passed_it(hp, n, b):
+    """The reference's count (8 * code bytes / b - tail) falls short of n when n mod 2^b != 0:
+    out[count, n) keeps the caller's values and hipress_compll_decoded_count names the count."""
+    rng = np.random.default_rng(n + b)
+    want = oracle.compll_encode(rng.normal(0, 1, n).astype(F), rng.random(n, dtype=F), b)
+    count = hp.compll_decoded_count(n, b)
+    ref = oracle.compll_decode(want, n)
+    assert count == ref.size and count < n
+    out = torch.full((n,), 7.0, device="cuda")
+    hp.compll_terngrad_decode(dev(want), out)
+    got = host(out)
+    np.testing.assert_array_equal(got[:count], ref)
+    assert (got[count:] == 7.0).all()
