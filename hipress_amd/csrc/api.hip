@@ -71,7 +71,7 @@ inline SparseWsLayout sparse_ws_layout(int64_t total_ns, int64_t total_tiles, in
     l.thr_off = off;
     off += round_up(4 * 2 * nsegs, 256);
     l.hist_off = off;
-    off += round_up(4 * 3 * 2048 * nsegs, 256);
+    off += round_up(4 * (int64_t)kSelHistWords * nsegs, 256);
     l.ctl_off = off;
     off += round_up(4 * 8 * nsegs, 256);
     l.bytes = off;
@@ -90,10 +90,9 @@ inline SparseWs sparse_ws_at(void* base, const SparseWsLayout& l) {
     return w;
 }
 
-// Index part of a sparse merge workspace: per chunk npeers x (tiles + 1) tile
-// pointers, then one "not sorted" flag per (chunk, peer).
-inline int64_t merge_index_bytes(int64_t tileptr_words, int64_t nchunks, int64_t npeers) {
-    return round_up(4 * tileptr_words, 256) + round_up(4 * nchunks * npeers, 256);
+// Index part of a sparse merge workspace: per tile a head and one run record per peer.
+inline int64_t merge_index_bytes(int64_t ntiles, int64_t npeers) {
+    return round_up((int64_t)sizeof(PeerRun) * ntiles * kMergeRecs((unsigned)npeers), 256);
 }
 
 inline int hiperr(hipError_t e) { return e == hipSuccess ? HIPRESS_OK : HIPRESS_ERR_HIP; }
@@ -342,8 +341,7 @@ struct hipress_merge_batch {
     unsigned ntiles = 0, nstiles = 0;
     void* ws = nullptr;
     SparseWsLayout swl{};
-    void* iws = nullptr;  // sparse: tile pointers and "not sorted" flags
-    int64_t tp_words = 0;
+    void* iws = nullptr;  // sparse: per tile a head and one run record per peer
 };
 
 extern "C" {
@@ -717,7 +715,7 @@ int hipress_terngrad_decode_merge(const void* const* payloads, const int64_t* pa
 int64_t hipress_sparse_merge_workspace_bytes(int64_t n, int32_t npeers, double ratio, int32_t reencode) {
     if (bad_sparse_n(n)) return HIPRESS_ERR_SIZE;
     if (npeers < 1 || npeers > HIPRESS_MAX_PEERS) return HIPRESS_ERR_PARAM;
-    int64_t bytes = merge_index_bytes((int64_t)npeers * (tiles_of(n) + 1), 1, npeers);
+    int64_t bytes = merge_index_bytes(tiles_of(n), npeers);
     if (reencode) {
         if (bad_ratio(ratio)) return HIPRESS_ERR_PARAM;
         bytes += sparse_ws_layout(sparse_plan(n, ratio).ns, tiles_of(n), 1).bytes;
@@ -734,8 +732,7 @@ int hipress_sparse_decode_merge(const void* const* payloads, const int64_t* payl
     int rc = build_merge_seg(HIPRESS_DGC, payloads, payload_bytes, npeers, aggregate, n, reenc, &m);
     if (rc) return rc;
     SparseWsLayout l{};
-    const int64_t tp_words = (int64_t)npeers * (m.s.ntiles + 1);
-    const int64_t ibytes = merge_index_bytes(tp_words, 1, npeers);
+    const int64_t ibytes = merge_index_bytes(m.s.ntiles, npeers);
     int64_t need = ibytes;
     if (reenc) {
         // the gradient of this descriptor is never read (the merge kernel takes the sum from LDS): any valid pointer passes its checks
@@ -749,12 +746,11 @@ int hipress_sparse_decode_merge(const void* const* payloads, const int64_t* payl
     if (!workspace || workspace_bytes < need) return HIPRESS_ERR_WORKSPACE;
     if (mis(workspace, 16)) return HIPRESS_ERR_ALIGN;
     uint8_t* wsb = static_cast<uint8_t*>(workspace);
-    uint32_t* tileptr = reinterpret_cast<uint32_t*>(wsb);
-    uint32_t* unsorted = reinterpret_cast<uint32_t*>(wsb + round_up(4 * tp_words, 256));
+    PeerRun* runs = reinterpret_cast<PeerRun*>(wsb);
     SparseWs ws{};
     if (reenc) ws = sparse_ws_at(wsb + ibytes, l);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipError_t e = launch_sparse_merge(single_merge_launch(m, npeers, reenc), ws, tileptr, unsorted, -1, st);
+    hipError_t e = launch_sparse_merge(single_merge_launch(m, npeers, reenc), ws, runs, -1, st);
     if (e != hipSuccess) return HIPRESS_ERR_HIP;
     if (reenc) e = launch_sparse_encode(single_launch(m.r), false, ws, kSparseAfterAccum, st);
     return hiperr(e);
@@ -981,13 +977,7 @@ int hipress_merge_batch_create(hipress_merge_batch** out, int32_t alg, const hip
         for (size_t i = 0; i < b->segs.size(); ++i) b->segs[i].r = b->renc[i];  // the merge kernel runs their first launch
     }
     if (sparse) {
-        int64_t words = 0;
-        for (MergeSeg& m : b->segs) {
-            m.tp0 = (unsigned long long)words;
-            words += (int64_t)npeers * (m.s.ntiles + 1);
-        }
-        b->tp_words = words;
-        if (hipMalloc(&b->iws, (size_t)merge_index_bytes(words, count, npeers)) != hipSuccess) return fail(HIPRESS_ERR_HIP);
+        if (hipMalloc(&b->iws, (size_t)merge_index_bytes(b->ntiles ? b->ntiles : 1, npeers)) != hipSuccess) return fail(HIPRESS_ERR_HIP);
     }
     if ((rc = upload(b->segs, &b->d_segs))) return fail(rc);
     if ((rc = upload(b->renc, &b->d_renc))) return fail(rc);
@@ -1013,12 +1003,11 @@ static int merge_batch_run_impl(hipress_merge_batch* b, int phase, void* stream)
     L.reencode = b->reencode;
     if (b->alg == HIPRESS_DGC || b->alg == HIPRESS_GRADDROP) {
         if (phase > 2) return HIPRESS_ERR_PARAM;
-        uint32_t* tileptr = static_cast<uint32_t*>(b->iws);
-        uint32_t* unsorted = reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(b->iws) + round_up(4 * b->tp_words, 256));
+        PeerRun* runs = static_cast<PeerRun*>(b->iws);
         SparseWs ws{};
         if (b->reencode) ws = sparse_ws_at(b->ws, b->swl);
         hipError_t e = hipSuccess;
-        if (phase < 0 || phase < 2) e = launch_sparse_merge(L, ws, tileptr, unsorted, phase, st);
+        if (phase < 0 || phase < 2) e = launch_sparse_merge(L, ws, runs, phase, st);
         if (e != hipSuccess) return HIPRESS_ERR_HIP;
         if (b->reencode && (phase < 0 || phase == 2)) {
             Launch R;

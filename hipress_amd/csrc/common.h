@@ -23,6 +23,10 @@ constexpr int kHeaderBytes = 16;
 constexpr int kMaxPeers = 16;
 constexpr int kSampleStride = 100;      // sparse: every 100th element of a large tensor is a sample
 constexpr long long kSampleFrom = 262144;  // sparse: tensors at least this large are sampled
+// sparse: the threshold's 31 key bits are found 12 + 12 + 7 at a time, one histogram each
+constexpr unsigned kSelBins = 4096, kSelBinsLast = 128;
+constexpr unsigned kSelShift0 = 19, kSelShift1 = 7;
+constexpr unsigned kSelHistWords = 2 * kSelBins + kSelBinsLast;  // per tensor
 
 // One tensor (or one chunk) as the kernels see it.  Batched launches index a
 // device-resident array of these through a tile map; single-tensor launches
@@ -60,7 +64,6 @@ struct MergeSeg {
     unsigned int peer_slots[kMaxPeers];  // sparse: pairs each peer's buffer has room for
     Seg s;  // out = aggregate, s0 = aggregator residual (tbq), pay = re-encoded payload
     Seg r;  // sparse re-encode of the aggregate (GradDrop descriptor: s1 = accumulator, pay = out payload)
-    unsigned long long tp0;  // sparse: first tile pointer of this chunk
 };
 
 // where(k) = {tensor index, tile index inside the tensor} of tile k of the launch;

@@ -26,16 +26,31 @@ struct SparseWs {
     uint2* grec;        // per 64-element group (64 per tile): {bits of the acc' value with the largest |.|,
                         //  (upper bound of the second-largest key, multiple of 64) | position of the largest}
     uint32_t* counts;   // per tile {above, equal} counts, then their exclusive scans
-    uint32_t* thr;      // per tensor {threshold key, equal-quota}
-    uint32_t* hist;     // per tensor 3 x 2048 bins, one histogram per select pass
-    uint32_t* ctl;      // per tensor 8 words: select prefix, remaining rank, done counters
+    uint32_t* thr;      // per tensor {threshold key, equal-quota}, written by the scan launch
+    uint32_t* hist;     // per tensor 4096 + 4096 + 128 bins, one histogram per select pass
+    uint32_t* ctl;      // per tensor 8 words: key prefix and remaining rank after the first and the second digit
 };
 hipError_t launch_sparse_encode(const Launch& L, bool dgc, const SparseWs& ws, int phase, hipStream_t st);
 hipError_t launch_sparse_decode(const Launch& L, hipStream_t st);
 hipError_t launch_sparse_decode_indexed(const Launch& L, uint32_t* tptr, uint32_t* disorder, unsigned epoch,
                                         bool few_pairs, hipStream_t st);
 constexpr int kSparseAfterAccum = 100;  // launch_sparse_encode phase: everything after the accumulate launch
-hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, uint32_t* tileptr, uint32_t* unsorted,
-                               int phase, hipStream_t st);
+// Sparse decode-and-merge: what the index launch leaves for the merge launch, records of
+// 32 bytes: the heads of all T tiles of the launch, then every peer's runs for those tiles
+// (record of peer p, tile t at (1 + p) * T + t), kMergeRecs(npeers) * T records in all.
+struct PeerRun {
+    const int32_t* idx;  // first index of the run
+    const float* val;    // first value of the run
+    unsigned cnt;        // pairs in the run
+    unsigned pad[3];     // 32 bytes: one record is two 16-byte loads
+};
+struct TileHead {
+    const float* acc;    // re-encode: the tile's first accumulator element (NULL without re-encode)
+    unsigned fast;       // 1: whole tile, every pointer 16-byte aligned
+    unsigned pad[5];
+};
+static_assert(sizeof(PeerRun) == 32 && sizeof(TileHead) == 32, "merge records are 32 bytes");
+constexpr unsigned kMergeRecs(unsigned npeers) { return npeers + 1; }
+hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, PeerRun* runs, int phase, hipStream_t st);
 
 }  // namespace hp

@@ -8,10 +8,13 @@
 //                   leaves a record on the way: its largest |acc'| with value and
 //                   place, and a bound on its second largest;
 //   1-3. select     the k-th largest sample key of every tensor by radix
-//                   selection, 11 + 10 + 10 bits from the top: every pass is one
-//                   launch over all sample tiles, LDS histograms merged into a
-//                   per-tensor global one, the last workgroup of a tensor to
-//                   finish picks the digit;
+//                   selection, 12 + 12 + 7 bits from the top: every pass is one
+//                   launch over all sample tiles that adds LDS histograms into a
+//                   per-tensor global one; which digit holds the k-th key is
+//                   worked out from the finished histogram by every workgroup of
+//                   the NEXT launch (the last digit by count and scan), so all
+//                   that workgroups hand each other travels across a kernel
+//                   boundary;
 //   4. count        per-tile counts of keys above / equal to the threshold: a
 //                   group whose record shows no or one such key is counted from
 //                   the record, only the others are read again;
@@ -30,7 +33,6 @@ namespace hp {
 
 constexpr unsigned kNoQuota = 0xffffffffu;
 constexpr int kSampleTile = 4096;  // sample keys per workgroup in the select passes
-constexpr int kBins = 2048;        // histogram bins per select pass (11-bit first digit)
 
 __device__ __forceinline__ unsigned key_of(float x) { return __float_as_uint(x) & 0x7fffffffu; }
 
@@ -65,14 +67,10 @@ __device__ __forceinline__ unsigned popc_lt(unsigned long long m, unsigned lane)
     return __popcll(m & ((1ull << lane) - 1ull));
 }
 
-// per-tensor control words of the select passes
-enum { kCtlPrefix = 0, kCtlK = 1, kCtlDone = 2 /* +pass */, kCtlWords = 8 };
-
-__device__ __forceinline__ unsigned digit_shift(int pass) { return pass == 0 ? 20u : (pass == 1 ? 10u : 0u); }
-__device__ __forceinline__ unsigned digit_bins(int pass) { return pass == 0 ? 2048u : 1024u; }
-__device__ __forceinline__ unsigned digit_mask_above(int pass) {
-    return pass == 0 ? 0u : (pass == 1 ? 0x7ff00000u : 0x7ffffc00u);
-}
+// per-tensor control words of the select passes: what the digit picks of passes 1 and 2
+// found, written by the first workgroup of the tensor in that pass and read by the launch
+// after it
+enum { kCtlPrefix1 = 0, kCtlK1 = 1, kCtlPrefix2 = 2, kCtlK2 = 3, kCtlWords = 8 };
 
 // ---- 0. accumulate -------------------------------------------------------------
 
@@ -155,9 +153,9 @@ __device__ __forceinline__ void sparse_accum_tile(const Seg& s, unsigned tile, c
 
 // Tile 0 of a tensor resets that tensor's select-pass state.
 __device__ __forceinline__ void sparse_reset_select(const Seg& s, const SparseWs& ws) {
-    uint32_t* h = ws.hist + (unsigned long long)s.id * (3 * kBins);
-    for (unsigned i = threadIdx.x; i < 3 * kBins; i += kBlock) h[i] = 0;
-    if (threadIdx.x < kCtlWords) ws.ctl[s.id * kCtlWords + threadIdx.x] = threadIdx.x == kCtlK ? s.ks : 0u;
+    uint32_t* h = ws.hist + (unsigned long long)s.id * kSelHistWords;
+    for (unsigned i = threadIdx.x; i < kSelHistWords; i += kBlock) h[i] = 0;
+    if (threadIdx.x < kCtlWords) ws.ctl[s.id * kCtlWords + threadIdx.x] = 0u;
     if (threadIdx.x == 0) {
         ws.thr[2 * s.id] = 0;
         ws.thr[2 * s.id + 1] = kNoQuota;
@@ -180,23 +178,78 @@ __global__ __launch_bounds__(kBlock) void sparse_accum_kernel(Src src, SparseWs 
 
 // ---- 1-3. select -----------------------------------------------------------------
 
-// One radix pass.  Workgroup = one tile of kSampleTile sample keys of one tensor.
-template <class Src>
-__global__ __launch_bounds__(kBlock) void sparse_select_kernel(Src src, SparseWs ws, int pass) {
-    __shared__ unsigned lh[kBins];
-    __shared__ unsigned chunk[kBlock];
-    __shared__ unsigned is_last;
+// Which of 4096 bins holds the k-th largest key (bins walked from the top), and the rank
+// of that key inside the bin: every thread of a 256-thread workgroup gets {bin, rank} in
+// res[] after the call.  Thread t owns the 16 bins [4096 - 16 (t + 1), 4096 - 16 t).  If the
+// counts fall short of k the lowest bin is taken.
+__device__ __forceinline__ void block_pick4096(const uint32_t* gh, unsigned k, unsigned (&xw)[4], unsigned (&res)[2]) {
+    const uint4* p = reinterpret_cast<const uint4*>(gh + kSelBins - 16 * (threadIdx.x + 1));
+    const uint4 q0 = p[0], q1 = p[1], q2 = p[2], q3 = p[3];
+    const unsigned c[16] = {q3.w, q3.z, q3.y, q3.x, q2.w, q2.z, q2.y, q2.x, q1.w, q1.z, q1.y, q1.x, q0.w, q0.z, q0.y, q0.x};
+    unsigned mine = 0;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) mine += c[j];
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const unsigned incl = wave_incl_scan_u(mine);
+    if (lane == 63) xw[wave] = incl;
+    __syncthreads();
+    unsigned before = incl - mine;
+    for (unsigned w = 0; w < wave; ++w) before += xw[w];
+    k = k ? k : 1u;
+    // exactly one thread owns the chunk that holds rank k (the last one takes what is left)
+    const bool owner = (k > before && k <= before + mine) || (threadIdx.x == kBlock - 1 && k > before + mine);
+    if (owner) {
+        unsigned kk = k - before, j = 0;
+#pragma unroll
+        for (int i = 0; i < 15; ++i) {
+            const bool stay = j == (unsigned)i && kk > c[i];  // not in bin i from the top: move on
+            kk -= stay ? c[i] : 0u;
+            j += stay ? 1u : 0u;
+        }
+        res[0] = kSelBins - 1 - 16 * threadIdx.x - j;
+        res[1] = kk;
+    }
+    __syncthreads();
+}
+
+// The last digit (128 bins) by one wavefront, all 64 lanes active: lane l owns bins
+// 127 - 2l and 126 - 2l.  Returns the threshold key, the same value in every lane.
+__device__ __forceinline__ unsigned wave_pick_threshold(const SparseWs& ws, unsigned id, unsigned lane) {
+    const uint2 pk = *reinterpret_cast<const uint2*>(ws.ctl + id * kCtlWords + kCtlPrefix2);
+    const uint2 v = *reinterpret_cast<const uint2*>(ws.hist + (unsigned long long)id * kSelHistWords + 2 * kSelBins + 126 - 2 * lane);
+    const unsigned mine = v.x + v.y;
+    const unsigned incl = wave_incl_scan_u(mine), before = incl - mine;
+    const unsigned k = pk.y ? pk.y : 1u;
+    const bool owner = (k > before && k <= before + mine) || (lane == 63 && k > before + mine);
+    const unsigned d = (k - before) <= v.y ? 127u - 2 * lane : 126u - 2 * lane;
+    const unsigned src = (unsigned)__ffsll((long long)__ballot(owner)) - 1u;
+    return pk.x | (unsigned)__builtin_amdgcn_readlane((int)d, (int)__builtin_amdgcn_readfirstlane((int)src));
+}
+
+// One radix pass.  Workgroup = one tile of kSampleTile sample keys of one tensor.  Pass 0
+// counts the top 12 bits of every key; pass 1 first works out, from pass 0's finished
+// histogram, which of those digits holds the k-th largest key, and counts the next 12 bits
+// of the keys that carry it; pass 2 does the same for the last 7 bits.  Nothing is read
+// that another workgroup of the same launch writes: the adds go to this pass's histogram,
+// which only the next launch reads, and what the first workgroup of a tensor records of
+// its pick (every workgroup of the tensor computes the same) is likewise for the launch
+// after it.
+template <class Src, int PASS>
+__global__ __launch_bounds__(kBlock) void sparse_select_kernel(Src src, SparseWs ws) {
+    constexpr unsigned NB = PASS == 2 ? kSelBinsLast : kSelBins;
+    constexpr unsigned SHIFT = PASS == 0 ? kSelShift0 : (PASS == 1 ? kSelShift1 : 0u);
+    constexpr unsigned ABOVE = PASS == 0 ? 0u : (PASS == 1 ? (0x7fffffffu >> kSelShift0) << kSelShift0
+                                                           : (0x7fffffffu >> kSelShift1) << kSelShift1);
+    __shared__ unsigned lh[NB];
+    __shared__ unsigned xw[4], res[2];
     unsigned stile;
     const Seg s = src.get(stile, blockIdx.x);
     const uint32_t* keys = ws.sample + s.ws0;
     uint32_t* ctl = ws.ctl + s.id * kCtlWords;
-    uint32_t* gh = ws.hist + ((unsigned long long)s.id * 3 + pass) * kBins;
-    const unsigned shift = digit_shift(pass), nb = digit_bins(pass), above = digit_mask_above(pass);
-    const unsigned prefix = pass ? ctl[kCtlPrefix] : 0u;
-    const unsigned k = pass ? ctl[kCtlK] : s.ks;  // read before the barriers; the owner below rewrites it
-    for (unsigned i = threadIdx.x; i < nb; i += kBlock) lh[i] = 0;
-    __syncthreads();
-    // all sixteen keys of a thread are requested before the first one is looked at
+    uint32_t* hist = ws.hist + (unsigned long long)s.id * kSelHistWords;
+    uint32_t* gh = hist + PASS * kSelBins;
+    for (unsigned i = threadIdx.x; i < NB; i += kBlock) lh[i] = 0;
+    // all sixteen keys of a thread are requested before anything else is waited for
     const unsigned long long lo = (unsigned long long)stile * kSampleTile;
     unsigned key[kSampleTile / kBlock];
 #pragma unroll
@@ -204,66 +257,30 @@ __global__ __launch_bounds__(kBlock) void sparse_select_kernel(Src src, SparseWs
         const unsigned long long i = lo + j * kBlock + threadIdx.x;
         key[j] = i < s.ns ? keys[i] : 0u;
     }
-#pragma unroll
-    for (int j = 0; j < kSampleTile / kBlock; ++j) {
-        const unsigned long long i = lo + j * kBlock + threadIdx.x;
-        if (i < s.ns && (key[j] & above) == prefix) atomicAdd(&lh[(key[j] >> shift) & (nb - 1)], 1u);
-    }
-    __syncthreads();
-    unsigned was[kBins / kBlock];  // what the adds return; all are issued before any is waited for
-#pragma unroll
-    for (int q = 0; q < kBins / kBlock; ++q) {
-        const unsigned i = q * kBlock + threadIdx.x;
-        const unsigned c = i < nb ? lh[i] : 0u;
-        was[q] = 0;
-        if (c) was[q] = atomicAdd(&gh[i], c);
-    }
-    unsigned seen = 0;
-#pragma unroll
-    for (int q = 0; q < kBins / kBlock; ++q) seen |= was[q];
-    // Everything workgroups exchange here travels through device-scope atomics
-    // (the histogram adds above, the ticket below, the atomic loads after it), so
-    // no cache write-back is needed.  The ticket may only be taken once this
-    // workgroup's adds have been performed where all XCDs meet.  An add without a
-    // result counts as done when the local L2 has accepted it, which is too early;
-    // one whose result is waited for has been performed, so the results are kept
-    // alive up to the barrier.
-    asm volatile("" ::"v"(seen));
-    __syncthreads();
-    if (threadIdx.x == 0) is_last = atomicAdd(&ctl[kCtlDone + pass], 1u) == s.nsblk - 1;
-    __syncthreads();
-    if (!is_last) return;
-    // Every other workgroup of this tensor has merged its histogram: pick the digit
-    // that holds the k-th largest key, walking the bins from the top.
-    for (unsigned i = threadIdx.x; i < nb; i += kBlock)
-        lh[i] = __hip_atomic_load(&gh[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    const unsigned per = nb / kBlock;  // bins per thread, thread t owns the t-th chunk from the top
-    unsigned mine = 0;
-    for (unsigned b = 0; b < per; ++b) mine += lh[nb - 1 - (threadIdx.x * per + b)];
-    // exclusive prefix of the chunk sums, from the top: wavefront scan, then the
-    // four wavefront totals through LDS
-    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const unsigned incl = wave_incl_scan_u(mine);
-    if (lane == 63) chunk[wave] = incl;
-    __syncthreads();
-    unsigned before = incl - mine;
-    for (unsigned w = 0; w < wave; ++w) before += chunk[w];
-    // exactly one thread owns the chunk that holds rank k (the last thread takes
-    // whatever is left if the counts fall short)
-    const bool owner = (k > before && k <= before + mine) || (threadIdx.x == kBlock - 1 && k > before + mine);
-    if (owner) {
-        unsigned kk = k - before;
-        unsigned d = nb - 1 - threadIdx.x * per;
-        for (unsigned b = 0; b < per - 1; ++b, --d) {
-            unsigned c = lh[d];
-            if (kk <= c) break;
-            kk -= c;
+    unsigned prefix = 0;
+    if (PASS > 0) {
+        const unsigned pprev = PASS == 1 ? 0u : ctl[kCtlPrefix1];
+        const unsigned kprev = PASS == 1 ? s.ks : ctl[kCtlK1];
+        block_pick4096(hist + (PASS - 1) * kSelBins, kprev, xw, res);
+        prefix = pprev | (res[0] << (PASS == 1 ? kSelShift0 : kSelShift1));
+        if (stile == 0 && threadIdx.x == 0) {
+            ctl[PASS == 1 ? kCtlPrefix1 : kCtlPrefix2] = prefix;
+            ctl[PASS == 1 ? kCtlK1 : kCtlK2] = res[1];
         }
-        unsigned np = prefix | (d << shift);
-        ctl[kCtlPrefix] = np;
-        ctl[kCtlK] = kk;
-        if (pass == 2) ws.thr[2 * s.id] = np;
+    } else {
+        __syncthreads();
+    }
+    // Zero keys (and the 0 that stands for a key past the end) are left out: they are the
+    // smallest there is, a pick that runs short of counts takes the lowest bin anyway, and a
+    // sample that is mostly zeros (the sum of sparse payloads) would otherwise send every
+    // lane to the same LDS word.
+#pragma unroll
+    for (int j = 0; j < kSampleTile / kBlock; ++j)
+        if (key[j] != 0u && (key[j] & ABOVE) == prefix) atomicAdd(&lh[(key[j] >> SHIFT) & (NB - 1)], 1u);
+    __syncthreads();
+    for (unsigned i = threadIdx.x; i < NB; i += kBlock) {
+        const unsigned c = lh[i];
+        if (c) atomicAdd(&gh[i], c);  // no result is asked for: the next launch reads the sums
     }
 }
 
@@ -344,11 +361,12 @@ __global__ __launch_bounds__(kBlock) void sparse_count_kernel(Src src, SparseWs 
     const unsigned lane = threadIdx.x & 63u, wave = (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const unsigned gt_idx = blockIdx.x * 4 + wave;
     if (gt_idx >= total_tiles) return;
-    // the record needs nothing but the tile's place in the launch, the threshold only
-    // the tensor's index: neither waits for the descriptor
+    // the record needs nothing but the tile's place in the launch, the threshold (the pick
+    // of the last digit from pass 2's histogram) only the tensor's index: neither waits for
+    // the descriptor
     const uint2 rec = ws.grec[(unsigned long long)gt_idx * 64 + lane];
     const uint2 m = src.where(gt_idx);
-    const unsigned thr = ws.thr[2 * m.x];
+    const unsigned thr = wave_pick_threshold(ws, m.x, lane);
     const Seg s = src.at(m.x);
     unsigned gt, eq;
     count_tile(s, rec, m.y, thr, lane, gt, eq);
@@ -502,7 +520,7 @@ __global__ __launch_bounds__(kScanBlock) void sparse_scan_kernel(SegSrc src, Spa
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const unsigned nw = s.ntiles;
     uint32_t* c = ws.counts + (unsigned long long)s.tile0 * 2;
-    unsigned thr = ws.thr[2 * s.id];
+    unsigned thr = wave_pick_threshold(ws, s.id, lane);  // every wavefront works out the same value
     unsigned quota = kNoQuota;
     unsigned tot_gt, tot_eq;
     block_scan_pairs(c, nw, sh, stage, tot_gt, tot_eq);
@@ -876,12 +894,16 @@ __global__ __launch_bounds__(kBlock) void sparse_decode_tile_kernel(Src src, con
 
 // ---- sparse decode-and-merge -------------------------------------------------------
 // Pairs arrive in ascending index order, so the pairs of one 4096-element tile are
-// one contiguous run of every peer's payload.  A small index kernel finds those
-// runs (and notices a payload that is not sorted); the merge kernel then gives
-// every tile to one workgroup, which adds the peers' runs into an LDS tile in
-// peer order, writes the aggregate once and, if asked, continues with the
-// GradDrop-style re-encode pass on the values it already holds.  Summation order
-// per element is the peer order, as in a sequential implementation.
+// one contiguous run of every peer's payload.  A small index kernel finds those runs
+// and leaves, for every (tile, peer), a record with the addresses of the run's indices
+// and values and its length, at a place that depends on nothing but the tile's number in
+// the launch (the merge launch's grid is the launch's tiles); the merge kernel then gives every tile to one workgroup, which asks for the
+// records before anything else, adds the peers' runs into an LDS tile in peer order,
+// writes the aggregate once and, if asked, continues with the GradDrop-style re-encode
+// pass on the values it already holds.  Summation order per element is the peer order,
+// as in a sequential implementation.  A payload that is not sorted gets its whole length
+// as the run of every tile (the merge kernel drops the pairs that belong elsewhere):
+// correct, slow.
 
 // first position in idx[0, nnz) whose index is >= key
 __device__ __forceinline__ unsigned lower_bound_idx(const int32_t* idx, unsigned nnz, long long key) {
@@ -894,69 +916,125 @@ __device__ __forceinline__ unsigned lower_bound_idx(const int32_t* idx, unsigned
     return lo;
 }
 
-// One workgroup per (chunk, peer): tile pointers ptr[t] = first pair of tile t
-// (ptr[ntiles] = nnz) and a flag that is set when the indices are not ascending.
+// One workgroup per (chunk, peer): run records of that peer for every tile of the chunk.
+// The walk that checks the order of the indices also sees where the tile number changes
+// from one pair to the next, which is where runs begin: for a chunk of up to kIndexTiles
+// tiles those places are collected in LDS in that one pass; a larger chunk finds them by
+// binary search.  Indices outside [0, n) count for the first or the last tile (the merge
+// kernel drops them).
+constexpr unsigned kIndexTiles = 2048;
+
 template <class MSegSrc>
-__global__ __launch_bounds__(kBlock) void sparse_merge_index_kernel(MSegSrc src, uint32_t* tileptr, uint32_t* unsorted,
-                                                                    int npeers) {
+__global__ __launch_bounds__(kBlock) void sparse_merge_index_kernel(MSegSrc src, PeerRun* runs, int npeers,
+                                                                    unsigned total_tiles) {
     __shared__ unsigned bad;
+    __shared__ unsigned bound[kIndexTiles + 1];
     const unsigned chunk = blockIdx.x / npeers, p = blockIdx.x % npeers;
     const MergeSeg& m = src.at(chunk);
     const int32_t* idx;
     const float* val;
     const unsigned nnz = sparse_header(m.peer[p], m.peer_slots[p], idx, val);
     const unsigned nt = m.s.ntiles;
-    uint32_t* ptr = tileptr + m.tp0 + (unsigned long long)p * (nt + 1);
+    // heads of all tiles of the launch first, then the runs peer by peer: what one workgroup
+    // writes here is contiguous
+    PeerRun* out = runs + (unsigned long long)(1 + p) * total_tiles + m.s.tile0;  // record of tile t: out[t]
+    const bool walk = nt <= kIndexTiles;
     if (threadIdx.x == 0) bad = 0;
     __syncthreads();
+    auto tile_of = [&](int32_t i) -> unsigned {
+        if (i < 0) return 0u;
+        const unsigned t = (unsigned)i / kTile;
+        return t < nt ? t : nt - 1;
+    };
     unsigned b = 0;
-    for (unsigned j = threadIdx.x + 1; j < nnz; j += kBlock) b |= idx[j - 1] > idx[j];
+    for (unsigned j = threadIdx.x; j < nnz; j += kBlock) {
+        const int32_t cur = idx[j];
+        unsigned first = 0;
+        if (j) {
+            const int32_t prev = idx[j - 1];
+            b |= prev > cur;
+            first = tile_of(prev) + 1;
+        }
+        if (walk) {
+            const unsigned tc = tile_of(cur);
+            for (unsigned t = first; t <= tc; ++t) bound[t] = j;       // tiles that begin at this pair
+            if (j == nnz - 1)
+                for (unsigned t = tc + 1; t <= nt; ++t) bound[t] = nnz;  // nothing left for the rest
+        }
+    }
+    if (walk && nnz == 0)
+        for (unsigned t = threadIdx.x; t <= nt; t += kBlock) bound[t] = 0;
     if (b) bad = 1;  // benign race: every writer stores 1
-    for (unsigned t = threadIdx.x; t <= nt; t += kBlock) ptr[t] = lower_bound_idx(idx, nnz, (long long)t * kTile);
     __syncthreads();
-    if (threadIdx.x == 0) unsorted[(unsigned long long)chunk * npeers + p] = bad;
+    const bool sorted = bad == 0;
+    for (unsigned t0 = 0; t0 < nt; t0 += kBlock) {
+        const unsigned cnt = nt - t0 < kBlock ? nt - t0 : kBlock;  // tiles of this round
+        if (!walk) {
+            __syncthreads();  // bound[] may still be read from the round before
+            if (sorted)
+                for (unsigned i = threadIdx.x; i <= cnt; i += kBlock) bound[i] = lower_bound_idx(idx, nnz, (long long)(t0 + i) * kTile);
+            __syncthreads();
+        }
+        if (threadIdx.x < cnt) {
+            const unsigned at = walk ? t0 + threadIdx.x : threadIdx.x;
+            const unsigned lo = sorted ? bound[at] : 0u, hi = sorted ? bound[at + 1] : nnz;
+            PeerRun r;
+            r.idx = idx + lo;
+            r.val = val + lo;
+            r.cnt = hi - lo;
+            r.pad[0] = r.pad[1] = r.pad[2] = 0;
+            out[t0 + threadIdx.x] = r;
+            if (p == 0) {  // the tile's head
+                const unsigned t = t0 + threadIdx.x;
+                TileHead h;
+                h.acc = m.r.s1 ? m.r.s1 + (unsigned long long)t * kTile : nullptr;
+                h.fast = m.s.aligned && (!m.r.s1 || m.r.aligned) && (unsigned long long)(t + 1) * kTile <= m.s.n;
+                h.pad[0] = h.pad[1] = h.pad[2] = h.pad[3] = h.pad[4] = 0;
+                *reinterpret_cast<TileHead*>(runs + m.s.tile0 + t) = h;
+            }
+        }
+    }
 }
 
 template <class MSrc, bool REENC>
-__global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs ws, const uint32_t* tileptr,
-                                                              const uint32_t* unsorted, int npeers) {
+__global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs ws, const PeerRun* runs, int npeers) {
     __shared__ __attribute__((aligned(16))) float lds[kTile];
-    __shared__ unsigned plo[kMaxPeers], pcnt[kMaxPeers], pcap[kMaxPeers];
+    __shared__ const int32_t* pidx[kMaxPeers];
+    __shared__ const float* pval[kMaxPeers];
+    __shared__ unsigned pcnt[kMaxPeers];
+    // What this tile needs first lies where the tile's number in the launch says, so it is
+    // asked for before the descriptor: the head (where the accumulator tile starts) and the
+    // peers' runs.  The accumulator tile of the re-encode is requested as soon as the head is
+    // there and is in flight while the peers are merged.
+    const unsigned gtile = xcd_grouped(blockIdx.x, gridDim.x);
+    const TileHead head = *reinterpret_cast<const TileHead*>(runs + gtile);
+    PeerRun run;
+    run.idx = nullptr;
+    run.val = nullptr;
+    run.cnt = 0;
+    if ((int)threadIdx.x < npeers) run = runs[(unsigned long long)(1 + threadIdx.x) * gridDim.x + gtile];
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const bool fast = head.fast != 0;
+    f4 apre[4];
+    if (REENC && fast) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) apre[j] = ld4(head.acc + wave * kWaveTile + j * 256 + lane * 4);
+    }
     unsigned tile;
-    const MergeSeg& m = src.get(tile, xcd_grouped(blockIdx.x, gridDim.x));
+    const MergeSeg& m = src.get(tile, gtile);
     const Seg s = m.s;
     const Seg r = m.r;  // re-encode descriptor of this chunk: same tile numbering
     const long long n = (long long)s.n;
     const long long t_lo = (long long)tile * kTile, t_hi = t_lo + kTile < n ? t_lo + kTile : n;
-    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const bool fast = s.aligned && (!REENC || r.aligned) && (unsigned long long)(tile + 1) * kTile <= s.n;
-    // the accumulator tile of the re-encode is requested first: it is in flight while the peers are merged
-    f4 apre[4];
-    if (REENC) {
+    if (REENC && !fast) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            long long e = t_lo + wave * kWaveTile + j * 256 + lane * 4;
-            apre[j] = fast ? ld4(r.s1 + e) : ld4_guard(r.s1, e, n);
-        }
+        for (int j = 0; j < 4; ++j) apre[j] = ld4_guard(r.s1, t_lo + wave * kWaveTile + j * 256 + lane * 4, n);
     }
     for (unsigned i = threadIdx.x; i < kTile; i += kBlock) lds[i] = 0.f;
-    // one thread per peer: where this tile's pairs are in that peer's payload
     if ((int)threadIdx.x < npeers) {
-        const unsigned p = threadIdx.x;
-        const int32_t* idx;
-        const float* val;
-        const unsigned nnz = sparse_header(m.peer[p], m.peer_slots[p], idx, val);
-        unsigned lo = 0, hi = nnz;
-        if (!unsorted[(unsigned long long)s.id * npeers + p]) {
-            const uint32_t* ptr = tileptr + m.tp0 + (unsigned long long)p * (s.ntiles + 1);
-            lo = ptr[tile];
-            hi = ptr[tile + 1];
-            if (hi > nnz) hi = nnz;
-            if (lo > hi) lo = hi;
-        }
-        plo[p] = lo;
-        pcnt[p] = hi - lo;
-        pcap[p] = reinterpret_cast<const uint32_t*>(m.peer[p])[2];
+        pidx[threadIdx.x] = run.idx;
+        pval[threadIdx.x] = run.val;
+        pcnt[threadIdx.x] = run.cnt;
     }
     __syncthreads();
     unsigned total = 0;
@@ -972,9 +1050,8 @@ __global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs
         long long i = -1;
         float v = 0.f;
         if (have) {
-            const unsigned j = plo[myp] + (f - before);
-            i = reinterpret_cast<const int32_t*>(m.peer[myp] + kHeaderBytes)[j];
-            v = reinterpret_cast<const float*>(m.peer[myp] + kHeaderBytes + 4ull * pcap[myp])[j];
+            i = pidx[myp][f - before];
+            v = pval[myp][f - before];
         }
         const bool inside = have && i >= t_lo && i < t_hi;
         // peers present in this round (uniform): first and last flat entry of the round
@@ -1020,9 +1097,9 @@ static hipError_t sparse_encode_src(const Src& src, const Src& ssrc_tiles, const
         if (dgc) hipLaunchKernelGGL((sparse_accum_kernel<Src, true>), dim3(ntiles), dim3(kBlock), 0, st, src, ws);
         else hipLaunchKernelGGL((sparse_accum_kernel<Src, false>), dim3(ntiles), dim3(kBlock), kLdsFor4, st, src, ws);
     }
-    for (int pass = 0; pass < 3; ++pass)
-        if (on(1 + pass) && nstiles)
-            hipLaunchKernelGGL((sparse_select_kernel<Src>), dim3(nstiles), dim3(kBlock), 0, st, ssrc_tiles, ws, pass);
+    if (on(1) && nstiles) hipLaunchKernelGGL((sparse_select_kernel<Src, 0>), dim3(nstiles), dim3(kBlock), 0, st, ssrc_tiles, ws);
+    if (on(2) && nstiles) hipLaunchKernelGGL((sparse_select_kernel<Src, 1>), dim3(nstiles), dim3(kBlock), 0, st, ssrc_tiles, ws);
+    if (on(3) && nstiles) hipLaunchKernelGGL((sparse_select_kernel<Src, 2>), dim3(nstiles), dim3(kBlock), 0, st, ssrc_tiles, ws);
     if (on(4)) hipLaunchKernelGGL((sparse_count_kernel<Src>), dim3(g4), dim3(kBlock), 0, st, src, ws, ntiles);
     if (on(5)) hipLaunchKernelGGL((sparse_scan_kernel<SegSrcT>), dim3(nsegs), dim3(kScanBlock), 0, st, ssrc, ws);
     if (on(6)) hipLaunchKernelGGL((sparse_emit_kernel<Src>), dim3(g4), dim3(kBlock), 0, st, src, ws, ntiles);
@@ -1085,35 +1162,35 @@ hipError_t launch_sparse_decode_indexed(const Launch& L, uint32_t* tptr, uint32_
 
 // Index kernel (phase 0) + tile-owner merge (phase 1); phase < 0 runs both.  With
 // L.reencode the merge kernel also runs launch 0 of the GradDrop-style re-encode
-// (the caller follows with launch_sparse_encode, kSparseAfterAccum).
-hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, uint32_t* tileptr, uint32_t* unsorted,
-                               int phase, hipStream_t st) {
+// (the caller follows with launch_sparse_encode, kSparseAfterAccum).  runs: one record
+// per (tile of the launch, peer).
+hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, PeerRun* runs, int phase, hipStream_t st) {
     if (L.ntiles == 0) return hipSuccess;
     const bool index = phase < 0 || phase == 0, merge = phase < 0 || phase == 1;
     if (L.single) {
         MergeSingleSegSrc isrc{L.seg};
         if (index)
             hipLaunchKernelGGL((sparse_merge_index_kernel<MergeSingleSegSrc>), dim3(L.npeers), dim3(kBlock), 0, st, isrc,
-                               tileptr, unsorted, L.npeers);
+                               runs, L.npeers, L.ntiles);
         MergeSingleSrc src{L.seg};
         if (merge && L.reencode)
             hipLaunchKernelGGL((sparse_merge_kernel<MergeSingleSrc, true>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
-                               tileptr, unsorted, L.npeers);
+                               runs, L.npeers);
         else if (merge)
             hipLaunchKernelGGL((sparse_merge_kernel<MergeSingleSrc, false>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
-                               tileptr, unsorted, L.npeers);
+                               runs, L.npeers);
     } else {
         MergeBatchSegSrc isrc{L.dsegs};
         if (index)
             hipLaunchKernelGGL((sparse_merge_index_kernel<MergeBatchSegSrc>), dim3(L.nsegs * L.npeers), dim3(kBlock), 0,
-                               st, isrc, tileptr, unsorted, L.npeers);
+                               st, isrc, runs, L.npeers, L.ntiles);
         MergeBatchSrc src{L.dsegs, L.dmap};
         if (merge && L.reencode)
             hipLaunchKernelGGL((sparse_merge_kernel<MergeBatchSrc, true>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
-                               tileptr, unsorted, L.npeers);
+                               runs, L.npeers);
         else if (merge)
             hipLaunchKernelGGL((sparse_merge_kernel<MergeBatchSrc, false>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
-                               tileptr, unsorted, L.npeers);
+                               runs, L.npeers);
     }
     return hipGetLastError();
 }
