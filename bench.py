@@ -544,15 +544,29 @@ def c_level_latency():
         return {"error": str(exc)}
 
 
-def measure(name, steps, warmup, cpu_budget_s=0.0):
+def _warm_up(w, warmup, min_seconds):
+    """At least `warmup` untimed steps, and as many more as it takes to keep the GPU busy for
+    min_seconds: after set-up (or a CPU-baseline leg) the GPU has idled and its clocks take
+    tens of milliseconds of work to come back, which a handful of sub-millisecond steps is not."""
+    import torch
+
+    done, t0 = 0, time.perf_counter()
+    while done < warmup or time.perf_counter() - t0 < min_seconds:
+        for _ in range(max(1, min(warmup, 10))):
+            w.step()
+            done += 1
+        torch.cuda.synchronize()
+    return done
+
+
+def measure(name, steps, warmup, cpu_budget_s=0.0, min_warmup_s=0.25):
     import torch
 
     dev = torch.device("cuda:0")
     graph = name.endswith("_graph")
     w = make_workload(name[: -len("_graph")] if graph else name)
     w.setup(dev)
-    for _ in range(warmup):
-        w.step()
+    warm_steps = _warm_up(w, warmup, min_warmup_s)
     captured = None
     if graph:  # one step captured on a side stream; every later step is one graph launch
         side = torch.cuda.Stream()
@@ -606,6 +620,7 @@ def measure(name, steps, warmup, cpu_budget_s=0.0):
     alg_gbs = (enc_b + dec_b) * w.elements * steps / elapsed / 1e9
     res = {
         "workload": name,
+        "warmup_steps_run": warm_steps,
         "value": gbs,
         "ms_per_step": elapsed / steps * 1e3,
         "median_ms_per_step": median_ms,
@@ -649,6 +664,8 @@ def main():
     ap.add_argument("--others-steps", type=int, default=10)
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="one-thread CPU budget of the headline workload")
     ap.add_argument("--others-cpu-seconds", type=float, default=2.0, help="one-thread CPU budget of every other workload")
+    ap.add_argument("--min-warmup-ms", type=float, default=250.0,
+                    help="keep warming up (beyond --warmup steps) until the GPU has been busy this long")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 1 GiB device-to-device copy (a kernel of known traffic: 1 GiB read, "
                          "1 GiB written) so that rocprofv3 FETCH_SIZE / WRITE_SIZE can be scaled against it")
@@ -674,12 +691,14 @@ def main():
                           "launches": args.steps}))
         return
 
-    main_res = measure(args.workload, args.steps, args.warmup, 0.0 if args.no_cpu else args.cpu_seconds)
+    main_res = measure(args.workload, args.steps, args.warmup, 0.0 if args.no_cpu else args.cpu_seconds,
+                       args.min_warmup_ms * 1e-3)
     others = []
     if not args.no_others:
         for name in ALL_WORKLOADS:
             if name != args.workload:
-                others.append(measure(name, args.others_steps, 3, 0.0 if args.no_cpu else args.others_cpu_seconds))
+                others.append(measure(name, args.others_steps, 3, 0.0 if args.no_cpu else args.others_cpu_seconds,
+                                      args.min_warmup_ms * 1e-3))
     line = {
         "metric": "fp32 grad GB/s through encode+decode",
         "value": main_res["value"],
@@ -687,6 +706,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "warmup_steps_run": main_res["warmup_steps_run"],
         "ms_per_step": main_res["ms_per_step"],
         "median_ms_per_step": main_res["median_ms_per_step"],
         "higher_is_better": True,

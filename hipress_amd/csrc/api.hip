@@ -2,6 +2,7 @@
 // launch objects.  Kernels live in dense.hip, sparse.hip and merge.hip.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <cstring>
@@ -94,6 +95,16 @@ inline SparseWs sparse_ws_at(void* base, const SparseWsLayout& l) {
 inline int64_t merge_index_bytes(int64_t ntiles, int64_t npeers) {
     return round_up((int64_t)sizeof(PeerRun) * ntiles * kMergeRecs((unsigned)npeers), 256);
 }
+
+// Sparse merges stamp records with a number that differs from call to call (0 is never used).
+inline unsigned next_epoch(std::atomic<unsigned>& counter) {
+    unsigned e = counter.fetch_add(1u, std::memory_order_relaxed) + 1u;
+    if (e == 0) e = counter.fetch_add(1u, std::memory_order_relaxed) + 1u;
+    return e;
+}
+std::atomic<unsigned> g_merge_epoch{0};  // per-tensor calls (their workspace belongs to the caller)
+
+inline unsigned slices_of(unsigned slots) { return (unsigned)(((uint64_t)slots + 1023) / 1024); }
 
 inline int hiperr(hipError_t e) { return e == hipSuccess ? HIPRESS_OK : HIPRESS_ERR_HIP; }
 
@@ -342,6 +353,9 @@ struct hipress_merge_batch {
     void* ws = nullptr;
     SparseWsLayout swl{};
     void* iws = nullptr;  // sparse: per tile a head and one run record per peer
+    unsigned slices = 1;  // sparse: the largest peer buffer's slots / 1024, rounded up
+    std::atomic<unsigned> epoch{0};
+    unsigned cur_epoch = 0;
 };
 
 extern "C" {
@@ -750,7 +764,9 @@ int hipress_sparse_decode_merge(const void* const* payloads, const int64_t* payl
     SparseWs ws{};
     if (reenc) ws = sparse_ws_at(wsb + ibytes, l);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipError_t e = launch_sparse_merge(single_merge_launch(m, npeers, reenc), ws, runs, -1, st);
+    unsigned slices = 1;
+    for (int p = 0; p < npeers; ++p) slices = std::max(slices, slices_of(m.peer_slots[p]));
+    hipError_t e = launch_sparse_merge(single_merge_launch(m, npeers, reenc), ws, runs, slices, next_epoch(g_merge_epoch), -1, st);
     if (e != hipSuccess) return HIPRESS_ERR_HIP;
     if (reenc) e = launch_sparse_encode(single_launch(m.r), false, ws, kSparseAfterAccum, st);
     return hiperr(e);
@@ -977,7 +993,11 @@ int hipress_merge_batch_create(hipress_merge_batch** out, int32_t alg, const hip
         for (size_t i = 0; i < b->segs.size(); ++i) b->segs[i].r = b->renc[i];  // the merge kernel runs their first launch
     }
     if (sparse) {
-        if (hipMalloc(&b->iws, (size_t)merge_index_bytes(b->ntiles ? b->ntiles : 1, npeers)) != hipSuccess) return fail(HIPRESS_ERR_HIP);
+        const size_t ibytes = (size_t)merge_index_bytes(b->ntiles ? b->ntiles : 1, npeers);
+        if (hipMalloc(&b->iws, ibytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
+        if (hipMemset(b->iws, 0, ibytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
+        for (const MergeSeg& m : b->segs)
+            for (int p = 0; p < npeers; ++p) b->slices = std::max(b->slices, slices_of(m.peer_slots[p]));
     }
     if ((rc = upload(b->segs, &b->d_segs))) return fail(rc);
     if ((rc = upload(b->renc, &b->d_renc))) return fail(rc);
@@ -1007,7 +1027,9 @@ static int merge_batch_run_impl(hipress_merge_batch* b, int phase, void* stream)
         SparseWs ws{};
         if (b->reencode) ws = sparse_ws_at(b->ws, b->swl);
         hipError_t e = hipSuccess;
-        if (phase < 0 || phase < 2) e = launch_sparse_merge(L, ws, runs, phase, st);
+        // the index and the merge launch of one run share an epoch, also when a caller asks for them one by one
+        if (phase <= 0) b->cur_epoch = next_epoch(b->epoch);
+        if (phase < 0 || phase < 2) e = launch_sparse_merge(L, ws, runs, b->slices, b->cur_epoch, phase, st);
         if (e != hipSuccess) return HIPRESS_ERR_HIP;
         if (b->reencode && (phase < 0 || phase == 2)) {
             Launch R;

@@ -41,8 +41,9 @@ constexpr int kSparseAfterAccum = 100;  // launch_sparse_encode phase: everythin
 struct PeerRun {
     const int32_t* idx;  // first index of the run
     const float* val;    // first value of the run
-    unsigned cnt;        // pairs in the run
-    unsigned pad[3];     // 32 bytes: one record is two 16-byte loads
+    const int32_t* end;  // just behind the run's last index
+    unsigned disorder;   // == the call's epoch: this peer's payload is not in order, ignore the run
+    unsigned pad;        // 32 bytes: one record is two 16-byte loads
 };
 struct TileHead {
     const float* acc;    // re-encode: the tile's first accumulator element (NULL without re-encode)
@@ -51,6 +52,7 @@ struct TileHead {
 };
 static_assert(sizeof(PeerRun) == 32 && sizeof(TileHead) == 32, "merge records are 32 bytes");
 constexpr unsigned kMergeRecs(unsigned npeers) { return npeers + 1; }
-hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, PeerRun* runs, int phase, hipStream_t st);
+hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, PeerRun* runs, unsigned slices, unsigned epoch,
+                               int phase, hipStream_t st);
 
 }  // namespace hp

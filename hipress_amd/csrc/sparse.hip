@@ -894,110 +894,112 @@ __global__ __launch_bounds__(kBlock) void sparse_decode_tile_kernel(Src src, con
 
 // ---- sparse decode-and-merge -------------------------------------------------------
 // Pairs arrive in ascending index order, so the pairs of one 4096-element tile are
-// one contiguous run of every peer's payload.  A small index kernel finds those runs
-// and leaves, for every (tile, peer), a record with the addresses of the run's indices
-// and values and its length, at a place that depends on nothing but the tile's number in
-// the launch (the merge launch's grid is the launch's tiles); the merge kernel then gives every tile to one workgroup, which asks for the
-// records before anything else, adds the peers' runs into an LDS tile in peer order,
-// writes the aggregate once and, if asked, continues with the GradDrop-style re-encode
-// pass on the values it already holds.  Summation order per element is the peer order,
-// as in a sequential implementation.  A payload that is not sorted gets its whole length
-// as the run of every tile (the merge kernel drops the pairs that belong elsewhere):
-// correct, slow.
+// one contiguous run of every peer's payload.  An index launch walks the payloads once,
+// 1024 slots per workgroup: where the tile number changes from one pair to the next a
+// run ends and the next begins, and the workgroup that sees it writes both facts into
+// the run records of the tiles concerned (begin and end of one record may come from
+// different workgroups).  A record holds the addresses of the run's first index and
+// value and the address just behind its last index, at a place that depends on nothing
+// but the tile's number in the launch (the merge launch's grid is the launch's tiles).
+// The merge kernel then gives every tile to one workgroup, which asks for the records
+// before anything else, adds the peers' runs into an LDS tile in peer order, writes the
+// aggregate once and, if asked, continues with the GradDrop-style re-encode pass on the
+// values it already holds.  Summation order per element is the peer order, as in a
+// sequential implementation.
+// A payload that is not in order: the workgroup that notices stamps every record of that
+// (chunk, peer) with the call's epoch, and a merge workgroup that finds the stamp looks
+// through the peer's whole payload instead of a run (correct, slow).  The stamp is never
+// cleared, only compared with the epoch, which differs from call to call: whatever an
+// earlier call or uninitialised memory left there can at worst send a sorted payload
+// down the slow path, never the other way round.
 
-// first position in idx[0, nnz) whose index is >= key
-__device__ __forceinline__ unsigned lower_bound_idx(const int32_t* idx, unsigned nnz, long long key) {
-    unsigned lo = 0, hi = nnz;
-    while (lo < hi) {
-        unsigned mid = (lo + hi) >> 1;
-        if ((long long)idx[mid] < key) lo = mid + 1;
-        else hi = mid;
-    }
-    return lo;
-}
-
-// One workgroup per (chunk, peer): run records of that peer for every tile of the chunk.
-// The walk that checks the order of the indices also sees where the tile number changes
-// from one pair to the next, which is where runs begin: for a chunk of up to kIndexTiles
-// tiles those places are collected in LDS in that one pass; a larger chunk finds them by
-// binary search.  Indices outside [0, n) count for the first or the last tile (the merge
-// kernel drops them).
-constexpr unsigned kIndexTiles = 2048;
-
+// One workgroup per 1024 payload slots of one (chunk, peer); blockIdx.y and .z number the slice.
 template <class MSegSrc>
 __global__ __launch_bounds__(kBlock) void sparse_merge_index_kernel(MSegSrc src, PeerRun* runs, int npeers,
-                                                                    unsigned total_tiles) {
-    __shared__ unsigned bad;
-    __shared__ unsigned bound[kIndexTiles + 1];
-    const unsigned chunk = blockIdx.x / npeers, p = blockIdx.x % npeers;
+                                                                    unsigned total_tiles, unsigned epoch) {
+    __shared__ unsigned gap_first[kSlotTile + 2], gap_count[kSlotTile + 2], gap_value[kSlotTile + 2];
+    __shared__ unsigned ngaps, bad;
+    const unsigned chunk = blockIdx.x / npeers, p = blockIdx.x % npeers, slice = blockIdx.z * gridDim.y + blockIdx.y;
     const MergeSeg& m = src.at(chunk);
     const int32_t* idx;
     const float* val;
     const unsigned nnz = sparse_header(m.peer[p], m.peer_slots[p], idx, val);
     const unsigned nt = m.s.ntiles;
-    // heads of all tiles of the launch first, then the runs peer by peer: what one workgroup
-    // writes here is contiguous
-    PeerRun* out = runs + (unsigned long long)(1 + p) * total_tiles + m.s.tile0;  // record of tile t: out[t]
-    const bool walk = nt <= kIndexTiles;
-    if (threadIdx.x == 0) bad = 0;
+    // heads of all tiles of the launch first, then the runs peer by peer
+    PeerRun* rec = runs + (unsigned long long)(1 + p) * total_tiles + m.s.tile0;  // record of tile t: rec[t]
+    if (slice == 0 && p == 0) {  // the chunk's tile heads
+        for (unsigned t = threadIdx.x; t < nt; t += kBlock) {
+            TileHead h;
+            h.acc = m.r.s1 ? m.r.s1 + (unsigned long long)t * kTile : nullptr;
+            h.fast = m.s.aligned && (!m.r.s1 || m.r.aligned) && (unsigned long long)(t + 1) * kTile <= m.s.n;
+            h.pad[0] = h.pad[1] = h.pad[2] = h.pad[3] = h.pad[4] = 0;
+            *reinterpret_cast<TileHead*>(runs + m.s.tile0 + t) = h;
+        }
+    }
+    const unsigned long long lo = (unsigned long long)slice * kSlotTile;
+    if (lo >= nnz && !(slice == 0 && nnz == 0)) return;  // nothing in this slice
+    if (threadIdx.x == 0) {
+        ngaps = 0;
+        bad = 0;
+    }
     __syncthreads();
-    auto tile_of = [&](int32_t i) -> unsigned {
+    auto tile_of = [&](int32_t i) -> unsigned {  // indices outside the chunk count for the first / last tile
         if (i < 0) return 0u;
         const unsigned t = (unsigned)i / kTile;
         return t < nt ? t : nt - 1;
     };
-    unsigned b = 0;
-    for (unsigned j = threadIdx.x; j < nnz; j += kBlock) {
-        const int32_t cur = idx[j];
-        unsigned first = 0;
-        if (j) {
-            const int32_t prev = idx[j - 1];
-            b |= prev > cur;
-            first = tile_of(prev) + 1;
+    // tiles t0 .. t1-1 begin at slot v, and the tiles before them end there
+    auto mark = [&](unsigned t, unsigned v) {
+        rec[t].idx = idx + v;
+        rec[t].val = val + v;
+        if (t) rec[t - 1].end = idx + v;
+    };
+    auto start = [&](unsigned t0, unsigned t1, unsigned v) {
+        if (t1 - t0 <= 8u) {
+            for (unsigned t = t0; t < t1; ++t) mark(t, v);
+        } else {  // a long stretch of empty tiles: left to the whole workgroup
+            const unsigned g = atomicAdd(&ngaps, 1u);
+            gap_first[g] = t0;
+            gap_count[g] = t1 - t0;
+            gap_value[g] = v;
         }
-        if (walk) {
+    };
+    bool disorder = false;
+#pragma unroll
+    for (int k = 0; k < kSlotTile / kBlock; ++k) {
+        const unsigned long long j = lo + k * kBlock + threadIdx.x;
+        if (j < nnz) {
+            const int32_t cur = idx[j];
             const unsigned tc = tile_of(cur);
-            for (unsigned t = first; t <= tc; ++t) bound[t] = j;       // tiles that begin at this pair
-            if (j == nnz - 1)
-                for (unsigned t = tc + 1; t <= nt; ++t) bound[t] = nnz;  // nothing left for the rest
-        }
-    }
-    if (walk && nnz == 0)
-        for (unsigned t = threadIdx.x; t <= nt; t += kBlock) bound[t] = 0;
-    if (b) bad = 1;  // benign race: every writer stores 1
-    __syncthreads();
-    const bool sorted = bad == 0;
-    for (unsigned t0 = 0; t0 < nt; t0 += kBlock) {
-        const unsigned cnt = nt - t0 < kBlock ? nt - t0 : kBlock;  // tiles of this round
-        if (!walk) {
-            __syncthreads();  // bound[] may still be read from the round before
-            if (sorted)
-                for (unsigned i = threadIdx.x; i <= cnt; i += kBlock) bound[i] = lower_bound_idx(idx, nnz, (long long)(t0 + i) * kTile);
-            __syncthreads();
-        }
-        if (threadIdx.x < cnt) {
-            const unsigned at = walk ? t0 + threadIdx.x : threadIdx.x;
-            const unsigned lo = sorted ? bound[at] : 0u, hi = sorted ? bound[at + 1] : nnz;
-            PeerRun r;
-            r.idx = idx + lo;
-            r.val = val + lo;
-            r.cnt = hi - lo;
-            r.pad[0] = r.pad[1] = r.pad[2] = 0;
-            out[t0 + threadIdx.x] = r;
-            if (p == 0) {  // the tile's head
-                const unsigned t = t0 + threadIdx.x;
-                TileHead h;
-                h.acc = m.r.s1 ? m.r.s1 + (unsigned long long)t * kTile : nullptr;
-                h.fast = m.s.aligned && (!m.r.s1 || m.r.aligned) && (unsigned long long)(t + 1) * kTile <= m.s.n;
-                h.pad[0] = h.pad[1] = h.pad[2] = h.pad[3] = h.pad[4] = 0;
-                *reinterpret_cast<TileHead*>(runs + m.s.tile0 + t) = h;
+            unsigned first = 0;
+            if (j) {
+                const int32_t prev = idx[j - 1];
+                disorder |= prev > cur;
+                first = tile_of(prev) + 1;
+            }
+            if (tc + 1 > first) start(first, tc + 1, (unsigned)j);
+            if (j == nnz - 1) {  // nothing is left for the tiles behind this pair's
+                if (tc + 1 < nt) start(tc + 1, nt, nnz);
+                rec[nt - 1].end = idx + nnz;
             }
         }
     }
+    if (slice == 0 && nnz == 0 && threadIdx.x == 0) {
+        start(0, nt, 0u);
+        rec[nt - 1].end = idx;
+    }
+    if (disorder) bad = 1;  // every writer stores 1
+    __syncthreads();
+    const unsigned ng = ngaps;
+    for (unsigned g = 0; g < ng; ++g)
+        for (unsigned t = threadIdx.x; t < gap_count[g]; t += kBlock) mark(gap_first[g] + t, gap_value[g]);
+    if (bad)
+        for (unsigned t = threadIdx.x; t < nt; t += kBlock) rec[t].disorder = epoch;
 }
 
 template <class MSrc, bool REENC>
-__global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs ws, const PeerRun* runs, int npeers) {
+__global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs ws, const PeerRun* runs, int npeers,
+                                                              unsigned epoch) {
     __shared__ __attribute__((aligned(16))) float lds[kTile];
     __shared__ const int32_t* pidx[kMaxPeers];
     __shared__ const float* pval[kMaxPeers];
@@ -1009,9 +1011,9 @@ __global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs
     const unsigned gtile = xcd_grouped(blockIdx.x, gridDim.x);
     const TileHead head = *reinterpret_cast<const TileHead*>(runs + gtile);
     PeerRun run;
-    run.idx = nullptr;
+    run.idx = run.end = nullptr;
     run.val = nullptr;
-    run.cnt = 0;
+    run.disorder = epoch + 1u;
     if ((int)threadIdx.x < npeers) run = runs[(unsigned long long)(1 + threadIdx.x) * gridDim.x + gtile];
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const bool fast = head.fast != 0;
@@ -1032,9 +1034,13 @@ __global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs
     }
     for (unsigned i = threadIdx.x; i < kTile; i += kBlock) lds[i] = 0.f;
     if ((int)threadIdx.x < npeers) {
+        if (run.disorder == epoch) {  // this peer's payload was seen out of order: every pair is looked at
+            const unsigned nnz = sparse_header(m.peer[threadIdx.x], m.peer_slots[threadIdx.x], run.idx, run.val);
+            run.end = run.idx + nnz;
+        }
         pidx[threadIdx.x] = run.idx;
         pval[threadIdx.x] = run.val;
-        pcnt[threadIdx.x] = run.cnt;
+        pcnt[threadIdx.x] = run.end > run.idx ? (unsigned)(run.end - run.idx) : 0u;
     }
     __syncthreads();
     unsigned total = 0;
@@ -1160,37 +1166,41 @@ hipError_t launch_sparse_decode_indexed(const Launch& L, uint32_t* tptr, uint32_
     return hipGetLastError();
 }
 
-// Index kernel (phase 0) + tile-owner merge (phase 1); phase < 0 runs both.  With
+// Index launch (phase 0) + tile-owner merge (phase 1); phase < 0 runs both.  With
 // L.reencode the merge kernel also runs launch 0 of the GradDrop-style re-encode
-// (the caller follows with launch_sparse_encode, kSparseAfterAccum).  runs: one record
-// per (tile of the launch, peer).
-hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, PeerRun* runs, int phase, hipStream_t st) {
+// (the caller follows with launch_sparse_encode, kSparseAfterAccum).  runs: records as
+// described at PeerRun; slices: the largest peer buffer's slots / 1024, rounded up; epoch:
+// a number no earlier call on these records used.
+hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, PeerRun* runs, unsigned slices, unsigned epoch,
+                               int phase, hipStream_t st) {
     if (L.ntiles == 0) return hipSuccess;
     const bool index = phase < 0 || phase == 0, merge = phase < 0 || phase == 1;
+    if (slices == 0) slices = 1;
+    const unsigned sy = slices < 65535u ? slices : 65535u, sz = (slices + sy - 1) / sy;  // a grid dimension ends at 65535
     if (L.single) {
         MergeSingleSegSrc isrc{L.seg};
         if (index)
-            hipLaunchKernelGGL((sparse_merge_index_kernel<MergeSingleSegSrc>), dim3(L.npeers), dim3(kBlock), 0, st, isrc,
-                               runs, L.npeers, L.ntiles);
+            hipLaunchKernelGGL((sparse_merge_index_kernel<MergeSingleSegSrc>), dim3(L.npeers, sy, sz), dim3(kBlock), 0, st,
+                               isrc, runs, L.npeers, L.ntiles, epoch);
         MergeSingleSrc src{L.seg};
         if (merge && L.reencode)
             hipLaunchKernelGGL((sparse_merge_kernel<MergeSingleSrc, true>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
-                               runs, L.npeers);
+                               runs, L.npeers, epoch);
         else if (merge)
             hipLaunchKernelGGL((sparse_merge_kernel<MergeSingleSrc, false>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
-                               runs, L.npeers);
+                               runs, L.npeers, epoch);
     } else {
         MergeBatchSegSrc isrc{L.dsegs};
         if (index)
-            hipLaunchKernelGGL((sparse_merge_index_kernel<MergeBatchSegSrc>), dim3(L.nsegs * L.npeers), dim3(kBlock), 0,
-                               st, isrc, runs, L.npeers, L.ntiles);
+            hipLaunchKernelGGL((sparse_merge_index_kernel<MergeBatchSegSrc>), dim3(L.nsegs * L.npeers, sy, sz), dim3(kBlock),
+                               0, st, isrc, runs, L.npeers, L.ntiles, epoch);
         MergeBatchSrc src{L.dsegs, L.dmap};
         if (merge && L.reencode)
             hipLaunchKernelGGL((sparse_merge_kernel<MergeBatchSrc, true>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
-                               runs, L.npeers);
+                               runs, L.npeers, epoch);
         else if (merge)
             hipLaunchKernelGGL((sparse_merge_kernel<MergeBatchSrc, false>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
-                               runs, L.npeers);
+                               runs, L.npeers, epoch);
     }
     return hipGetLastError();
 }

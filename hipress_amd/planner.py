@@ -11,10 +11,27 @@ kernels on the GPU at hand.
 
     python -m hipress_amd.planner --input input.txt --output SeCoPaPlan.txt --topology PS --nnodes 4
     python -m hipress_amd.planner --calibrate tbq ...     # encode/decode/merge models measured on cuda:0
+    python -m hipress_amd.planner --measured tbq ...      # the models measured on MI355X that ship with the package
+    python -m hipress_amd.planner --calibrate-all out.json   # measure every algorithm, write such a file
+
+Units.  The reference states no unit for its coefficients and no hardware
+(SeCoPa.py:25-39; README.md:14 "measured in our local cluster").  Its encode model gives
+0.054 for a small tensor and its 4-node gather 0.42 + 2.7e-6 per element: read as
+milliseconds these are a 54 us kernel sequence and about 1.5 GB/s per peer, read as
+seconds they would be a 54 ms encode of a few kilobytes, so milliseconds is the reading
+taken here, and the models measured by `calibrate` are in milliseconds so that they can
+stand beside the reference's gather / broadcast / ring-send models, which one GPU cannot
+measure and which therefore stay the reference's.
 """
 import argparse
 import json
+import os
 from dataclasses import dataclass, field
+
+MEASURED_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "models_mi355x.json")
+# bytes on the wire per fp32 byte of gradient: 1 or 2 bits per element (+ one scale per 512
+# for terngrad), 8-byte pairs for the kept fraction of the sparsifiers
+COMP_RATIO = {"onebit": 1 / 32, "tbq": 1 / 16, "terngrad": 1 / 16 + 1 / 512, "dgc": 2 * 0.001, "graddrop": 2 * 0.01}
 
 
 @dataclass(frozen=True)
@@ -63,6 +80,23 @@ class Planner:
     # partition size, for nodes - 1 peers) the PS cost counts it once in place of the
     # reference's nodes - 1 decodes, nodes - 1 aggregations and one encode at the server.
     merge: CostModel = field(default=None)
+
+    @classmethod
+    def from_measured(cls, alg, nodes, path=None, **kw):
+        """Planner with the encode / decode / merge models of `alg` measured on MI355X
+        (hipress_amd/models_mi355x.json, written by `--calibrate-all`); the merge model is the
+        one measured for nodes - 1 peers when there is one.  Communication models stay the
+        reference's."""
+        with open(path or MEASURED_PATH) as f:
+            data = json.load(f)
+        model = lambda d: CostModel(d["weight"], d["bias"], d["overhead"])
+        args = {"encode": model(data["encode"][alg]), "decode": model(data["decode"][alg]),
+                "comp_ratio": data["comp_ratio"][alg]}
+        merge = data.get("merge", {}).get(alg, {}).get(str(nodes - 1))
+        if merge is not None:
+            args["merge"] = model(merge)
+        args.update(kw)
+        return cls(nodes=nodes, **args)
 
     def __post_init__(self):
         if self.gather is None or self.broadcast is None:
@@ -164,7 +198,7 @@ def calibrate(alg="tbq", sizes=None, reps=20, comp_ratio=None):
     import hipress_amd as hp
 
     sizes = sizes or [1 << k for k in range(10, 28, 2)]
-    ratio = comp_ratio if comp_ratio is not None else {"onebit": 1 / 32}.get(alg, 1 / 16)
+    ratio = comp_ratio if comp_ratio is not None else COMP_RATIO[alg]
     enc_t, dec_t = [], []
     for n in sizes:
         g = torch.randn(n, device="cuda") * 1e-2
@@ -237,8 +271,38 @@ def calibrate_merge(alg="tbq", npeers=3, sizes=None, reps=20):
     return {"alg": alg, "npeers": npeers, "unit": "ms", "sizes": sizes, "merge_ms": times, "merge": fit_cost_model(sizes, times)}
 
 
+def calibrate_all(reps=20, sizes=None):
+    """Every model the planner can take from this library, measured on cuda:0: encode and
+    decode of the five compressors, the fused decode-and-merge of tbq / dgc / graddrop for
+    3, 7 and 15 peers (4, 8 and 16 nodes).  Returns the dictionary `from_measured` reads."""
+    import torch
+
+    as_dict = lambda m: {"weight": m.weight, "bias": m.bias, "overhead": m.overhead}
+    props = torch.cuda.get_device_properties(0)
+    out = {"device": f"{getattr(props, 'gcnArchName', '?').split(':')[0]} ({torch.cuda.get_device_name(0)})", "unit": "ms",
+           "note": "t(x) = overhead below the break-even size, weight * x + bias above it; encode and merge take "
+                   "fp32 elements, decode takes elements * comp_ratio",
+           "encode": {}, "decode": {}, "comp_ratio": {}, "merge": {}, "raw": {}}
+    for alg in ("onebit", "tbq", "terngrad", "dgc", "graddrop"):
+        cal = calibrate(alg, sizes=sizes, reps=reps)
+        out["encode"][alg], out["decode"][alg] = as_dict(cal["encode"]), as_dict(cal["decode"])
+        out["comp_ratio"][alg] = cal["comp_ratio"]
+        out["raw"][alg] = {"sizes": cal["sizes"], "encode_ms": cal["encode_ms"], "decode_ms": cal["decode_ms"]}
+    for alg in ("tbq", "dgc", "graddrop"):
+        out["merge"][alg] = {}
+        for npeers in (3, 7, 15):
+            mer = calibrate_merge(alg, npeers=npeers, sizes=sizes, reps=reps)
+            out["merge"][alg][str(npeers)] = as_dict(mer["merge"])
+            out["raw"][f"merge_{alg}_{npeers}"] = {"sizes": mer["sizes"], "merge_ms": mer["merge_ms"]}
+    return out
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description="SeCoPa: selective compression and partitioning plan")
+    ap.add_argument("--measured", metavar="ALG", default=None,
+                    help="plan with the models of ALG measured on MI355X that ship with the package")
+    ap.add_argument("--calibrate-all", metavar="JSON", default=None,
+                    help="measure every algorithm's models on cuda:0 and write them to JSON (no plan is made)")
     ap.add_argument("--input", default="input.txt", help="lines of name,size (fp32 elements)")
     ap.add_argument("--output", default="SeCoPaPlan.txt")
     ap.add_argument("--topology", default="PS", choices=["PS", "RING"])
@@ -247,7 +311,17 @@ def main(argv=None):
                     help="measure ALG's encode/decode on cuda:0 and plan with the fitted models "
                          "(communication models stay the reference's)")
     args = ap.parse_args(argv)
+    if args.calibrate_all:
+        with open(args.calibrate_all, "w") as f:
+            json.dump(calibrate_all(), f, indent=1)
+        return
     kw = {}
+    if args.measured:
+        planner = Planner.from_measured(args.measured, args.nnodes)
+        with open(args.output, "w") as f:
+            for line in planner.plan(read_gradients(args.input), args.topology):
+                f.write(line + "\n")
+        return
     if args.calibrate:
         cal = calibrate(args.calibrate)
         kw = {"encode": cal["encode"], "decode": cal["decode"], "comp_ratio": cal["comp_ratio"]}

@@ -578,3 +578,56 @@ def test_batches_accept_empty_tensors_among_others(hp):
             check_sparse(host(ts[1]["compressed"]), oracle.graddrop_encode(g, z, 0.01)[0])
             assert oracle.sparse_unpack(host(ts[2]["compressed"]))[0] == 0
         b.close()
+
+
+# ================================================================ large single chunks
+def test_sparse_merge_of_one_large_chunk(hp):
+    """One chunk of 20 M elements at one per cent: 4883 tiles and ~200 K pairs per peer, so the
+    index launch spreads every peer's payload over some 200 workgroups and the two ends of a
+    run record often come from different ones.  Then the same call with one peer's pairs out of
+    order (the slow path), and once more with the sorted payloads on the same workspace."""
+    n, P, ratio = 20_000_003, 4, 0.01
+    rng = np.random.default_rng(9)
+    z = np.zeros(n, F)
+    pays = [oracle.graddrop_encode(rng.normal(0, 1e-3, n).astype(F), z, ratio)[0] for _ in range(P)]
+    acc0 = rng.normal(0, 1e-4, n).astype(F)
+    want_agg, want_out, want_acc = oracle.sparse_decode_merge(pays, n, acc0, ratio)
+
+    def run(payloads):
+        agg, acc = torch.full((n,), 7.0, device="cuda"), dev(acc0)
+        outp = payload(hp.sparse_payload_bytes(n, ratio))
+        hp.dgc_decode_merge([dev(p) for p in payloads], agg, acc, outp, ratio)
+        np.testing.assert_array_equal(host(agg), want_agg)
+        check_sparse(host(outp), want_out)
+        np.testing.assert_array_equal(host(acc), want_acc)
+
+    run(pays)
+    # peer 2 with two far-apart pairs swapped: same content, not in order
+    nnz, _, cap, _, idx, val = oracle.sparse_unpack(pays[2])
+    shuffled = pays[2].copy()
+    i32, f32 = shuffled[16:16 + 4 * cap].view(np.int32), shuffled[16 + 4 * cap:16 + 8 * cap].view(F)
+    a, b = 1000, nnz - 2000
+    i32[a], i32[b] = idx[b], idx[a]
+    f32[a], f32[b] = val[b], val[a]
+    run([pays[0], pays[1], shuffled, pays[3]])
+    run(pays)
+
+
+def test_sparse_merge_with_few_pairs_in_many_tiles(hp):
+    """Long stretches of tiles without a pair (the index launch fills them workgroup-wide), a
+    peer with no pair at all, and pairs in the first and the last tile only."""
+    n, ratio = 4096 * 3000 + 17, 0.001
+    cap = hp.sparse_capacity(n, ratio)
+
+    def handmade(idx, val):
+        p = np.zeros(16 + 8 * cap, np.uint8)
+        p[:16].view(np.uint32)[:3] = [len(idx), n, cap]
+        p[16:16 + 4 * len(idx)].view(np.int32)[:] = idx
+        p[16 + 4 * cap:16 + 4 * cap + 4 * len(val)].view(F)[:] = val
+        return p
+
+    pays = [handmade([0, 5, n - 1], [1.0, 2.0, 3.0]), handmade([], []), handmade([4096 * 1500 + 7], [4.0]),
+            handmade([5, 4096 * 1500 + 7, n - 1], [0.5, 0.25, 0.125])]
+    agg = torch.full((n,), 7.0, device="cuda")
+    hp.dgc_decode_merge([dev(p) for p in pays], agg)
+    np.testing.assert_array_equal(host(agg), oracle.sparse_decode_merge(pays, n))

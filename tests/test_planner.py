@@ -102,3 +102,72 @@ def test_fused_merge_model_replaces_the_server_side_terms():
     assert fused.compressed_costs(size)[0] == pytest.approx(1 * 2e-9 * size + 1 * 1e-9 * size * r + 5e-10 * size)
     # the ring formula has no server and is unchanged
     assert fused.compressed_costs(size, "RING") == base.compressed_costs(size, "RING")
+
+
+# ---------------------------------------------------------------- measured models
+def test_measured_models_ship_with_the_package():
+    """hipress_amd/models_mi355x.json (written by `planner --calibrate-all` on an MI355X)
+    holds encode / decode models for the five compressors and merge models for 3, 7 and 15
+    peers; every model has a positive floor and slope, in milliseconds."""
+    import json
+
+    with open(P.MEASURED_PATH) as f:
+        data = json.load(f)
+    assert data["unit"] == "ms" and "gfx950" in data["device"]
+    for alg in ("onebit", "tbq", "terngrad", "dgc", "graddrop"):
+        for kind in ("encode", "decode"):
+            m = data[kind][alg]
+            assert m["overhead"] > 0 and m["weight"] > 0, (alg, kind)
+            assert m["overhead"] < 0.1  # a launch sequence takes microseconds, not tenths of a second
+        assert data["comp_ratio"][alg] == pytest.approx(P.COMP_RATIO[alg])
+    for alg in ("tbq", "dgc", "graddrop"):
+        for peers in ("3", "7", "15"):
+            m = data["merge"][alg][peers]
+            assert m["overhead"] > 0 and m["weight"] > 0
+
+
+def test_plan_from_the_measured_models_is_the_committed_one(tmp_path):
+    grads = P.read_gradients(os.path.join(GOLDEN, "secopa_input.txt"))
+    want = [l.strip() for l in open(os.path.join(GOLDEN, "plan_vgg19_tbq_ps4_mi355x.txt")) if l.strip()]
+    pl = P.Planner.from_measured("tbq", 4)
+    assert pl.merge is not None and pl.comp_ratio == 1 / 16
+    assert pl.plan(grads, "PS") == want
+    # with kernels this fast every weight tensor from 36,864 elements up is worth compressing on
+    # 4 nodes; the reference's coefficients put the first one at 1,179,648 (its shipped plan)
+    first = next(l for l in want if ",y," in l)
+    assert first.startswith("vgg0_conv1_weight,36864,")
+    out = tmp_path / "plan.txt"
+    P.main(["--input", os.path.join(GOLDEN, "secopa_input.txt"), "--output", str(out), "--topology", "PS",
+            "--nnodes", "4", "--measured", "tbq"])
+    assert out.read_text().splitlines() == want
+
+
+def test_fit_recovers_a_known_model():
+    true = P.CostModel(2e-9, 1e-3, 4e-3)
+    sizes = [1 << k for k in range(10, 28, 2)]
+    fit = P.fit_cost_model(sizes, [true.cost(x) for x in sizes])
+    assert fit.overhead == pytest.approx(4e-3)
+    assert fit.weight == pytest.approx(2e-9, rel=1e-6) and fit.bias == pytest.approx(1e-3, rel=1e-3)
+
+
+@pytest.mark.gpu
+def test_calibration_on_this_gpu_agrees_with_the_committed_models():
+    """Three sizes of TBQ measured on cuda:0: a positive floor, a slope within a factor of two
+    of the committed one, and the same VGG19 plan as the committed models give."""
+    import json
+
+    with open(P.MEASURED_PATH) as f:
+        data = json.load(f)
+    cal = P.calibrate("tbq", sizes=[2 ** 10, 2 ** 20, 2 ** 24], reps=10)
+    for kind in ("encode", "decode"):
+        got, want = cal[kind], data[kind]["tbq"]
+        assert got.overhead > 0
+        assert 0.5 * want["weight"] <= got.weight <= 2.0 * want["weight"], (kind, got, want)
+    ref = P.Planner.from_measured("tbq", 4)
+    pl = P.Planner(nodes=4, encode=cal["encode"], decode=cal["decode"], comp_ratio=cal["comp_ratio"], merge=ref.merge)
+    grads = P.read_gradients(os.path.join(GOLDEN, "secopa_input.txt"))
+    want = [l.strip() for l in open(os.path.join(GOLDEN, "plan_vgg19_tbq_ps4_mi355x.txt")) if l.strip()]
+    assert pl.plan(grads, "PS") == want
+    mer = P.calibrate_merge("dgc", npeers=3, sizes=[2 ** 12, 2 ** 20, 2 ** 24], reps=5)
+    assert mer["merge"].overhead > 0
+    assert 0.5 * data["merge"]["dgc"]["3"]["weight"] <= mer["merge"].weight <= 2.0 * data["merge"]["dgc"]["3"]["weight"]
