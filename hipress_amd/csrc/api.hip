@@ -360,7 +360,7 @@ struct hipress_merge_batch {
 
 extern "C" {
 
-int hipress_version(void) { return 100; }
+int hipress_version(void) { return 110; }
 
 const char* hipress_strerror(int code) {
     switch (code) {

@@ -199,7 +199,10 @@ int hipress_terngrad_decode_merge(const void *const *payloads, const int64_t *pa
 /* Sparse payloads must hold their pairs in ascending index order (the encoders
  * here write them so); a payload that does not is still merged correctly, but
  * slowly.  workspace: hipress_sparse_merge_workspace_bytes(n, npeers, ratio,
- * accumulator != NULL). */
+ * accumulator != NULL); it needs no initialisation.  Every call stamps what it
+ * finds out of order with a number of its own (a process-wide counter), which a
+ * HIP graph freezes: in replays a peer whose payload was once out of order keeps
+ * taking the slow path (results stay correct). */
 int hipress_sparse_decode_merge(const void *const *payloads, const int64_t *payload_bytes,
                                 int32_t npeers, float *aggregate, int64_t n, float *accumulator,
                                 void *out_payload, int64_t out_payload_bytes, double ratio,
