@@ -343,6 +343,7 @@ struct hipress_merge_batch {
     hipress_params params{};
     int npeers = 0;
     bool reencode = false;
+    bool aggregate = false;  // some chunk writes its fp32 sum
     std::vector<MergeSeg> segs;
     std::vector<Seg> renc;  // sparse re-encode descriptors
     MergeSeg* d_segs = nullptr;
@@ -681,6 +682,7 @@ static MergeLaunch single_merge_launch(const MergeSeg& m, int npeers, bool reenc
     L.nsegs = 1;
     L.npeers = npeers;
     L.reencode = reencode;
+    L.aggregate = m.s.out != nullptr;
     return L;
 }
 
@@ -976,6 +978,7 @@ int hipress_merge_batch_create(hipress_merge_batch** out, int32_t alg, const hip
             if ((rc = build_encode_seg(HIPRESS_GRADDROP, t, *params, &s))) return fail(rc);
             b->renc.push_back(s);
         }
+        b->aggregate = b->aggregate || m.s.out != nullptr;
         b->segs.push_back(m);
     }
     std::vector<uint2> map;
@@ -1021,6 +1024,7 @@ static int merge_batch_run_impl(hipress_merge_batch* b, int phase, void* stream)
     L.nsegs = (unsigned)b->segs.size();
     L.npeers = b->npeers;
     L.reencode = b->reencode;
+    L.aggregate = b->aggregate;
     if (b->alg == HIPRESS_DGC || b->alg == HIPRESS_GRADDROP) {
         if (phase > 2) return HIPRESS_ERR_PARAM;
         PeerRun* runs = static_cast<PeerRun*>(b->iws);

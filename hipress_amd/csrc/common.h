@@ -277,6 +277,7 @@ struct MergeLaunch {
     unsigned nsegs;
     int npeers;
     bool reencode;
+    bool aggregate;  // some chunk of the launch writes its fp32 sum
 };
 
 }  // namespace hp

@@ -1177,6 +1177,12 @@ hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, PeerRun
     const bool index = phase < 0 || phase == 0, merge = phase < 0 || phase == 1;
     if (slices == 0) slices = 1;
     const unsigned sy = slices < 65535u ? slices : 65535u, sz = (slices + sy - 1) / sy;  // a grid dimension ends at 65535
+    // A merge that reads the accumulator and writes it and the aggregate (one read, two write
+    // streams) moves 3-6 % more bytes with four workgroups per CU than with the seven its own
+    // LDS tile allows (measured on MI355X on the VGG19 chunks and on 400 chunks of 1 Mi, with the
+    // buffers allocated chunk by chunk and kind by kind); without the aggregate (one read, one
+    // write stream) it is 10 % slower capped, so only the former is.
+    const unsigned cap = L.aggregate ? 16u * 1024u : 0u;
     if (L.single) {
         MergeSingleSegSrc isrc{L.seg};
         if (index)
@@ -1184,7 +1190,7 @@ hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, PeerRun
                                isrc, runs, L.npeers, L.ntiles, epoch);
         MergeSingleSrc src{L.seg};
         if (merge && L.reencode)
-            hipLaunchKernelGGL((sparse_merge_kernel<MergeSingleSrc, true>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
+            hipLaunchKernelGGL((sparse_merge_kernel<MergeSingleSrc, true>), dim3(L.ntiles), dim3(kBlock), cap, st, src, ws,
                                runs, L.npeers, epoch);
         else if (merge)
             hipLaunchKernelGGL((sparse_merge_kernel<MergeSingleSrc, false>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
@@ -1196,7 +1202,7 @@ hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, PeerRun
                                0, st, isrc, runs, L.npeers, L.ntiles, epoch);
         MergeBatchSrc src{L.dsegs, L.dmap};
         if (merge && L.reencode)
-            hipLaunchKernelGGL((sparse_merge_kernel<MergeBatchSrc, true>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
+            hipLaunchKernelGGL((sparse_merge_kernel<MergeBatchSrc, true>), dim3(L.ntiles), dim3(kBlock), cap, st, src, ws,
                                runs, L.npeers, epoch);
         else if (merge)
             hipLaunchKernelGGL((sparse_merge_kernel<MergeBatchSrc, false>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
