@@ -71,8 +71,9 @@ struct MergeSeg {
 // tiles tile0 .. tile0 + ntiles - 1, so k = tile0 + tile index.
 struct SingleSrc {
     Seg seg;
+    unsigned base;  // first tile of this launch when a tensor's tiles are spread over several launches
     __device__ __forceinline__ const Seg& get(unsigned& tile, unsigned blk) const {
-        tile = blk;
+        tile = blk + base;
         return seg;
     }
     __device__ __forceinline__ uint2 where(unsigned blk) const { return make_uint2(0u, blk); }

@@ -32,7 +32,10 @@ def test_traffic_is_read_from_the_committed_profile(name):
     fetch_kib, write_kib = float(cells[3]), float(cells[4])
     assert abs(traffic - (2.0 * fetch_kib + write_kib) * 1024) <= 2048
     # and no more than a third above what the kernel must move
-    algorithmic = w.dominant_bytes * w.elements
+    launches = 1  # a very long accumulate pass is issued in equal parts; the table holds bytes per dispatch
+    if w.dominant_kernel == "sparse_accum_kernel":
+        launches = -(-sum(-(-n // 4096) for n in w.sizes) // 49152)
+    algorithmic = w.dominant_bytes * w.elements / launches
     assert 0.9 * algorithmic <= traffic <= 1.35 * algorithmic, (traffic, algorithmic)
 
 
