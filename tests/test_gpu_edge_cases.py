@@ -631,3 +631,94 @@ def test_sparse_merge_with_few_pairs_in_many_tiles(hp):
     agg = torch.full((n,), 7.0, device="cuda")
     hp.dgc_decode_merge([dev(p) for p in pays], agg)
     np.testing.assert_array_equal(host(agg), oracle.sparse_decode_merge(pays, n))
+
+
+# ================================================================ streams and graphs
+def test_two_streams_run_different_batches_at_once(hp):
+    """Distinct batches are independent: a DGC set on one stream and a TBQ set on another,
+    enqueued alternately for several steps without waiting in between, give what each gives
+    alone."""
+    rng = np.random.default_rng(77)
+    sizes = [300007, 70001, 1048576]
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    gd = [rng.normal(0, 1e-3, n).astype(F) for n in sizes]
+    gt = [rng.normal(0, 0.02, n).astype(F) for n in sizes]
+    with torch.cuda.stream(s1):
+        td = [{"gradient": dev(g), "momentum": torch.zeros(g.size, device="cuda"), "accumulator": torch.zeros(g.size, device="cuda"),
+               "out": torch.empty(g.size, device="cuda"), "compressed": payload(hp.sparse_payload_bytes(g.size, 0.001))} for g in gd]
+        bd = hp.Batch("dgc", td, momentum_factor=0.9, ratio=0.001)
+    with torch.cuda.stream(s2):
+        tt = [{"gradient": dev(g), "residual": torch.zeros(g.size, device="cuda"), "out": torch.empty(g.size, device="cuda"),
+               "compressed": payload(hp.tbq_payload_bytes(g.size))} for g in gt]
+        bt = hp.Batch("tbq", tt, threshold=0.05)
+    torch.cuda.synchronize()
+    steps = 4
+    for _ in range(steps):
+        with torch.cuda.stream(s1):
+            bd.encode()
+            bd.decode()
+        with torch.cuda.stream(s2):
+            bt.encode()
+            bt.decode()
+    torch.cuda.synchronize()
+    for g, t in zip(gd, td):
+        mom, acc = np.zeros(g.size, F), np.zeros(g.size, F)
+        for _ in range(steps):
+            want, mom, acc = oracle.dgc_encode(g, mom, acc, 0.9, 0.001)
+        check_sparse(host(t["compressed"]), want)
+        np.testing.assert_array_equal(host(t["accumulator"]), acc)
+        np.testing.assert_array_equal(host(t["out"]), oracle.sparse_decode(want, g.size))
+    for g, t in zip(gt, tt):
+        r = np.zeros(g.size, F)
+        for _ in range(steps):
+            want, r = oracle.tbq_encode(g, r, 0.05)
+        np.testing.assert_array_equal(host(t["compressed"]), want)
+        np.testing.assert_array_equal(host(t["residual"]), r)
+    bd.close()
+    bt.close()
+
+
+def test_hip_graph_replay_of_a_sparse_merge_batch(hp):
+    """MergeBatch.run (index, merge + accumulate, three select passes, count, scan, emit)
+    captured once and replayed with new peer payloads before every replay: each replay equals
+    the oracle run from the same state, with the program's own eager work in between."""
+    sizes, P, ratio = [1048576, 300007, 4097], 4, 0.001
+    rng = np.random.default_rng(5)
+    chunks = [{"compressed": [torch.zeros(hp.sparse_payload_bytes(n, ratio), dtype=torch.uint8, device="cuda") for _ in range(P)],
+               "aggregate": torch.empty(n, device="cuda"), "state": torch.zeros(n, device="cuda"),
+               "out_compressed": torch.zeros(hp.sparse_payload_bytes(n, ratio), dtype=torch.uint8, device="cuda")} for n in sizes]
+    mb = hp.MergeBatch("dgc", chunks, ratio=ratio)
+
+    def new_payloads():
+        host_pays = []
+        for c, n in zip(chunks, sizes):
+            ps = [oracle.graddrop_encode(rng.normal(0, 1e-3, n).astype(F), np.zeros(n, F), ratio)[0] for _ in range(P)]
+            for dst, p in zip(c["compressed"], ps):
+                dst.copy_(dev(p))
+            host_pays.append(ps)
+        return host_pays
+
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    new_payloads()
+    with torch.cuda.stream(stream):
+        mb.run()  # warm-up on the capture stream, then back to the initial state
+        stream.synchronize()
+        for c in chunks:
+            c["state"].zero_()
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            mb.run()
+    ref = [np.zeros(n, F) for n in sizes]
+    for rep in range(3):
+        pays = new_payloads()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        _ = (chunks[0]["aggregate"] * 2).sum().item()  # unrelated eager work between replays
+        for i, (c, n) in enumerate(zip(chunks, sizes)):
+            agg, out, ref[i] = oracle.sparse_decode_merge(pays[i], n, ref[i], ratio)
+            np.testing.assert_array_equal(host(c["aggregate"]), agg, err_msg=f"aggregate, replay {rep} chunk {i}")
+            check_sparse(host(c["out_compressed"]), out, f"replay {rep} chunk {i}")
+            np.testing.assert_array_equal(host(c["state"]), ref[i], err_msg=f"state, replay {rep} chunk {i}")
+    mb.close()

@@ -234,6 +234,28 @@ def test_graddrop_150m_elements_three_steps(hp):
     b.close()
 
 
+def test_dgc_one_tensor_beyond_one_accumulate_launch(hp):
+    """One tensor of 49,152 tiles + 12,345 elements through the per-tensor entry point: the
+    accumulate pass is issued in two launches, the second starting in the middle of the
+    tensor.  Two steps against the oracle."""
+    n, ratio, m = 49152 * 4096 + 12345, 0.001, 0.9
+    gen = torch.Generator(device="cuda").manual_seed(23)
+    mom, acc = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    pay = torch.zeros(hp.dgc_payload_bytes(n, ratio), dtype=torch.uint8, device="cuda")
+    g = torch.empty(n, device="cuda")
+    ref_mom, ref_acc = np.zeros(n, F), np.zeros(n, F)
+    for step in range(2):
+        g.normal_(0, 1e-3, generator=gen)
+        hp.dgc_encode(g, mom, acc, pay, m, ratio)
+        want, ref_mom, ref_acc = oracle.dgc_encode(host(g), ref_mom, ref_acc, m, ratio)
+        got, w = oracle.sparse_unpack(host(pay)), oracle.sparse_unpack(want)
+        assert got[:3] == w[:3] and got[3].view(np.uint32) == w[3].view(np.uint32), f"step {step}"
+        np.testing.assert_array_equal(got[4], w[4])
+        np.testing.assert_array_equal(got[5], w[5])
+        np.testing.assert_array_equal(host(acc), ref_acc)
+        np.testing.assert_array_equal(host(mom), ref_mom)
+
+
 def test_merge_vgg19_chunks_tbq(hp):
     """configs[4], TBQ half: 8 peers x 168 chunks of at most 4 MB, decode-and-merge with the
     fused re-encode; every chunk against the oracle, and the integer identity on all."""
