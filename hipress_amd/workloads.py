@@ -4,6 +4,8 @@ import math
 
 import torch
 
+from . import datagen
+
 # VGG19 parameter-gradient sizes in the order of the reference's planner input
 # (/root/reference/src/SeCoPa/input.txt:1-38): 16 conv weight+bias pairs, 3 dense.
 VGG19 = [
@@ -61,36 +63,33 @@ assert sum(bert_large_sizes()) == 335_141_888
 assert len(chunk_sizes(VGG19)) == 168
 
 
-def generator(device, seed):
-    g = torch.Generator(device=device)
-    g.manual_seed(seed)
-    return g
+# Values come from the counter-based generator of datagen.py: element i of tensor t with seed s
+# is a function of (s, t, i) alone.  Streams of one seed are kept apart by an offset in the
+# tensor number.
+_GRAD, _PICK, _LAPLACE, _UNIFORM = 0, 1 << 20, 2 << 20, 3 << 20
 
 
 def normal_set(sizes, device, seed, sigma=None, log_sigma_range=None):
     """One N(0, sigma) tensor per size; with log_sigma_range=(a, b) each tensor
     draws its own sigma = 10**U(a, b)."""
-    gen = generator(device, seed)
-    cpu = torch.Generator().manual_seed(seed)
     out = []
-    for n in sizes:
+    for t, n in enumerate(sizes):
         s = sigma
         if log_sigma_range is not None:
             a, b = log_sigma_range
-            s = 10.0 ** (a + (b - a) * torch.rand((), generator=cpu).item())
-        out.append(torch.randn(n, generator=gen, device=device, dtype=torch.float32) * s)
+            s = 10.0 ** (a + (b - a) * datagen.scalar_uniform(seed, _GRAD + t))
+        out.append(datagen.normal(n, device, seed, _GRAD + t, s))
     return out
 
 
 def heavy_tailed_set(sizes, device, seed, sigma=1e-3, outlier_prob=0.01, laplace_scale=1e-2):
     """N(0, sigma) with each element replaced, with probability outlier_prob, by a
     Laplace(0, laplace_scale) draw."""
-    gen = generator(device, seed)
     out = []
-    for n in sizes:
-        g = torch.randn(n, generator=gen, device=device, dtype=torch.float32) * sigma
-        pick = torch.rand(n, generator=gen, device=device) < outlier_prob
-        u = torch.rand(n, generator=gen, device=device) - 0.5
+    for t, n in enumerate(sizes):
+        g = datagen.normal(n, device, seed, _GRAD + t, sigma)
+        pick = datagen.bernoulli(n, device, seed, _PICK + t, outlier_prob)
+        u = datagen.uniform(n, device, seed, _LAPLACE + t) - 0.5
         lap = -laplace_scale * torch.sign(u) * torch.log1p(-2 * u.abs())
         out.append(torch.where(pick, lap, g))
     return out
@@ -98,12 +97,7 @@ def heavy_tailed_set(sizes, device, seed, sigma=1e-3, outlier_prob=0.01, laplace
 
 def uniform_set(sizes, device, seed):
     """U[0,1) float32 built from 24 random bits, so 1.0 is never produced."""
-    gen = generator(device, seed)
-    out = []
-    for n in sizes:
-        bits = torch.randint(0, 1 << 24, (n,), generator=gen, device=device, dtype=torch.int32)
-        out.append(bits.to(torch.float32) * (1.0 / (1 << 24)))
-    return out
+    return [datagen.uniform(n, device, seed, _UNIFORM + t) for t, n in enumerate(sizes)]
 
 
 def total_bytes(sizes):
