@@ -705,7 +705,7 @@ def main():
                 others.append(measure(name, args.others_steps, 3, 0.0 if args.no_cpu else args.others_cpu_seconds,
                                       args.min_warmup_ms * 1e-3))
     line = {
-        "metric": "fp32 grad GB/s through encode+decode",
+        "metric": "fp32 grad GB/s through encode+decode, % of HBM roofline; VGG19 TBQ, DGC",
         "value": main_res["value"],
         "unit": "GB/s",
         "n_gpus": 1,
@@ -718,7 +718,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
-        "data": "synthetic",
+        "data": "synthetic (counter-based generator, seed 0; values as the configuration states them)",
         "config": {"workload": args.workload, "elements": main_res["elements"], "tensors": main_res["tensors"],
                    "algorithmic_bytes_per_element": main_res["algorithmic_bytes_per_element"]},
         "pct_of_hbm_roofline": main_res["pct_of_hbm_roofline"],
