@@ -1,0 +1,193 @@
+"""Seeded random configurations of every operator against the oracle: sizes that fall
+anywhere relative to word, bucket, group, tile and sample boundaries, parameters over their
+whole range, state carried over two steps.  The cases are fixed by the seed, so a failure
+names its case and repeats."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+@pytest.fixture(scope="module")
+def hp():
+    import hipress_amd
+
+    hipress_amd._lib.lib()
+    return hipress_amd
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def payload(nbytes):
+    return torch.full((nbytes,), 0xAB, dtype=torch.uint8, device="cuda")
+
+
+def sizes(rng, count, top=400_000):
+    """Sizes spread over the orders of magnitude, some of them right at a boundary."""
+    out = []
+    for _ in range(count):
+        n = int(10 ** rng.uniform(0, np.log10(top)))
+        if rng.random() < 0.4:
+            base = int(rng.choice([16, 32, 64, 512, 1024, 4096, 65536, 262144]))
+            n = max(1, base * int(rng.integers(1, 4)) + int(rng.integers(-2, 3)))
+        out.append(n)
+    return out
+
+
+def check_sparse(got_pay, want_pay, where):
+    g, w = oracle.sparse_unpack(got_pay), oracle.sparse_unpack(want_pay)
+    assert g[:3] == w[:3] and g[3].view(np.uint32) == w[3].view(np.uint32), (where, g[:4], w[:4])
+    np.testing.assert_array_equal(g[4], w[4], err_msg=where)
+    np.testing.assert_array_equal(g[5], w[5], err_msg=where)
+
+
+def test_dense_quantisers_random_cases(hp):
+    rng = np.random.default_rng(2024)
+    for case, n in enumerate(sizes(rng, 150)):
+        sigma = 10 ** rng.uniform(-4, 0)
+        tau = float(F(sigma * rng.uniform(0.2, 4.0)))
+        bucket = int(rng.choice([256, 512, 1024, 16, 100, 777, 4096]))
+        where = f"case {case}: n={n} sigma={sigma:.3g} tau={tau:.3g} bucket={bucket}"
+        r_t, r_o = rng.normal(0, sigma, n).astype(F), None
+        r_o = r_t.copy()
+        rt_gpu, ro_gpu = dev(r_t), dev(r_o)
+        for step in range(2):
+            g, u = rng.normal(0, sigma, n).astype(F), rng.random(n, dtype=F)
+            pay = payload(hp.tbq_payload_bytes(n))
+            hp.tbq_encode(dev(g), rt_gpu, pay, tau)
+            want, r_t = oracle.tbq_encode(g, r_t, tau)
+            np.testing.assert_array_equal(host(pay), want, err_msg="tbq " + where)
+            np.testing.assert_array_equal(host(rt_gpu), r_t, err_msg="tbq residual " + where)
+            out = torch.full((n,), 7.0, device="cuda")
+            hp.tbq_decode(pay, out)
+            np.testing.assert_array_equal(host(out), oracle.tbq_decode(want, n), err_msg="tbq decode " + where)
+            pay = payload(hp.onebit_payload_bytes(n))
+            hp.onebit_encode(dev(g), ro_gpu, pay)
+            got = host(pay)
+            s = got[:4].view(F)[0]
+            s_ref = oracle.onebit_scale(g, r_o)
+            assert abs(float(s) - float(s_ref)) <= 1e-5 * float(s_ref), "onebit scale " + where
+            want, r_o = oracle.onebit_encode(g, r_o, scale=s)
+            np.testing.assert_array_equal(got, want, err_msg="onebit " + where)
+            np.testing.assert_array_equal(host(ro_gpu), r_o, err_msg="onebit residual " + where)
+            pay = payload(hp.terngrad_payload_bytes(n, bucket))
+            hp.terngrad_encode(dev(g), dev(u), pay, bucket)
+            want = oracle.terngrad_encode(g, u, bucket)
+            np.testing.assert_array_equal(host(pay), want, err_msg="terngrad " + where)
+            hp.terngrad_decode(pay, out)
+            np.testing.assert_array_equal(host(out), oracle.terngrad_decode(want, n), err_msg="terngrad decode " + where)
+
+
+def test_sparsifiers_random_cases(hp):
+    rng = np.random.default_rng(2025)
+    for case, n in enumerate(sizes(rng, 150, top=1_500_000)):
+        ratio = float(10 ** rng.uniform(-3.3, -0.5))
+        m = float(F(rng.uniform(0.0, 0.99)))
+        heavy = rng.random() < 0.3  # many equal magnitudes: ties at the threshold, overflow of the slots
+        where = f"case {case}: n={n} ratio={ratio:.4g} m={m:.3g} heavy={heavy}"
+        mom_ref, acc_ref, gacc_ref = np.zeros(n, F), np.zeros(n, F), np.zeros(n, F)
+        mom, acc, gacc = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+        for step in range(2):
+            g = rng.normal(0, 1e-3, n).astype(F)
+            if heavy:
+                g = (np.round(g * 2000) / 2000).astype(F)
+            pay = payload(hp.sparse_payload_bytes(n, ratio))
+            hp.dgc_encode(dev(g), mom, acc, pay, m, ratio)
+            want, mom_ref, acc_ref = oracle.dgc_encode(g, mom_ref, acc_ref, m, ratio)
+            check_sparse(host(pay), want, "dgc " + where)
+            np.testing.assert_array_equal(host(mom), mom_ref, err_msg="dgc momentum " + where)
+            np.testing.assert_array_equal(host(acc), acc_ref, err_msg="dgc accumulator " + where)
+            out = torch.full((n,), 7.0, device="cuda")
+            hp.dgc_decode(pay, out)
+            np.testing.assert_array_equal(host(out), oracle.sparse_decode(want, n), err_msg="decode " + where)
+            pay = payload(hp.sparse_payload_bytes(n, ratio))
+            hp.graddrop_encode(dev(g), gacc, pay, ratio)
+            want, gacc_ref = oracle.graddrop_encode(g, gacc_ref, ratio)
+            check_sparse(host(pay), want, "graddrop " + where)
+            np.testing.assert_array_equal(host(gacc), gacc_ref, err_msg="graddrop accumulator " + where)
+
+
+def test_merges_random_cases(hp):
+    rng = np.random.default_rng(2026)
+    for case, n in enumerate(sizes(rng, 80, top=1_200_000)):
+        P = int(rng.integers(1, 17))
+        tau = float(F(rng.uniform(0.01, 0.1)))
+        ratio = float(10 ** rng.uniform(-3, -1.3))
+        where = f"case {case}: n={n} peers={P} tau={tau:.3g} ratio={ratio:.3g}"
+        z = np.zeros(n, F)
+        tp = [oracle.tbq_encode(rng.normal(0, 0.04, n).astype(F), z, tau)[0] for _ in range(P)]
+        r0 = rng.normal(0, 0.02, n).astype(F)
+        agg, res, outp = torch.full((n,), 7.0, device="cuda"), dev(r0), payload(hp.tbq_payload_bytes(n))
+        hp.tbq_decode_merge([dev(p) for p in tp], agg, res, outp, tau)
+        want_agg, want_out, want_r = oracle.tbq_decode_merge(tp, n, r0, tau)
+        np.testing.assert_array_equal(host(agg), want_agg, err_msg="tbq merge " + where)
+        np.testing.assert_array_equal(host(outp), want_out, err_msg="tbq merge payload " + where)
+        np.testing.assert_array_equal(host(res), want_r, err_msg="tbq merge residual " + where)
+        sp = [oracle.graddrop_encode(rng.normal(0, 1e-3, n).astype(F), z, ratio)[0] for _ in range(P)]
+        a0 = rng.normal(0, 1e-4, n).astype(F)
+        agg, acc, outp = torch.full((n,), 7.0, device="cuda"), dev(a0), payload(hp.sparse_payload_bytes(n, ratio))
+        hp.dgc_decode_merge([dev(p) for p in sp], agg, acc, outp, ratio)
+        want_agg, want_out, want_acc = oracle.sparse_decode_merge(sp, n, a0, ratio)
+        np.testing.assert_array_equal(host(agg), want_agg, err_msg="sparse merge " + where)
+        check_sparse(host(outp), want_out, "sparse merge payload " + where)
+        np.testing.assert_array_equal(host(acc), want_acc, err_msg="sparse merge accumulator " + where)
+
+
+def test_batches_of_random_tensor_tables(hp):
+    rng = np.random.default_rng(2027)
+    for alg in ("tbq", "terngrad", "dgc", "graddrop"):
+        for table in range(8):
+            ns = sizes(rng, int(rng.integers(2, 25)), top=600_000)
+            ratio = 0.01 if alg == "graddrop" else 0.001
+            ts, data = [], []
+            for n in ns:
+                g, u = rng.normal(0, 0.02 if alg == "tbq" else 1e-3, n).astype(F), rng.random(n, dtype=F)
+                nbytes = {"tbq": hp.tbq_payload_bytes(n), "terngrad": hp.terngrad_payload_bytes(n, 512),
+                          "dgc": hp.sparse_payload_bytes(n, ratio), "graddrop": hp.sparse_payload_bytes(n, ratio)}[alg]
+                t = {"gradient": dev(g), "out": torch.full((n,), 7.0, device="cuda"), "compressed": payload(nbytes)}
+                if alg == "tbq":
+                    t["residual"] = torch.zeros(n, device="cuda")
+                elif alg == "terngrad":
+                    t["uniform"] = dev(u)
+                elif alg == "dgc":
+                    t["momentum"], t["accumulator"] = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+                else:
+                    t["accumulator"] = torch.zeros(n, device="cuda")
+                ts.append(t)
+                data.append((g, u))
+            b = hp.Batch(alg, ts, threshold=0.05, bucket=512, momentum_factor=0.9, ratio=ratio)
+            b.encode()
+            b.decode()
+            for i, (t, n, (g, u)) in enumerate(zip(ts, ns, data)):
+                where = f"{alg} table {table} tensor {i} n={n}"
+                z = np.zeros(n, F)
+                got = host(t["compressed"])
+                if alg == "tbq":
+                    want = oracle.tbq_encode(g, z, 0.05)[0]
+                    np.testing.assert_array_equal(got, want, err_msg=where)
+                    ref = oracle.tbq_decode(want, n)
+                elif alg == "terngrad":
+                    want = oracle.terngrad_encode(g, u, 512)
+                    np.testing.assert_array_equal(got, want, err_msg=where)
+                    ref = oracle.terngrad_decode(want, n)
+                elif alg == "dgc":
+                    want = oracle.dgc_encode(g, z, z, 0.9, ratio)[0]
+                    check_sparse(got, want, where)
+                    ref = oracle.sparse_decode(want, n)
+                else:
+                    want = oracle.graddrop_encode(g, z, ratio)[0]
+                    check_sparse(got, want, where)
+                    ref = oracle.sparse_decode(want, n)
+                np.testing.assert_array_equal(host(t["out"]), ref, err_msg="decode " + where)
+            b.close()
