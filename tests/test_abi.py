@@ -159,3 +159,33 @@ def test_reference_operator_names_keep_the_reference_signature():
     assert len(schema.returns) == 0  # in place, zero outputs (TernGradEncode.cc:12-13)
     # the bucketed ternariser keeps its own name
     assert ops.ALIASES["BucketTernGradEncode"] is ops.terngrad_encode
+
+
+def test_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
+    """Without libhipress_amd.so the operators raise; nothing computes on the CPU instead."""
+    import torch
+
+    from hipress_amd import _lib, ops
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libhipress_amd.so"))
+    with pytest.raises(ImportError, match="no CPU fallback"):
+        _lib.lib()
+    with pytest.raises(ImportError):
+        ops.tbq_payload_bytes(16)
+    # and a CPU tensor is refused before any library call
+    monkeypatch.undo()
+    with pytest.raises(ValueError, match="GPU"):
+        ops.tbq_encode(torch.zeros(16), torch.zeros(16), torch.zeros(32, dtype=torch.uint8), 0.05)
+    # the package never imports the oracle
+    import hipress_amd
+    import os
+    import re
+
+    root = os.path.dirname(hipress_amd.__file__)
+    for dirpath, _, files in os.walk(root):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f), errors="ignore").read()
+                assert not re.search(r"^\s*(import oracle|from oracle)", text, re.M), f
+                assert "libhipress_oracle" not in text, f
