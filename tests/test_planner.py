@@ -152,13 +152,14 @@ def test_fit_recovers_a_known_model():
 
 @pytest.mark.gpu
 def test_calibration_on_this_gpu_agrees_with_the_committed_models():
-    """Three sizes of TBQ measured on cuda:0: a positive floor, a slope within a factor of two
-    of the committed one, and the same VGG19 plan as the committed models give."""
+    """Three sizes of TBQ measured on cuda:0 (the two large ones far enough apart that the line
+    through them is the kernel's rate, not timer noise): a positive floor, a slope within a
+    factor of two of the committed one, and the same VGG19 plan as the committed models give."""
     import json
 
     with open(P.MEASURED_PATH) as f:
         data = json.load(f)
-    cal = P.calibrate("tbq", sizes=[2 ** 10, 2 ** 20, 2 ** 24], reps=10)
+    cal = P.calibrate("tbq", sizes=[2 ** 10, 2 ** 22, 2 ** 26], reps=10)
     for kind in ("encode", "decode"):
         got, want = cal[kind], data[kind]["tbq"]
         assert got.overhead > 0
@@ -168,6 +169,6 @@ def test_calibration_on_this_gpu_agrees_with_the_committed_models():
     grads = P.read_gradients(os.path.join(GOLDEN, "secopa_input.txt"))
     want = [l.strip() for l in open(os.path.join(GOLDEN, "plan_vgg19_tbq_ps4_mi355x.txt")) if l.strip()]
     assert pl.plan(grads, "PS") == want
-    mer = P.calibrate_merge("dgc", npeers=3, sizes=[2 ** 12, 2 ** 20, 2 ** 24], reps=5)
+    mer = P.calibrate_merge("dgc", npeers=3, sizes=[2 ** 12, 2 ** 22, 2 ** 26], reps=5)
     assert mer["merge"].overhead > 0
     assert 0.5 * data["merge"]["dgc"]["3"]["weight"] <= mer["merge"].weight <= 2.0 * data["merge"]["dgc"]["3"]["weight"]
