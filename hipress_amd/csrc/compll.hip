@@ -65,31 +65,39 @@ constexpr int kHeaderBlock = 1024;
 
 template <class SegSrc>
 __global__ __launch_bounds__(kHeaderBlock) void compll_header_kernel(SegSrc src, const float* partial) {
-    __shared__ float smx[kHeaderBlock], smn[kHeaderBlock];
+    __shared__ float smx[kHeaderBlock / 64], smn[kHeaderBlock / 64];
     const Seg s = src.at(blockIdx.x);
-    float mx = kMaxInit, mn = kMinInit;
+    const unsigned nt = s.ntiles;
     const float2* p2 = reinterpret_cast<const float2*>(partial) + s.tile0;
-    for (unsigned t = threadIdx.x; t < s.ntiles; t += kHeaderBlock) {
+    float mx = kMaxInit, mn = kMinInit;
+    unsigned t = threadIdx.x;
+    for (; t + 3 * kHeaderBlock < nt; t += 4 * kHeaderBlock) {  // four loads in flight per lane
+        float2 v0 = p2[t], v1 = p2[t + kHeaderBlock], v2 = p2[t + 2 * kHeaderBlock], v3 = p2[t + 3 * kHeaderBlock];
+        mx = fmaxf(fmaxf(mx, v0.x), fmaxf(fmaxf(v1.x, v2.x), v3.x));
+        mn = fminf(fminf(mn, v0.y), fminf(fminf(v1.y, v2.y), v3.y));
+    }
+    for (; t < nt; t += kHeaderBlock) {
         float2 v = p2[t];
         mx = fmaxf(mx, v.x);
         mn = fminf(mn, v.y);
     }
-    smx[threadIdx.x] = mx;
-    smn[threadIdx.x] = mn;
-    __syncthreads();
-    for (int w = kHeaderBlock / 2; w >= 1; w >>= 1) {
-        if ((int)threadIdx.x < w) {
-            smx[threadIdx.x] = fmaxf(smx[threadIdx.x], smx[threadIdx.x + w]);
-            smn[threadIdx.x] = fminf(smn[threadIdx.x], smn[threadIdx.x + w]);
-        }
-        __syncthreads();
+    mx = wave_max(mx);
+    mn = -wave_max(-mn);
+    if ((threadIdx.x & 63u) == 0) {
+        smx[threadIdx.x >> 6] = mx;
+        smn[threadIdx.x >> 6] = mn;
     }
+    __syncthreads();
     if (threadIdx.x == 0) {
+        for (int w = 1; w < kHeaderBlock / 64; ++w) {
+            mx = fmaxf(mx, smx[w]);
+            mn = fminf(mn, smn[w]);
+        }
         const unsigned b = s.bucket;  // bit width
         s.pay[0] = (uint8_t)b;
         s.pay[1] = (uint8_t)(s.n % (1ull << b));  // the DSL's tail = size % (1 << bitwidth)
-        store_f32_bytes(s.pay + 2, smn[0]);
-        store_f32_bytes(s.pay + 6, smx[0]);
+        store_f32_bytes(s.pay + 2, mn);
+        store_f32_bytes(s.pay + 6, mx);
     }
 }
 

@@ -232,13 +232,29 @@ __global__ __launch_bounds__(kBlock) void reduce_tiles_kernel(Args a, const Dev*
 // After::run: the scalar statements that follow the reduce in the program, if any.
 template <class Args, class Dev, class Folds, class After>
 __global__ __launch_bounds__(kFinalBlock) void reduce_final_kernel(Args a, Dev* d, const float* partial, unsigned ntiles) {
-    __shared__ float sh[kFinalBlock][Folds::K];
-    __shared__ int sh_any[kFinalBlock];
+    constexpr int kWaves = kFinalBlock / 64;
+    __shared__ float wave_acc[kWaves][Folds::K];
+    __shared__ int wave_any[kWaves];
     float acc[Folds::K];
 #pragma unroll
     for (int k = 0; k < Folds::K; ++k) acc[k] = 0.f;
     bool any = false;
-    for (unsigned t = threadIdx.x; t < ntiles; t += kFinalBlock) {
+    unsigned t = threadIdx.x;
+    for (; t + 3 * kFinalBlock < ntiles; t += 4 * kFinalBlock) {  // four rows of loads in flight per lane
+        float p[4][Folds::K];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int k = 0; k < Folds::K; ++k) p[u][k] = partial[(long long)(t + u * kFinalBlock) * Folds::K + k];
+#pragma unroll
+        for (int k = 0; k < Folds::K; ++k) {
+            const float q = Folds::apply(a, *d, k, Folds::apply(a, *d, k, p[0][k], p[1][k]),
+                                         Folds::apply(a, *d, k, p[2][k], p[3][k]));
+            acc[k] = any ? Folds::apply(a, *d, k, acc[k], q) : q;
+        }
+        any = true;
+    }
+    for (; t < ntiles; t += kFinalBlock) {
 #pragma unroll
         for (int k = 0; k < Folds::K; ++k) {
             const float p = partial[(long long)t * Folds::K + k];
@@ -246,25 +262,32 @@ __global__ __launch_bounds__(kFinalBlock) void reduce_final_kernel(Args a, Dev* 
         }
         any = true;
     }
-    sh_any[threadIdx.x] = any;
 #pragma unroll
-    for (int k = 0; k < Folds::K; ++k) sh[threadIdx.x][k] = acc[k];
-    __syncthreads();
-    for (int w = kFinalBlock / 2; w >= 1; w >>= 1) {
-        if ((int)threadIdx.x < w && sh_any[threadIdx.x + w]) {
+    for (int m = 1; m < 64; m <<= 1) {
+        const bool other_any = __shfl_xor((int)any, m, 64) != 0;
 #pragma unroll
-            for (int k = 0; k < Folds::K; ++k)
-                sh[threadIdx.x][k] = sh_any[threadIdx.x] ? Folds::apply(a, *d, k, sh[threadIdx.x][k], sh[threadIdx.x + w][k])
-                                                         : sh[threadIdx.x + w][k];
-            sh_any[threadIdx.x] = 1;
+        for (int k = 0; k < Folds::K; ++k) {
+            const float other = __shfl_xor(acc[k], m, 64);
+            acc[k] = (any && other_any) ? Folds::apply(a, *d, k, acc[k], other) : (any ? acc[k] : other);
         }
-        __syncthreads();
+        any = any || other_any;
     }
-    if (threadIdx.x == 0) {
+    if ((threadIdx.x & 63u) == 0) {
+        wave_any[threadIdx.x >> 6] = any;
+#pragma unroll
+        for (int k = 0; k < Folds::K; ++k) wave_acc[threadIdx.x >> 6][k] = acc[k];
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {  // lanes are filled from thread 0 upwards, so wavefront 0 holds a value whenever any does
+        for (int w = 1; w < kWaves; ++w)
+            if (wave_any[w]) {
+#pragma unroll
+                for (int k = 0; k < Folds::K; ++k) acc[k] = Folds::apply(a, *d, k, acc[k], wave_acc[w][k]);
+            }
 #pragma unroll
         for (int k = 0; k < Folds::K; ++k) {
             const float init = Folds::init(a, *d, k);
-            Folds::store(*d, k, sh_any[0] ? Folds::apply(a, *d, k, init, sh[0][k]) : init);
+            Folds::store(*d, k, any ? Folds::apply(a, *d, k, init, acc[k]) : init);
         }
         After::run(a, *d);
     }
