@@ -74,6 +74,12 @@ enum { kCtlPrefix1 = 0, kCtlK1 = 1, kCtlPrefix2 = 2, kCtlK2 = 3, kCtlWords = 8 }
 
 // ---- 0. accumulate -------------------------------------------------------------
 
+// y / kSampleStride for y < 1024 + kSampleStride
+__device__ __forceinline__ unsigned sample_quot(unsigned y) {
+    static_assert(kSampleStride == 100, "the multiplier below is the one for 100");
+    return __umul24(y, 5243u) >> 19;
+}
+
 // gload(j, e) supplies the four gradient values of step j (element e): global
 // memory for the encoders, the LDS tile of merged peers for decode-and-merge.
 // aload(j, e) supplies the accumulator values the same way (decode-and-merge
@@ -86,6 +92,12 @@ __device__ __forceinline__ void sparse_accum_tile(const Seg& s, unsigned tile, c
     const long long base = (long long)tile * kTile + wave * kWaveTile;
     const float mf = s.f0;
     uint32_t* sample = ws.sample + s.ws0;
+    // the first sample position q0*S + S/2 at or behind the wavefront's first element, and its
+    // distance off0 < S from that element: the same in every lane, so scalar arithmetic
+    const unsigned long long wbase =
+        (unsigned long long)tile * kTile + (unsigned)__builtin_amdgcn_readfirstlane((int)wave) * kWaveTile;
+    const unsigned long long q0 = (wbase + (kSampleStride - 1 - kSampleStride / 2)) / kSampleStride;
+    const unsigned off0 = (unsigned)(q0 * kSampleStride + kSampleStride / 2 - wbase);
     f4 g[4], a[4], m[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -140,12 +152,15 @@ __device__ __forceinline__ void sparse_accum_tile(const Seg& s, unsigned tile, c
             if (e + 2 < n) sample[e + 2] = k2;
             if (e + 3 < n) sample[e + 3] = k3;
         } else {  // sample positions are q*S + S/2; at most one falls into [e, e+4)
-            constexpr unsigned long long S = kSampleStride, h = S / 2;  // a constant: division by multiply
-            unsigned long long q = ((unsigned long long)e + (S - 1 - h)) / S;  // first q with q*S+h >= e
-            unsigned long long p = q * S + h;
-            if (p < (unsigned long long)e + 4 && q < s.ns) {
-                unsigned d = (unsigned)(p - (unsigned long long)e);
-                sample[q] = d == 0 ? k0 : (d == 1 ? k1 : (d == 2 ? k2 : k3));
+            // first sample at or behind this step's four elements, counted from the wavefront's
+            // first sample: x + S-1 - off0 < 1024 + S, so the quotient by S is a 24-bit
+            // multiply and a shift
+            const unsigned x = (unsigned)j * 256u + lane * 4u;
+            const unsigned t = sample_quot(x + (unsigned)kSampleStride - 1u - off0);
+            const unsigned at = off0 + t * (unsigned)kSampleStride;  // place of that sample in the wavefront's 1024
+            if (at < x + 4u && q0 + t < s.ns) {
+                const unsigned d = at - x;
+                sample[q0 + t] = d == 0 ? k0 : (d == 1 ? k1 : (d == 2 ? k2 : k3));
             }
         }
     }
