@@ -298,16 +298,16 @@ class MergeWorkload:
             self.mb.run()
 
     def cpu_job(self):
-        """decode-and-merge + re-encode of the first chunks in the CPU oracle, on the very
+        """decode-and-merge + re-encode of four full-sized chunks in the CPU oracle, on the very
         peer payloads the GPU run merges."""
         import numpy as np
 
-        picks, total = _sample_front(self.sizes)
-        picks = picks[:4]
-        total = sum(k for _, k in picks)
+        # four full-sized chunks: the set's first chunks are a few thousand elements each, which
+        # times call overhead rather than the merge
+        order = sorted(range(len(self.sizes)), key=lambda i: (-self.sizes[i], i))[:4]
         P, alg, ratio = self.npeers, self.alg, self.ratio
         jobs = []
-        for i, k in picks:
+        for i in sorted(order):
             n = self.sizes[i]
             pays = [p.cpu().numpy() for p in self.chunks[i]["compressed"]]
             arr = (ctypes.c_void_p * P)(*[p.ctypes.data for p in pays])
@@ -322,7 +322,7 @@ class MergeWorkload:
                 else:
                     L.hpo_sparse_decode_merge(arr, P, _vp(agg), n, _vp(state), _vp(outp), ratio)
 
-        what = (f"{alg} decode-and-merge of {P} peers + re-encode over the first {len(jobs)} of "
+        what = (f"{alg} decode-and-merge of {P} peers + re-encode over the {len(jobs)} largest of "
                 f"{len(self.sizes)} chunks ({total:,} elements per pass)")
         return CpuJob(total, what, run)
 
