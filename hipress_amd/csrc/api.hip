@@ -790,8 +790,8 @@ int hipress_batch_destroy(hipress_batch* b) {
     return HIPRESS_OK;
 }
 
-int hipress_batch_create(hipress_batch** out, int32_t alg, const hipress_tensor* tensors, int32_t count,
-                         const hipress_params* params) {
+static int batch_create_impl(hipress_batch** out, int32_t alg, const hipress_tensor* tensors, int32_t count,
+                             const hipress_params* params) {
     if (!out || !params || (count > 0 && !tensors)) return HIPRESS_ERR_NULL;
     *out = nullptr;
     if (count < 0) return HIPRESS_ERR_SIZE;
@@ -814,7 +814,11 @@ int hipress_batch_create(hipress_batch** out, int32_t alg, const hipress_tensor*
     if (!enc_ok && !dec_ok) { delete b; return HIPRESS_ERR_NULL; }
     b->can_encode = enc_ok;
     b->can_decode = dec_ok;
-    auto fail = [&](int code) { hipress_batch_destroy(b); return code; };
+    struct Guard {  // frees the half-built batch on every way out but the last
+        hipress_batch* b;
+        ~Guard() { hipress_batch_destroy(b); }
+    } guard{b};
+    auto fail = [](int code) { return code; };
     for (int i = 0; i < count; ++i) {
         const hipress_tensor& t = tensors[i];
         Seg s;
@@ -856,8 +860,21 @@ int hipress_batch_create(hipress_batch** out, int32_t alg, const hipress_tensor*
     if ((rc = upload(b->enc, &b->d_enc))) return fail(rc);
     if ((rc = upload(b->dec, &b->d_dec))) return fail(rc);
     if ((rc = upload(map, &b->d_map))) return fail(rc);
+    guard.b = nullptr;
     *out = b;
     return HIPRESS_OK;
+}
+
+// Host allocations of the set-up (descriptor vectors, maps) may fail with an exception,
+// which must not leave a C function: it is reported as an error code instead.
+int hipress_batch_create(hipress_batch** out, int32_t alg, const hipress_tensor* tensors, int32_t count,
+                         const hipress_params* params) {
+    try {
+        return batch_create_impl(out, alg, tensors, count, params);
+    } catch (...) {
+        if (out) *out = nullptr;
+        return HIPRESS_ERR_HIP;
+    }
 }
 
 static Launch batch_launch(const hipress_batch* b, bool encode) {
@@ -943,19 +960,24 @@ int hipress_merge_batch_destroy(hipress_merge_batch* b) {
     return HIPRESS_OK;
 }
 
-int hipress_merge_batch_create(hipress_merge_batch** out, int32_t alg, const hipress_merge_chunk* chunks,
-                               int32_t count, int32_t npeers, const hipress_params* params) {
+static int merge_batch_create_impl(hipress_merge_batch** out, int32_t alg, const hipress_merge_chunk* chunks,
+                                   int32_t count, int32_t npeers, const hipress_params* params) {
     if (!out || !params || (count > 0 && !chunks)) return HIPRESS_ERR_NULL;
     *out = nullptr;
     if (count < 0) return HIPRESS_ERR_SIZE;
     if (alg < HIPRESS_ONEBIT || alg > HIPRESS_GRADDROP) return HIPRESS_ERR_PARAM;
+    if (npeers < 1 || npeers > HIPRESS_MAX_PEERS) return HIPRESS_ERR_PARAM;
     hipress_merge_batch* b = new (std::nothrow) hipress_merge_batch;
     if (!b) return HIPRESS_ERR_HIP;
     b->alg = alg;
     b->params = *params;
     b->npeers = npeers;
     const bool sparse = alg == HIPRESS_DGC || alg == HIPRESS_GRADDROP;
-    auto fail = [&](int code) { hipress_merge_batch_destroy(b); return code; };
+    struct Guard {  // frees the half-built batch on every way out but the last
+        hipress_merge_batch* b;
+        ~Guard() { hipress_merge_batch_destroy(b); }
+    } guard{b};
+    auto fail = [](int code) { return code; };
     int rc;
     bool any_state = false, all_state = true;
     for (int i = 0; i < count; ++i) {
@@ -1005,8 +1027,19 @@ int hipress_merge_batch_create(hipress_merge_batch** out, int32_t alg, const hip
     if ((rc = upload(b->segs, &b->d_segs))) return fail(rc);
     if ((rc = upload(b->renc, &b->d_renc))) return fail(rc);
     if ((rc = upload(map, &b->d_map))) return fail(rc);
+    guard.b = nullptr;
     *out = b;
     return HIPRESS_OK;
+}
+
+int hipress_merge_batch_create(hipress_merge_batch** out, int32_t alg, const hipress_merge_chunk* chunks,
+                               int32_t count, int32_t npeers, const hipress_params* params) {
+    try {
+        return merge_batch_create_impl(out, alg, chunks, count, npeers, params);
+    } catch (...) {
+        if (out) *out = nullptr;
+        return HIPRESS_ERR_HIP;
+    }
 }
 
 // phase < 0: everything.  Sparse: 0 index, 1 merge (+ accumulate of the re-encode),

@@ -89,6 +89,13 @@ def test_null_and_range_checks_need_no_gpu(lib):
     nb = (ctypes.c_int64 * 1)(1 << 20)
     assert L.hipress_tbq_decode_merge(pay, nb, 1, None, 16, None, None, 0, 0.05, None) == -1
     assert L.hipress_onebit_decode_merge(pay, nb, 1, None, 16, None) == -1
+    # a peer count outside 1 .. 16 is refused before anything is allocated, also for an empty chunk list
+    pr = lib.Params(0.05, 512, 0.9, 0.0, 0.001)
+    h = ctypes.c_void_p()
+    for alg in (lib.TBQ, lib.DGC):
+        for npeers in (0, -1, 17):
+            assert L.hipress_merge_batch_create(ctypes.byref(h), alg, None, 0, npeers, ctypes.byref(pr)) == -4
+            assert not h.value
 
 
 def test_sparse_entry_points_reject_what_int32_indices_cannot_address(lib):
