@@ -230,6 +230,37 @@ class SetWorkload:
         self.batches, self.tensors = [], []
 
 
+class PlannedWorkload(SetWorkload):
+    """The VGG19 set as the planner cuts it for `nodes` nodes with the models measured on
+    MI355X: gradients the plan marks `n` are left out, the others are compressed partition
+    by partition (hipress_amd.PlannedSet), all partitions in one launch sequence."""
+
+    def __init__(self, name, alg, params, enc_bytes, dec_bytes, dominant_kernel, nodes=4):
+        from hipress_amd import planner
+        from hipress_amd import workloads as W
+
+        self.full_sizes = W.vgg19_sizes()
+        names = [f"g{i}" for i in range(len(self.full_sizes))]
+        self.plan = [planner.parse_plan_line(l) for l in
+                     planner.Planner.from_measured(alg, nodes).plan(zip(names, self.full_sizes), "PS")]
+        sizes = [ln for _, size, c, k in self.plan if c for _, ln in planner.partition_bounds(size, k)]
+        super().__init__(name, alg, sizes, "vgg", params, enc_bytes, dec_bytes, 0, dominant_kernel, enc_bytes)
+
+    def setup(self, dev):
+        import hipress_amd as hp
+        from hipress_amd import workloads as W
+
+        grads = W.normal_set(self.full_sizes, dev, 0, log_sigma_range=(-4.0, -2.0))
+        self.planned = hp.PlannedSet(self.alg, self.plan, {p[0]: g for p, g in zip(self.plan, grads)}, **self.params)
+        self.batches = [self.planned._batch]
+        self.tensors = [self.planned._batch._keep]
+        self.k = 0
+
+    def close(self):
+        self.planned.close()
+        self.batches, self.tensors = [], []
+
+
 class MergeWorkload:
     """Decode-and-merge of 8 peer payloads per 4 MB chunk of the VGG19 set, with the
     fused re-encode for the next hop."""
@@ -479,6 +510,8 @@ def make_workload(name):
         return GeneratedTbqWorkload(name, max(vgg), generated=False)
     if name == "tbq_generated_fc6":
         return GeneratedTbqWorkload(name, max(vgg), generated=True)
+    if name == "tbq_vgg19_planned":
+        return PlannedWorkload(name, "tbq", {"threshold": 0.05}, 12.25, 4.25, "tbq_encode_kernel")
     if name == "merge_tbq_vgg19":
         return MergeWorkload(name, "tbq", W.chunk_sizes(vgg))
     if name == "merge_dgc_vgg19":
@@ -495,7 +528,7 @@ ALL_WORKLOADS = [
     "tbq_vgg19", "dgc_vgg19", "onebit_vgg19", "terngrad_vgg19", "graddrop_vgg19", "onebit_deferred_vgg19",
     "tbq_262144", "tbq_262144_x512", "terngrad_resnet50", "dgc_bert_large", "graddrop_bert_large",
     "merge_tbq_vgg19", "merge_dgc_vgg19", "compll_b2_fc6", "compll_generated_b2_fc6", "tbq_fc6", "tbq_generated_fc6",
-    "merge_tbq_vgg19_payload_only", "merge_dgc_vgg19_payload_only",
+    "merge_tbq_vgg19_payload_only", "merge_dgc_vgg19_payload_only", "tbq_vgg19_planned",
 ]
 # any workload with the suffix _graph: the same step captured once into a HIP graph and replayed
 EXTRA_WORKLOADS = [w + "_graph" for w in ALL_WORKLOADS]

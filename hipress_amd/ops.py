@@ -31,7 +31,7 @@ __all__ = [
     "dgc_encode", "dgc_decode", "graddrop_encode", "graddrop_decode",
     "compll_payload_bytes", "compll_decoded_count", "compll_terngrad_encode", "compll_terngrad_decode",
     "onebit_decode_merge", "tbq_decode_merge", "terngrad_decode_merge", "dgc_decode_merge",
-    "graddrop_decode_merge", "Batch", "MergeBatch", "ALIASES",
+    "graddrop_decode_merge", "Batch", "MergeBatch", "PlannedSet", "ALIASES",
 ]
 
 
@@ -524,6 +524,96 @@ class MergeBatch:
             self.close()
         except Exception:
             pass
+
+class PlannedSet:
+    """A model's gradients under a SeCoPa plan, on one GPU.
+
+    The plan (`name,size,y|n,K` lines, /root/reference/src/SeCoPa/SeCoPa.py:139-151, or the
+    tuples ``planner.read_plan`` returns) says for every gradient whether to compress it
+    and into how many partitions to cut it.  A gradient marked ``y`` is cut with
+    ``planner.partition_bounds`` and every partition is compressed on its own - its own
+    payload, header and statistics - since the partition is the unit the runtime encodes,
+    sends and merges (/root/reference/README.md:134).  A gradient marked ``n`` is left
+    alone and listed in ``uncompressed``.  All partitions of the set run in one launch
+    sequence (a ``Batch``).
+
+    ``gradients``: dict name -> contiguous float32 tensor, which must keep its address.
+    The set allocates what the algorithm needs beside them and exposes it by gradient
+    name: ``state[name]`` (dict of whole-gradient tensors: residual / momentum,
+    accumulator / state, scale_state per partition), ``compressed[name]`` (one uint8
+    payload per partition), ``out[name]`` (the decoded gradient, whole).  TernGrad reads
+    its rounding noise from ``uniform[name]``, one float32 tensor per compressed gradient.
+    """
+
+    def __init__(self, alg, plan, gradients, uniform=None, threshold=0.0, bucket=512, momentum_factor=0.9,
+                 ratio=0.001):
+        from . import planner
+
+        if alg not in ALG_IDS:
+            raise ValueError(f"unknown algorithm {alg!r}")
+        self.alg = alg
+        self.parts, self.uncompressed = [], []
+        self.state, self.compressed, self.out = {}, {}, {}
+        nbytes = {"onebit": onebit_payload_bytes, "onebit_deferred": onebit_payload_bytes, "tbq": tbq_payload_bytes,
+                  "terngrad": lambda n: terngrad_payload_bytes(n, bucket),
+                  "dgc": lambda n: sparse_payload_bytes(n, ratio),
+                  "graddrop": lambda n: sparse_payload_bytes(n, ratio)}[alg]
+        state_names = {"onebit": ("residual",), "tbq": ("residual",), "onebit_deferred": ("state",),
+                       "dgc": ("momentum", "accumulator"), "graddrop": ("accumulator",), "terngrad": ()}[alg]
+        tensors = []
+        for entry in plan:
+            name, size_, compress, k = planner.parse_plan_line(entry) if isinstance(entry, str) else entry
+            if name not in gradients:
+                raise KeyError(f"the plan names {name!r}, which is not among the gradients")
+            g = gradients[name]
+            if g.numel() != size_:
+                raise ValueError(f"{name}: the plan says {size_} elements, the gradient has {g.numel()}")
+            if not compress:
+                self.uncompressed.append(name)
+                continue
+            _f32(g, name)
+            flat = g.view(-1)
+            st = {s: torch.zeros_like(flat) for s in state_names}
+            out = torch.empty_like(flat)
+            bounds = planner.partition_bounds(size_, k)
+            if alg == "onebit_deferred":
+                st["scale_state"] = torch.zeros(max(len(bounds), 1), device=g.device)
+            u = None
+            if alg == "terngrad":
+                if uniform is None or name not in uniform:
+                    raise KeyError(f"terngrad needs uniform[{name!r}]")
+                u = _f32(uniform[name], "uniform", g).view(-1)
+                _same_numel(u, flat, "uniform", name)
+            pays = []
+            for i, (off, length) in enumerate(bounds):
+                pay = torch.zeros(nbytes(length), dtype=torch.uint8, device=g.device)
+                t = {"gradient": flat[off:off + length], "out": out[off:off + length], "compressed": pay}
+                for s in state_names:
+                    t[s] = st[s][off:off + length]
+                if alg == "onebit_deferred":
+                    t["scale_state"] = st["scale_state"][i:i + 1]
+                if u is not None:
+                    t["uniform"] = u[off:off + length]
+                tensors.append(t)
+                pays.append(pay)
+                self.parts.append({"name": name, "index": i, "offset": off, "length": length})
+            self.state[name], self.compressed[name], self.out[name] = st, pays, out
+        self.elements = sum(p["length"] for p in self.parts)
+        self._batch = Batch(alg, tensors, threshold=threshold, bucket=bucket, momentum_factor=momentum_factor,
+                            ratio=ratio) if tensors else None
+
+    def encode(self):
+        if self._batch is not None:
+            self._batch.encode()
+
+    def decode(self):
+        if self._batch is not None:
+            self._batch.decode()
+
+    def close(self):
+        if getattr(self, "_batch", None) is not None:
+            self._batch.close()
+            self._batch = None
 
 
 # ---------------------------------------------------------------- aliases + torch.ops registration

@@ -168,6 +168,42 @@ def read_gradients(path):
     return out
 
 
+def read_plan(path):
+    """Plan lines `name,size,y|n,K` (SeCoPa.py:147) -> [(name, size, compress, partitions)]."""
+    out = []
+    with open(path) as f:
+        for line in f:
+            if line.strip():
+                out.append(parse_plan_line(line))
+    return out
+
+
+def parse_plan_line(line):
+    cols = [c.strip() for c in line.split(",")]
+    if len(cols) != 4 or cols[2] not in ("y", "n") or int(cols[3]) < 1 or int(cols[1]) < 0:
+        raise ValueError(f"not a plan line (name,size,y|n,K): {line.strip()!r}")
+    return str(cols[0]), int(cols[1]), cols[2] == "y", int(cols[3])
+
+
+def partition_bounds(size, parts, align=4):
+    """[(offset, length)] of the K partitions a plan cuts a gradient of `size` elements into.
+
+    The planner prices K equal parts of size / K (SeCoPa.py:52-59); the code that cuts
+    them is not in the reference checkout, so the rule is fixed here: parts of
+    ceil(size / K) elements rounded up to `align` (4 floats = 16 bytes, which keeps every
+    part on the operators' vector path when the gradient is), the last part taking what
+    is left, parts that would be empty dropped."""
+    if size < 0 or parts < 1 or align < 1:
+        raise ValueError("size >= 0, parts >= 1 and align >= 1 are required")
+    step = -(-size // parts)
+    step = -(-step // align) * align
+    out, off = [], 0
+    while off < size:
+        out.append((off, min(step, size - off)))
+        off += step
+    return out
+
+
 # ---------------------------------------------------------------- fitting
 def fit_cost_model(sizes, times):
     """Least-squares line through the measurements that rise above the floor; the floor

@@ -172,3 +172,56 @@ def test_calibration_on_this_gpu_agrees_with_the_committed_models():
     mer = P.calibrate_merge("dgc", npeers=3, sizes=[2 ** 12, 2 ** 22, 2 ** 26], reps=5)
     assert mer["merge"].overhead > 0
     assert 0.5 * data["merge"]["dgc"]["3"]["weight"] <= mer["merge"].weight <= 2.0 * data["merge"]["dgc"]["3"]["weight"]
+
+
+# ---------------------------------------------------------------- plans as the runtime consumes them
+def test_partition_bounds_cover_the_gradient_once():
+    from hipress_amd.planner import partition_bounds
+
+    for size in (0, 1, 3, 4, 7, 64, 1000, 4097, 102760448, (1 << 31) - 1):
+        for parts in (1, 2, 3, 4, 7, 16):
+            b = partition_bounds(size, parts)
+            assert len(b) <= parts
+            assert sum(ln for _, ln in b) == size
+            off = 0
+            for o, ln in b:
+                assert o == off and ln > 0 and o % 4 == 0
+                off += ln
+            if b:
+                assert all(ln == b[0][1] for _, ln in b[:-1]) and b[-1][1] <= b[0][1]
+                assert b[0][1] - size / parts < 4  # equal parts, rounded up to 16 bytes
+    assert partition_bounds(10, 3) == [(0, 4), (4, 4), (8, 2)]
+    assert partition_bounds(7, 16) == [(0, 4), (4, 3)]
+    with pytest.raises(ValueError):
+        partition_bounds(10, 0)
+
+
+def test_plan_lines_round_trip_and_bad_lines_are_named(tmp_path):
+    from hipress_amd.planner import Planner, parse_plan_line, read_gradients, read_plan
+
+    lines = Planner(nodes=4).plan(read_gradients(os.path.join(GOLDEN, "secopa_input.txt")))
+    path = tmp_path / "plan.txt"
+    path.write_text("\n".join(lines) + "\n\n")
+    plan = read_plan(str(path))
+    assert [f"{n},{s},{'y' if c else 'n'},{k}" for n, s, c, k in plan] == lines
+    assert parse_plan_line("w,12,y,3\n") == ("w", 12, True, 3)
+    for bad in ("w,12,maybe,3", "w,12,y", "w,12,y,0", "w,-1,n,1"):
+        with pytest.raises(ValueError, match="not a plan line"):
+            parse_plan_line(bad)
+
+
+def test_planned_set_checks_its_arguments_before_touching_the_gpu():
+    import torch
+
+    import hipress_amd as hp
+
+    g = {"w": torch.zeros(12)}
+    with pytest.raises(KeyError, match="not among the gradients"):
+        hp.PlannedSet("tbq", ["v,12,y,1"], g)
+    with pytest.raises(ValueError, match="no CPU path"):
+        hp.PlannedSet("tbq", ["w,12,y,1"], g)
+    with pytest.raises(ValueError, match="unknown algorithm"):
+        hp.PlannedSet("topk", ["w,12,y,1"], g)
+    ps = hp.PlannedSet("tbq", ["w,12,n,1"], g)  # nothing to compress: no batch, no GPU call
+    assert ps.uncompressed == ["w"] and ps.parts == []
+    ps.encode(), ps.decode(), ps.close()
