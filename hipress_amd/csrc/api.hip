@@ -257,6 +257,9 @@ int finish_terngrad_decode_seg(Seg* s, int64_t payload_bytes, int32_t bucket) {
     return HIPRESS_OK;
 }
 
+// Pairs a sparse encode of this tensor is expected to select: the sample's rank times the stride.
+inline unsigned long long expected_pairs(const Seg& s) { return (unsigned long long)s.ks * s.sstride; }
+
 Launch single_launch(const Seg& s) {
     Launch L;
     std::memset(&L, 0, sizeof L);
@@ -267,6 +270,7 @@ Launch single_launch(const Seg& s) {
     L.seg.ws0 = 0;
     L.ntiles = s.ntiles;
     L.nsegs = 1;
+    L.expect_pairs = expected_pairs(s);
     return L;
 }
 
@@ -336,6 +340,7 @@ struct hipress_batch {
     unsigned ntiles = 0, nstiles = 0, nctiles = 0;
     void* ws = nullptr;  // onebit: one float per tile; sparse: SparseWsLayout
     SparseWsLayout swl{};
+    unsigned long long expect_pairs = 0;  // sparse encode: sum over the tensors
 };
 
 struct hipress_merge_batch {
@@ -355,6 +360,7 @@ struct hipress_merge_batch {
     SparseWsLayout swl{};
     void* iws = nullptr;  // sparse: per tile a head and one run record per peer
     unsigned slices = 1;  // sparse: the largest peer buffer's slots / 1024, rounded up
+    unsigned long long expect_pairs = 0;  // sparse re-encode: sum over the chunks
     std::atomic<unsigned> epoch{0};
     unsigned cur_epoch = 0;
 };
@@ -839,6 +845,7 @@ static int batch_create_impl(hipress_batch** out, int32_t alg, const hipress_ten
     if (enc_ok && sparse) {
         std::vector<uint2> smap;
         int64_t total_ns = layout_samples(b->enc, smap);
+        for (const Seg& s : b->enc) b->expect_pairs += expected_pairs(s);
         b->nstiles = (unsigned)smap.size();
         b->swl = sparse_ws_layout(total_ns, b->ntiles, count);
         if (b->swl.bytes && hipMalloc(&b->ws, (size_t)b->swl.bytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
@@ -889,6 +896,7 @@ static Launch batch_launch(const hipress_batch* b, bool encode) {
     L.nstiles = b->nstiles;
     L.nctiles = b->nctiles;
     L.nsegs = (unsigned)(encode ? b->enc.size() : b->dec.size());
+    L.expect_pairs = b->expect_pairs;
     return L;
 }
 
@@ -1011,6 +1019,7 @@ static int merge_batch_create_impl(hipress_merge_batch** out, int32_t alg, const
         if ((rc = layout_tiles(b->renc, [](Seg& s) -> Seg& { return s; }, map2, &nt2))) return fail(rc);
         std::vector<uint2> smap;
         int64_t total_ns = layout_samples(b->renc, smap);
+        for (const Seg& s : b->renc) b->expect_pairs += expected_pairs(s);
         b->nstiles = (unsigned)smap.size();
         b->swl = sparse_ws_layout(total_ns, b->ntiles, count);
         if (b->swl.bytes && hipMalloc(&b->ws, (size_t)b->swl.bytes) != hipSuccess) return fail(HIPRESS_ERR_HIP);
@@ -1078,6 +1087,7 @@ static int merge_batch_run_impl(hipress_merge_batch* b, int phase, void* stream)
             R.nstiles = b->nstiles;
             R.ntiles = b->ntiles;
             R.nsegs = (unsigned)b->renc.size();
+            R.expect_pairs = b->expect_pairs;
             e = launch_sparse_encode(R, false, ws, kSparseAfterAccum, st);
         }
         return hiperr(e);

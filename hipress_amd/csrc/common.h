@@ -267,6 +267,7 @@ struct Launch {
     unsigned nstiles;     // batch, sparse: sample tiles
     unsigned nctiles;     // batch, sparse decode: payload-slot tiles
     unsigned nsegs;       // tensors in the table (1 for single)
+    unsigned long long expect_pairs;  // sparse encode: pairs the launch is expected to select (ratio x elements)
 };
 
 struct MergeLaunch {
