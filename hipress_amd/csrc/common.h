@@ -182,6 +182,28 @@ __device__ __forceinline__ unsigned xcd_grouped(unsigned b, unsigned nblocks) {
     return b < (nblocks & ~63u) ? ((b & ~63u) | ((b & 7u) << 3) | ((b >> 3) & 7u)) : b;
 }
 
+// Two-pass operators (a reduction over the tensor, then the pass that needs its result) read
+// the same arrays twice.  The second pass walks the launch backwards so that it begins where
+// the first one ended, and it does so in groups of eight so that workgroup b still runs on
+// the XCD that ran workgroup b' = b (mod 8) of the first pass: every XCD has its own L2, and
+// only the lines it fetched itself are in it.  A permutation of [0, nblocks).
+__device__ __forceinline__ unsigned xcd_reversed(unsigned b, unsigned nblocks) {
+    const unsigned groups = nblocks >> 3, g = b >> 3;
+    return g < groups ? (groups - 1 - g) * 8 + (b & 7u) : b;
+}
+// The first pass reads the last tiles of a launch with plain loads so that they stay in L2
+// for the second pass (a streamed load marks its line for early eviction): as many tiles as
+// the eight 4 MiB L2s hold of `streams` fp32 arrays.
+__device__ __forceinline__ bool l2_tail(unsigned b, unsigned nblocks, unsigned streams) {
+    return b + (32u << 20) / (streams * kTile * 4u) >= nblocks;
+}
+// (The empty statement keeps the compiler from folding a branch of such loads into an
+// otherwise identical branch of streamed ones, which would make all of them plain.)
+__device__ __forceinline__ f4 ld4_keep(const float* p) {
+    asm volatile("");
+    return *reinterpret_cast<const f4*>(p);
+}
+
 // ---- cross-lane -------------------------------------------------------------
 // quad_perm broadcast of lane k of every group of four lanes (DPP, no LDS traffic)
 template <int K>

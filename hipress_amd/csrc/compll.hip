@@ -37,11 +37,12 @@ __global__ __launch_bounds__(kBlock) void compll_minmax_kernel(Src src, float* p
     const long long n = (long long)s.n;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
     const bool fast = s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n;
+    const bool keep = fast && l2_tail(blockIdx.x, gridDim.x, 1);  // left in L2 for the quantise pass
     float mx = kMaxInit, mn = kMinInit;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         long long e = base + j * 256 + lane * 4;
-        f4 v = fast ? ld4(s.g + e) : ld4_guard(s.g, e, n);
+        f4 v = keep ? ld4_keep(s.g + e) : (fast ? ld4(s.g + e) : ld4_guard(s.g, e, n));
         unsigned ok = fast ? 0xfu : valid4(e, n);
         if (ok & 1u) { mx = v.x > mx ? v.x : mx; mn = v.x < mn ? v.x : mn; }
         if (ok & 2u) { mx = v.y > mx ? v.y : mx; mn = v.y < mn ? v.y : mn; }
@@ -110,7 +111,7 @@ __device__ __forceinline__ unsigned compll_code(float g, float u, float mn, floa
 template <class Src, int B>
 __global__ __launch_bounds__(kBlock) void compll_quant_kernel(Src src) {
     unsigned tile;
-    const Seg s = src.get(tile, blockIdx.x);
+    const Seg s = src.get(tile, xcd_reversed(blockIdx.x, gridDim.x));  // begins where the min/max pass ended
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long n = (long long)s.n;
     const long long base = (long long)tile * kTile + wave * kWaveTile;

@@ -144,7 +144,8 @@ __device__ __forceinline__ float abs4sum(f4 v) {
 }
 
 // Pass 1: one partial sum of |r+g| per tile, in a fixed order (deterministic).
-template <bool FAST>
+// KEEP: plain loads, for the tiles the quantise pass is to find in L2.
+template <bool FAST, bool KEEP = false>
 __device__ __forceinline__ float onebit_abs_tile(const Seg& s, unsigned tile) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long n = (long long)s.n;
@@ -153,8 +154,8 @@ __device__ __forceinline__ float onebit_abs_tile(const Seg& s, unsigned tile) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         long long e = base + j * 256 + lane * 4;
-        g[j] = load4<FAST>(s.g, e, n);
-        r[j] = load4<FAST>(s.s0, e, n);
+        g[j] = KEEP ? ld4_keep(s.g + e) : load4<FAST>(s.g, e, n);
+        r[j] = KEEP ? ld4_keep(s.s0 + e) : load4<FAST>(s.s0, e, n);
     }
     float a = 0.f;
 #pragma unroll
@@ -168,7 +169,9 @@ __global__ __launch_bounds__(kBlock) void onebit_abs_kernel(Src src, float* part
     unsigned tile;
     const Seg s = src.get(tile, blockIdx.x);
     float a;
-    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) a = onebit_abs_tile<true>(s, tile);
+    const bool whole = s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n;
+    if (whole && l2_tail(blockIdx.x, gridDim.x, 2)) a = onebit_abs_tile<true, true>(s, tile);
+    else if (whole) a = onebit_abs_tile<true>(s, tile);
     else a = onebit_abs_tile<false>(s, tile);
     a = wave_sum(a);
     if ((threadIdx.x & 63u) == 0) wsum[threadIdx.x >> 6] = a;
@@ -255,12 +258,12 @@ __device__ __forceinline__ void onebit_quant_tile(const Seg& s, unsigned tile) {
     if ((lane & 7u) < 4u && (FAST || widx < (long long)((n + 31) >> 5))) words[widx] = myword;
 }
 
-// Tiles are walked from the end of each tensor towards its start: the pass that
-// summed |r+g| finished there, so the most recently read lines are still in cache.
+// The launch is walked from its end towards its start, XCD by XCD: the pass that summed
+// |r+g| finished there and left its last tiles in L2 (xcd_reversed, l2_tail).
 template <class Src>
 __global__ __launch_bounds__(kBlock) void onebit_quant_kernel(Src src) {
     unsigned tile;
-    const Seg s = src.get(tile, gridDim.x - 1 - blockIdx.x);
+    const Seg s = src.get(tile, xcd_reversed(blockIdx.x, gridDim.x));
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) onebit_quant_tile<true>(s, tile);
     else onebit_quant_tile<false>(s, tile);
 }
