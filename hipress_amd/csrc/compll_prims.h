@@ -94,8 +94,11 @@ __global__ void serial_kernel(Args a, Dev* d) {
 // A lane owns four consecutive indices of each of four rows of 256 of its
 // wavefront's 1024.  Fn::stream(a, k), k < Fn::NS, are the float vectors a lambda
 // reads at its own index; they are loaded as 16-byte vectors, whole rows per wavefront.
-template <class Args, class Fn>
-__device__ __forceinline__ void load_streams(const Args& a, long long base, long long count, f4 (&x)[Fn::NS > 0 ? Fn::NS : 1][4]) {
+// KEEP: plain loads, which leave their lines in L2 for the sweep that follows; the others are
+// streamed.  (The empty statement keeps the compiler from folding the two otherwise identical
+// branches into one, which would drop the streaming hint from both.)
+template <class Args, class Fn, bool KEEP>
+__device__ __forceinline__ void load_streams_as(const Args& a, long long base, long long count, f4 (&x)[Fn::NS > 0 ? Fn::NS : 1][4]) {
 #pragma unroll
     for (int k = 0; k < Fn::NS; ++k) {
         const float* p = Fn::stream(a, k);
@@ -104,7 +107,12 @@ __device__ __forceinline__ void load_streams(const Args& a, long long base, long
         for (int j = 0; j < 4; ++j) {
             const long long e = base + j * 256;
             if (e + 3 < count && vec_ok) {
-                x[k][j] = __builtin_nontemporal_load(reinterpret_cast<const f4*>(p + e));
+                if (KEEP) {
+                    asm volatile("");
+                    x[k][j] = *reinterpret_cast<const f4*>(p + e);
+                } else {
+                    x[k][j] = __builtin_nontemporal_load(reinterpret_cast<const f4*>(p + e));
+                }
             } else {
                 x[k][j].x = e < count ? p[e] : 0.f;
                 x[k][j].y = e + 1 < count ? p[e + 1] : 0.f;
@@ -113,6 +121,24 @@ __device__ __forceinline__ void load_streams(const Args& a, long long base, long
             }
         }
     }
+}
+template <class Args, class Fn>
+__device__ __forceinline__ void load_streams(const Args& a, long long base, long long count, f4 (&x)[Fn::NS > 0 ? Fn::NS : 1][4],
+                                             bool keep = false) {
+    if (keep) load_streams_as<Args, Fn, true>(a, base, count, x);
+    else load_streams_as<Args, Fn, false>(a, base, count, x);
+}
+
+// A sweep that follows a reduce over the same vectors walks its tiles backwards, in groups of
+// eight so that workgroup b stays on the XCD (b mod 8) whose L2 holds what workgroup b' = b
+// (mod 8) of the reduce read last; the reduce reads as many of its last tiles with plain
+// loads as the eight 4 MiB L2s hold.
+__device__ __forceinline__ unsigned tile_reversed(unsigned b, unsigned nblocks) {
+    const unsigned groups = nblocks >> 3, g = b >> 3;
+    return g < groups ? (groups - 1 - g) * 8 + (b & 7u) : b;
+}
+__device__ __forceinline__ bool in_l2_tail(unsigned b, unsigned nblocks, unsigned streams) {
+    return b + (32u << 20) / ((streams ? streams : 1u) * (unsigned)kTile * 4u) >= nblocks;
 }
 
 // ---- reduce --------------------------------------------------------------------------------
@@ -135,7 +161,7 @@ __global__ __launch_bounds__(kBlock) void reduce_tiles_kernel(Args a, const Dev*
     const long long n = Src::count(a, *d);
     const long long base = (long long)blockIdx.x * kTile + wave * 1024 + lane * 4;
     f4 in[Src::NS > 0 ? Src::NS : 1][4];
-    load_streams<Args, Src>(a, base, n, in);
+    load_streams<Args, Src>(a, base, n, in, in_l2_tail(blockIdx.x, gridDim.x, Src::NS));
     f4 x[4];
     unsigned ok[4];
 #pragma unroll
@@ -365,7 +391,7 @@ __global__ __launch_bounds__(kBlock) void map_packed_kernel(Args a, Dev* dglobal
     if (!valid_bits(bits)) return;
     const long long count = Fn::count(a, *d);
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const long long base = (long long)blockIdx.x * kTile + wave * 1024 + lane * 4;
+    const long long base = (long long)tile_reversed(blockIdx.x, gridDim.x) * kTile + wave * 1024 + lane * 4;
     if (base - lane * 4 >= count) return;  // the whole wavefront leaves together
     f4 x[Fn::NS > 0 ? Fn::NS : 1][4];
     load_streams<Args, Fn>(a, base, count, x);
@@ -415,7 +441,7 @@ __global__ __launch_bounds__(kBlock) void map_fused_kernel(Args a, Dev* dglobal,
     if (!valid_bits(bits)) return;
     const long long count = Fn::count(a, *d);
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const long long base = (long long)blockIdx.x * kTile + wave * 1024 + lane * 4;
+    const long long base = (long long)tile_reversed(blockIdx.x, gridDim.x) * kTile + wave * 1024 + lane * 4;
     if (base - lane * 4 >= count) return;  // the whole wavefront leaves together
     const bool vec_ok = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
     f4 x[Fn::NS > 0 ? Fn::NS : 1][4];
