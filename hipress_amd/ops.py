@@ -31,7 +31,7 @@ __all__ = [
     "dgc_encode", "dgc_decode", "graddrop_encode", "graddrop_decode",
     "compll_payload_bytes", "compll_decoded_count", "compll_terngrad_encode", "compll_terngrad_decode",
     "onebit_decode_merge", "tbq_decode_merge", "terngrad_decode_merge", "dgc_decode_merge",
-    "graddrop_decode_merge", "Batch", "MergeBatch", "PlannedSet", "ALIASES",
+    "graddrop_decode_merge", "Batch", "MergeBatch", "PlannedSet", "PlannedMerge", "ALIASES",
 ]
 
 
@@ -609,6 +609,70 @@ class PlannedSet:
     def decode(self):
         if self._batch is not None:
             self._batch.decode()
+
+    def close(self):
+        if getattr(self, "_batch", None) is not None:
+            self._batch.close()
+            self._batch = None
+
+class PlannedMerge:
+    """The aggregator's side of a SeCoPa plan on one GPU: for every partition of every
+    gradient the plan marks ``y``, the peers' payloads are decoded and summed in peer order
+    and, with ``reencode=True`` (tbq, dgc, graddrop), the sum is compressed again for the next
+    hop with the aggregator's own residual / accumulator - all partitions of the model in
+    one launch sequence (a ``MergeBatch``).
+
+    ``peers``: one entry per peer, each a dict name -> list of that gradient's partition
+    payloads, as ``PlannedSet.compressed`` of the sending side holds them.  The object
+    allocates and exposes by gradient name ``aggregate[name]`` (the fp32 sum, whole
+    gradient), and with the re-encode ``state[name]`` and ``out_compressed[name]`` (one
+    payload per partition).
+    """
+
+    def __init__(self, alg, plan, peers, reencode=False, threshold=0.0, bucket=512, ratio=0.001):
+        from . import planner
+
+        if alg not in ALG_IDS or alg == "onebit_deferred":
+            raise ValueError(f"no decode-and-merge for algorithm {alg!r}")
+        if reencode and alg not in ("tbq", "dgc", "graddrop"):
+            raise ValueError(f"{alg} has no fused re-encode")
+        if not peers:
+            raise ValueError("at least one peer is needed")
+        nbytes = {"tbq": tbq_payload_bytes, "dgc": lambda n: sparse_payload_bytes(n, ratio),
+                  "graddrop": lambda n: sparse_payload_bytes(n, ratio)}.get(alg)
+        self.alg = alg
+        self.parts, self.uncompressed = [], []
+        self.aggregate, self.state, self.out_compressed = {}, {}, {}
+        chunks = []
+        for entry in plan:
+            name, size_, compress, k = planner.parse_plan_line(entry) if isinstance(entry, str) else entry
+            if not compress:
+                self.uncompressed.append(name)
+                continue
+            bounds = planner.partition_bounds(size_, k)
+            for p, peer in enumerate(peers):
+                if name not in peer or len(peer[name]) != len(bounds):
+                    raise ValueError(f"peer {p} does not hold the {len(bounds)} partition payloads of {name!r}")
+            if not bounds:
+                continue
+            dev = peers[0][name][0].device
+            agg = torch.empty(size_, device=dev)
+            self.aggregate[name] = agg
+            if reencode:
+                self.state[name] = torch.zeros(size_, device=dev)
+                self.out_compressed[name] = [torch.zeros(nbytes(ln), dtype=torch.uint8, device=dev) for _, ln in bounds]
+            for i, (off, ln) in enumerate(bounds):
+                c = {"compressed": [peer[name][i] for peer in peers], "aggregate": agg[off:off + ln]}
+                if reencode:
+                    c["state"] = self.state[name][off:off + ln]
+                    c["out_compressed"] = self.out_compressed[name][i]
+                chunks.append(c)
+                self.parts.append({"name": name, "index": i, "offset": off, "length": ln})
+        self._batch = MergeBatch(alg, chunks, threshold=threshold, bucket=bucket, ratio=ratio) if chunks else None
+
+    def run(self):
+        if self._batch is not None:
+            self._batch.run()
 
     def close(self):
         if getattr(self, "_batch", None) is not None:

@@ -169,3 +169,45 @@ def test_the_measured_vgg19_plan_runs_as_one_batch(hp):
         assert bool(((out == 0) | (out.abs() == 0.05)).all())
         assert torch.equal(r, g[nm].view(-1) - out)
     ps.close()
+
+
+@pytest.mark.parametrize("alg", ["tbq", "dgc"])
+def test_planned_merge_sums_every_partition_in_peer_order_and_reencodes(hp, alg):
+    """Three senders run the plan, the aggregator merges their partition payloads: every
+    partition's sum, re-encoded payload and aggregator state equal the oracle's merge of the
+    same payloads."""
+    kw = {"threshold": 0.05} if alg == "tbq" else {"ratio": 0.01}
+    senders, grads = [], []
+    for p in range(3):
+        g = {k: torch.from_numpy(v).cuda() for k, v in gradients(40 + p).items()}
+        ps = hp.PlannedSet(alg, PLAN, g, **kw)
+        ps.encode()
+        senders.append(ps)
+        grads.append(g)
+    pm = hp.PlannedMerge(alg, PLAN, [s.compressed for s in senders], reencode=True, **kw)
+    assert pm.uncompressed == ["conv_bias"] and len(pm.parts) == len(senders[0].parts)
+    state = {name: np.zeros(n, F) for name, n in SIZES}
+    for step in range(2):
+        pm.run()
+        for part in pm.parts:
+            name, i, off, ln = part["name"], part["index"], part["offset"], part["length"]
+            pays = [host(s.compressed[name][i]) for s in senders]
+            if alg == "tbq":
+                agg, out, r_new = oracle.tbq_decode_merge(pays, ln, state[name][off:off + ln], 0.05)
+            else:
+                agg, out, r_new = oracle.sparse_decode_merge(pays, ln, state[name][off:off + ln], 0.01)
+            state[name][off:off + ln] = r_new
+            np.testing.assert_array_equal(host(pm.aggregate[name])[off:off + ln], agg, err_msg=f"{name}[{i}] step {step}")
+            got = host(pm.out_compressed[name][i])
+            if alg == "tbq":
+                np.testing.assert_array_equal(got, out)
+            else:
+                *hg, ig, vg = oracle.sparse_unpack(got)
+                *hw, iw, vw = oracle.sparse_unpack(out)
+                assert hg == hw
+                np.testing.assert_array_equal(ig, iw)
+                np.testing.assert_array_equal(vg, vw)
+            np.testing.assert_array_equal(host(pm.state[name])[off:off + ln], r_new)
+    pm.close()
+    for s in senders:
+        s.close()

@@ -225,3 +225,17 @@ def test_planned_set_checks_its_arguments_before_touching_the_gpu():
     ps = hp.PlannedSet("tbq", ["w,12,n,1"], g)  # nothing to compress: no batch, no GPU call
     assert ps.uncompressed == ["w"] and ps.parts == []
     ps.encode(), ps.decode(), ps.close()
+
+
+def test_planned_merge_checks_its_arguments_before_touching_the_gpu():
+    import hipress_amd as hp
+
+    with pytest.raises(ValueError, match="at least one peer"):
+        hp.PlannedMerge("tbq", ["w,12,y,1"], [])
+    with pytest.raises(ValueError, match="no fused re-encode"):
+        hp.PlannedMerge("onebit", ["w,12,y,1"], [{}], reencode=True)
+    with pytest.raises(ValueError, match="does not hold the 3 partition payloads"):
+        hp.PlannedMerge("tbq", ["w,12,y,3"], [{"w": []}])
+    pm = hp.PlannedMerge("tbq", ["w,12,n,3"], [{}])  # nothing to merge: no batch, no GPU call
+    assert pm.uncompressed == ["w"] and pm.parts == []
+    pm.run(), pm.close()
