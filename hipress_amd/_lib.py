@@ -39,6 +39,7 @@ class MergeChunk(ctypes.Structure):
     _fields_ = [
         ("payloads", _vp * MAX_PEERS), ("payload_bytes", _i64 * MAX_PEERS),
         ("aggregate", _vp), ("state", _vp), ("out_payload", _vp), ("out_payload_bytes", _i64), ("n", _i64),
+        ("local", _vp),
     ]
 
 
@@ -75,6 +76,10 @@ SIGNATURES = {
     "hipress_onebit_decode_merge": (ctypes.c_int, [_vp, _vp, _i32, _vp, _i64, _vp]),
     "hipress_terngrad_decode_merge": (ctypes.c_int, [_vp, _vp, _i32, _vp, _i64, _vp]),
     "hipress_sparse_decode_merge": (ctypes.c_int, [_vp, _vp, _i32, _vp, _i64, _vp, _vp, _i64, _f64, _vp, _i64, _vp]),
+    "hipress_tbq_decode_merge_local": (ctypes.c_int, [_vp, _vp, _i32, _vp, _vp, _i64, _vp, _vp, _i64, _f32, _vp]),
+    "hipress_onebit_decode_merge_local": (ctypes.c_int, [_vp, _vp, _i32, _vp, _vp, _i64, _vp]),
+    "hipress_terngrad_decode_merge_local": (ctypes.c_int, [_vp, _vp, _i32, _vp, _vp, _i64, _vp]),
+    "hipress_sparse_decode_merge_local": (ctypes.c_int, [_vp, _vp, _i32, _vp, _vp, _i64, _vp, _vp, _i64, _f64, _vp, _i64, _vp]),
     "hipress_batch_create": (ctypes.c_int, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(Tensor), _i32, ctypes.POINTER(Params)]),
     "hipress_batch_encode": (ctypes.c_int, [_vp, _vp]),
     "hipress_batch_decode": (ctypes.c_int, [_vp, _vp]),

@@ -349,6 +349,7 @@ struct hipress_merge_batch {
     int npeers = 0;
     bool reencode = false;
     bool aggregate = false;  // some chunk writes its fp32 sum
+    bool local = false;      // some chunk starts from a local gradient
     std::vector<MergeSeg> segs;
     std::vector<Seg> renc;  // sparse re-encode descriptors
     MergeSeg* d_segs = nullptr;
@@ -367,7 +368,7 @@ struct hipress_merge_batch {
 
 extern "C" {
 
-int hipress_version(void) { return 110; }
+int hipress_version(void) { return 120; }
 
 const char* hipress_strerror(int code) {
     switch (code) {
@@ -647,13 +648,14 @@ int hipress_sparse_decode(const void* payload, int64_t payload_bytes, float* out
 // ---- decode-and-merge ------------------------------------------------------------------
 
 // reencode: the call also re-encodes the sum; only then may the aggregate be left out.
+// local: the aggregator's own uncompressed gradient the sum starts from, or NULL (zero).
 static int build_merge_seg(int alg, const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
-                           float* aggregate, int64_t n, bool reencode, MergeSeg* m) {
+                           const float* local, float* aggregate, int64_t n, bool reencode, MergeSeg* m) {
     std::memset(m, 0, sizeof(MergeSeg));
     if (bad_n(n) || (is_sparse(alg) && bad_sparse_n(n))) return HIPRESS_ERR_SIZE;
     if (npeers < 1 || npeers > HIPRESS_MAX_PEERS) return HIPRESS_ERR_PARAM;
     if (!payloads || !payload_bytes || (n > 0 && !aggregate && !reencode)) return HIPRESS_ERR_NULL;
-    if (mis(aggregate, 4)) return HIPRESS_ERR_ALIGN;
+    if (mis(aggregate, 4) || mis(local, 4)) return HIPRESS_ERR_ALIGN;
     for (int p = 0; p < npeers; ++p) {
         if (!payloads[p]) return HIPRESS_ERR_NULL;
         if (mis(payloads[p], 16)) return HIPRESS_ERR_ALIGN;
@@ -666,10 +668,11 @@ static int build_merge_seg(int alg, const void* const* payloads, const int64_t* 
         int64_t slots = (payload_bytes[p] - HIPRESS_HEADER_BYTES) / 8;
         m->peer_slots[p] = (unsigned)(slots > 0xffffffffLL ? 0xffffffffLL : slots);
     }
+    m->s.g = n > 0 ? local : nullptr;
     m->s.out = aggregate;
     m->s.n = (unsigned long long)n;
     m->s.ntiles = tiles_of(n);
-    m->s.aligned = al16(aggregate);
+    m->s.aligned = al16(aggregate) && al16(local);
     return HIPRESS_OK;
 }
 
@@ -689,6 +692,7 @@ static MergeLaunch single_merge_launch(const MergeSeg& m, int npeers, bool reenc
     L.npeers = npeers;
     L.reencode = reencode;
     L.aggregate = m.s.out != nullptr;
+    L.local = m.s.g != nullptr;
     return L;
 }
 
@@ -707,9 +711,16 @@ static int add_tbq_reencode(MergeSeg* m, float* residual, void* out_payload, int
 int hipress_tbq_decode_merge(const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
                              float* aggregate, int64_t n, float* residual, void* out_payload,
                              int64_t out_payload_bytes, float threshold, void* stream) {
+    return hipress_tbq_decode_merge_local(payloads, payload_bytes, npeers, nullptr, aggregate, n, residual, out_payload,
+                                          out_payload_bytes, threshold, stream);
+}
+
+int hipress_tbq_decode_merge_local(const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
+                                   const float* local, float* aggregate, int64_t n, float* residual, void* out_payload,
+                                   int64_t out_payload_bytes, float threshold, void* stream) {
     MergeSeg m;
     const bool reenc = wants_reencode(residual, out_payload, n);
-    int rc = build_merge_seg(HIPRESS_TBQ, payloads, payload_bytes, npeers, aggregate, n, reenc, &m);
+    int rc = build_merge_seg(HIPRESS_TBQ, payloads, payload_bytes, npeers, local, aggregate, n, reenc, &m);
     if (rc) return rc;
     if (reenc && (rc = add_tbq_reencode(&m, residual, out_payload, out_payload_bytes, threshold))) return rc;
     return hiperr(launch_dense_merge(single_merge_launch(m, npeers, reenc), HIPRESS_TBQ,
@@ -718,8 +729,13 @@ int hipress_tbq_decode_merge(const void* const* payloads, const int64_t* payload
 
 int hipress_onebit_decode_merge(const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
                                 float* aggregate, int64_t n, void* stream) {
+    return hipress_onebit_decode_merge_local(payloads, payload_bytes, npeers, nullptr, aggregate, n, stream);
+}
+
+int hipress_onebit_decode_merge_local(const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
+                                      const float* local, float* aggregate, int64_t n, void* stream) {
     MergeSeg m;
-    int rc = build_merge_seg(HIPRESS_ONEBIT, payloads, payload_bytes, npeers, aggregate, n, false, &m);
+    int rc = build_merge_seg(HIPRESS_ONEBIT, payloads, payload_bytes, npeers, local, aggregate, n, false, &m);
     if (rc) return rc;
     return hiperr(launch_dense_merge(single_merge_launch(m, npeers, false), HIPRESS_ONEBIT,
                                      static_cast<hipStream_t>(stream)));
@@ -727,8 +743,13 @@ int hipress_onebit_decode_merge(const void* const* payloads, const int64_t* payl
 
 int hipress_terngrad_decode_merge(const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
                                   float* aggregate, int64_t n, void* stream) {
+    return hipress_terngrad_decode_merge_local(payloads, payload_bytes, npeers, nullptr, aggregate, n, stream);
+}
+
+int hipress_terngrad_decode_merge_local(const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
+                                        const float* local, float* aggregate, int64_t n, void* stream) {
     MergeSeg m;
-    int rc = build_merge_seg(HIPRESS_TERNGRAD, payloads, payload_bytes, npeers, aggregate, n, false, &m);
+    int rc = build_merge_seg(HIPRESS_TERNGRAD, payloads, payload_bytes, npeers, local, aggregate, n, false, &m);
     if (rc) return rc;
     return hiperr(launch_dense_merge(single_merge_launch(m, npeers, false), HIPRESS_TERNGRAD,
                                      static_cast<hipStream_t>(stream)));
@@ -749,9 +770,17 @@ int hipress_sparse_decode_merge(const void* const* payloads, const int64_t* payl
                                 float* aggregate, int64_t n, float* accumulator, void* out_payload,
                                 int64_t out_payload_bytes, double ratio, void* workspace,
                                 int64_t workspace_bytes, void* stream) {
+    return hipress_sparse_decode_merge_local(payloads, payload_bytes, npeers, nullptr, aggregate, n, accumulator,
+                                             out_payload, out_payload_bytes, ratio, workspace, workspace_bytes, stream);
+}
+
+int hipress_sparse_decode_merge_local(const void* const* payloads, const int64_t* payload_bytes, int32_t npeers,
+                                      const float* local, float* aggregate, int64_t n, float* accumulator,
+                                      void* out_payload, int64_t out_payload_bytes, double ratio, void* workspace,
+                                      int64_t workspace_bytes, void* stream) {
     MergeSeg m;
     const bool reenc = wants_reencode(accumulator, out_payload, n);
-    int rc = build_merge_seg(HIPRESS_DGC, payloads, payload_bytes, npeers, aggregate, n, reenc, &m);
+    int rc = build_merge_seg(HIPRESS_DGC, payloads, payload_bytes, npeers, local, aggregate, n, reenc, &m);
     if (rc) return rc;
     SparseWsLayout l{};
     const int64_t ibytes = merge_index_bytes(m.s.ntiles, npeers);
@@ -998,7 +1027,7 @@ static int merge_batch_create_impl(hipress_merge_batch** out, int32_t alg, const
     for (int i = 0; i < count; ++i) {
         const hipress_merge_chunk& c = chunks[i];
         MergeSeg m;
-        if ((rc = build_merge_seg(alg, c.payloads, c.payload_bytes, npeers, c.aggregate, c.n, b->reencode, &m))) return fail(rc);
+        if ((rc = build_merge_seg(alg, c.payloads, c.payload_bytes, npeers, c.local, c.aggregate, c.n, b->reencode, &m))) return fail(rc);
         if (b->reencode && alg == HIPRESS_TBQ) {
             if ((rc = add_tbq_reencode(&m, c.state, c.out_payload, c.out_payload_bytes, params->threshold))) return fail(rc);
         }
@@ -1009,6 +1038,7 @@ static int merge_batch_create_impl(hipress_merge_batch** out, int32_t alg, const
             b->renc.push_back(s);
         }
         b->aggregate = b->aggregate || m.s.out != nullptr;
+        b->local = b->local || m.s.g != nullptr;
         b->segs.push_back(m);
     }
     std::vector<uint2> map;
@@ -1067,6 +1097,7 @@ static int merge_batch_run_impl(hipress_merge_batch* b, int phase, void* stream)
     L.npeers = b->npeers;
     L.reencode = b->reencode;
     L.aggregate = b->aggregate;
+    L.local = b->local;
     if (b->alg == HIPRESS_DGC || b->alg == HIPRESS_GRADDROP) {
         if (phase > 2) return HIPRESS_ERR_PARAM;
         PeerRun* runs = static_cast<PeerRun*>(b->iws);

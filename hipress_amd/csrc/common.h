@@ -302,6 +302,7 @@ struct MergeLaunch {
     int npeers;
     bool reencode;
     bool aggregate;  // some chunk of the launch writes its fp32 sum
+    bool local;      // some chunk of the launch starts its sum from a local gradient
 };
 
 }  // namespace hp

@@ -27,7 +27,8 @@ __device__ __forceinline__ unsigned tbq_q(float v, float tau, float& keep) {
     return c;
 }
 
-template <bool FAST, int ALG, bool REENC>
+// LOCAL: some chunk of the launch starts its sum from a local gradient (Seg::g).
+template <bool FAST, int ALG, bool REENC, bool LOCAL>
 __device__ __forceinline__ void merge_tile(const MergeSeg& m, unsigned tile, int npeers) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const Seg s = m.s;
@@ -36,7 +37,9 @@ __device__ __forceinline__ void merge_tile(const MergeSeg& m, unsigned tile, int
     f4 agg[4], rpre[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
+        // the sum starts from zero, or from the aggregator's own uncompressed gradient
         agg[j] = (f4){0.f, 0.f, 0.f, 0.f};
+        if (LOCAL && s.g) agg[j] = load4<FAST>(s.g, base + j * 256 + lane * 4, n);
         // the aggregator's residual is requested first: it is in flight while the peers are added
         if (REENC) rpre[j] = load4<FAST>(s.s0, base + j * 256 + lane * 4, n);
     }
@@ -153,7 +156,7 @@ __device__ __forceinline__ void merge_tile(const MergeSeg& m, unsigned tile, int
     }
 }
 
-template <class MSrc, int ALG, bool REENC>
+template <class MSrc, int ALG, bool REENC, bool LOCAL>
 __global__ __launch_bounds__(kBlock) void dense_merge_kernel(MSrc src, int npeers) {
     unsigned tile;
     const MergeSeg& m = src.get(tile, blockIdx.x);
@@ -164,28 +167,32 @@ __global__ __launch_bounds__(kBlock) void dense_merge_kernel(MSrc src, int npeer
         h[2] = 0;
         h[3] = 0;
     }
-    if (m.s.aligned && (unsigned long long)(tile + 1) * kTile <= m.s.n) merge_tile<true, ALG, REENC>(m, tile, npeers);
-    else merge_tile<false, ALG, REENC>(m, tile, npeers);
+    if (m.s.aligned && (unsigned long long)(tile + 1) * kTile <= m.s.n) merge_tile<true, ALG, REENC, LOCAL>(m, tile, npeers);
+    else merge_tile<false, ALG, REENC, LOCAL>(m, tile, npeers);
 }
 
-template <class MSrc>
+template <class MSrc, bool LOCAL>
 static hipError_t dense_merge_src(const MSrc& src, const MergeLaunch& L, int alg, hipStream_t st) {
     dim3 g(L.ntiles), b(kBlock);
     if (alg == HIPRESS_ONEBIT)
-        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_ONEBIT, false>), g, b, 0, st, src, L.npeers);
+        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_ONEBIT, false, LOCAL>), g, b, 0, st, src, L.npeers);
     else if (alg == HIPRESS_TERNGRAD)
-        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TERNGRAD, false>), g, b, 0, st, src, L.npeers);
+        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TERNGRAD, false, LOCAL>), g, b, 0, st, src, L.npeers);
     else if (L.reencode)
-        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TBQ, true>), g, b, 0, st, src, L.npeers);
+        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TBQ, true, LOCAL>), g, b, 0, st, src, L.npeers);
     else
-        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TBQ, false>), g, b, 0, st, src, L.npeers);
+        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TBQ, false, LOCAL>), g, b, 0, st, src, L.npeers);
     return hipGetLastError();
 }
 
 hipError_t launch_dense_merge(const MergeLaunch& L, int alg, hipStream_t st) {
     if (L.ntiles == 0) return hipSuccess;
-    if (L.single) return dense_merge_src(MergeSingleSrc{L.seg}, L, alg, st);
-    return dense_merge_src(MergeBatchSrc{L.dsegs, L.dmap}, L, alg, st);
+    if (L.single) {
+        if (L.local) return dense_merge_src<MergeSingleSrc, true>(MergeSingleSrc{L.seg}, L, alg, st);
+        return dense_merge_src<MergeSingleSrc, false>(MergeSingleSrc{L.seg}, L, alg, st);
+    }
+    if (L.local) return dense_merge_src<MergeBatchSrc, true>(MergeBatchSrc{L.dsegs, L.dmap}, L, alg, st);
+    return dense_merge_src<MergeBatchSrc, false>(MergeBatchSrc{L.dsegs, L.dmap}, L, alg, st);
 }
 
 }  // namespace hp

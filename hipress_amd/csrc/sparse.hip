@@ -1024,7 +1024,7 @@ __global__ __launch_bounds__(kBlock) void sparse_merge_index_kernel(MSegSrc src,
         for (unsigned t = threadIdx.x; t < nt; t += kBlock) rec[t].disorder = epoch;
 }
 
-template <class MSrc, bool REENC>
+template <class MSrc, bool REENC, bool LOCAL>
 __global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs ws, const PeerRun* runs, int npeers,
                                                               unsigned epoch) {
     __shared__ __attribute__((aligned(16))) float lds[kTile];
@@ -1059,7 +1059,14 @@ __global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs
 #pragma unroll
         for (int j = 0; j < 4; ++j) apre[j] = ld4_guard(r.s1, t_lo + wave * kWaveTile + j * 256 + lane * 4, n);
     }
-    for (unsigned i = threadIdx.x; i < kTile; i += kBlock) lds[i] = 0.f;
+    // the sum starts from zero, or from the aggregator's own uncompressed gradient
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const unsigned at = wave * kWaveTile + j * 256 + lane * 4;
+        f4 v = {0.f, 0.f, 0.f, 0.f};
+        if (LOCAL && s.g) v = fast ? ld4(s.g + t_lo + at) : ld4_guard(s.g, t_lo + at, n);
+        *reinterpret_cast<f4*>(&lds[at]) = v;
+    }
     if ((int)threadIdx.x < npeers) {
         if (run.disorder == epoch) {  // this peer's payload was seen out of order: every pair is looked at
             const unsigned nnz = sparse_header(m.peer[threadIdx.x], m.peer_slots[threadIdx.x], run.idx, run.val);
@@ -1234,30 +1241,30 @@ hipError_t launch_sparse_merge(const MergeLaunch& L, const SparseWs& ws, PeerRun
     // buffers allocated chunk by chunk and kind by kind); without the aggregate (one read, one
     // write stream) it is 10 % slower capped, so only the former is.
     const unsigned cap = L.aggregate ? 16u * 1024u : 0u;
+    auto merge_launch = [&](auto src) {
+        using S = decltype(src);
+        dim3 g(L.ntiles), b(kBlock);
+        if (L.reencode && L.local)
+            hipLaunchKernelGGL((sparse_merge_kernel<S, true, true>), g, b, cap, st, src, ws, runs, L.npeers, epoch);
+        else if (L.reencode)
+            hipLaunchKernelGGL((sparse_merge_kernel<S, true, false>), g, b, cap, st, src, ws, runs, L.npeers, epoch);
+        else if (L.local)
+            hipLaunchKernelGGL((sparse_merge_kernel<S, false, true>), g, b, 0, st, src, ws, runs, L.npeers, epoch);
+        else
+            hipLaunchKernelGGL((sparse_merge_kernel<S, false, false>), g, b, 0, st, src, ws, runs, L.npeers, epoch);
+    };
     if (L.single) {
         MergeSingleSegSrc isrc{L.seg};
         if (index)
             hipLaunchKernelGGL((sparse_merge_index_kernel<MergeSingleSegSrc>), dim3(L.npeers, sy, sz), dim3(kBlock), 0, st,
                                isrc, runs, L.npeers, L.ntiles, epoch);
-        MergeSingleSrc src{L.seg};
-        if (merge && L.reencode)
-            hipLaunchKernelGGL((sparse_merge_kernel<MergeSingleSrc, true>), dim3(L.ntiles), dim3(kBlock), cap, st, src, ws,
-                               runs, L.npeers, epoch);
-        else if (merge)
-            hipLaunchKernelGGL((sparse_merge_kernel<MergeSingleSrc, false>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
-                               runs, L.npeers, epoch);
+        if (merge) merge_launch(MergeSingleSrc{L.seg});
     } else {
         MergeBatchSegSrc isrc{L.dsegs};
         if (index)
             hipLaunchKernelGGL((sparse_merge_index_kernel<MergeBatchSegSrc>), dim3(L.nsegs * L.npeers, sy, sz), dim3(kBlock),
                                0, st, isrc, runs, L.npeers, L.ntiles, epoch);
-        MergeBatchSrc src{L.dsegs, L.dmap};
-        if (merge && L.reencode)
-            hipLaunchKernelGGL((sparse_merge_kernel<MergeBatchSrc, true>), dim3(L.ntiles), dim3(kBlock), cap, st, src, ws,
-                               runs, L.npeers, epoch);
-        else if (merge)
-            hipLaunchKernelGGL((sparse_merge_kernel<MergeBatchSrc, false>), dim3(L.ntiles), dim3(kBlock), 0, st, src, ws,
-                               runs, L.npeers, epoch);
+        if (merge) merge_launch(MergeBatchSrc{L.dsegs, L.dmap});
     }
     return hipGetLastError();
 }

@@ -325,10 +325,19 @@ def _peers(compressed_list, like):
     return ptrs, lens, P
 
 
-def tbq_decode_merge(compressed_list, aggregate, residual=None, out_compressed=None, threshold=0.0):
+def _local_of(local, like):
+    """The aggregator's own uncompressed gradient a merge starts from, or None (zero)."""
+    if local is not None:
+        _f32(local, "local", like)
+        _same_numel(like, local, "aggregate", "local")
+    return local
+
+
+def tbq_decode_merge(compressed_list, aggregate, residual=None, out_compressed=None, threshold=0.0, local=None):
     """aggregate = sum of the decoded peers; with `residual` given the aggregate is
     re-encoded into `out_compressed` with the aggregator's own residual, and `aggregate`
-    may then be None (only the re-encoded payload is produced)."""
+    may then be None (only the re-encoded payload is produced).  With `local` (fp32, the
+    aggregator's own gradient) the sum starts from it instead of zero: one hop of a ring."""
     like = aggregate if aggregate is not None else residual
     if like is None:
         raise TypeError("aggregate may only be None when residual and out_compressed are given")
@@ -338,33 +347,37 @@ def tbq_decode_merge(compressed_list, aggregate, residual=None, out_compressed=N
     if residual is not None:
         _f32(residual, "residual", like); _u8(out_compressed, "out_compressed", like)
         _same_numel(like, residual, "aggregate", "residual")
+    _local_of(local, like)
     with _on(like.device):
-        check(_lib.lib().hipress_tbq_decode_merge(
-            ptrs, lens, P, _p(aggregate), like.numel(), _p(residual), _p(out_compressed),
+        check(_lib.lib().hipress_tbq_decode_merge_local(
+            ptrs, lens, P, _p(local), _p(aggregate), like.numel(), _p(residual), _p(out_compressed),
             out_compressed.numel() if out_compressed is not None else 0, float(threshold), _stream(like)),
             "tbq_decode_merge")
 
 
-def onebit_decode_merge(compressed_list, aggregate):
+def onebit_decode_merge(compressed_list, aggregate, local=None):
     _f32(aggregate, "aggregate")
     ptrs, lens, P = _peers(compressed_list, aggregate)
+    _local_of(local, aggregate)
     with _on(aggregate.device):
-        check(_lib.lib().hipress_onebit_decode_merge(ptrs, lens, P, _p(aggregate), aggregate.numel(),
-                                                     _stream(aggregate)), "onebit_decode_merge")
+        check(_lib.lib().hipress_onebit_decode_merge_local(ptrs, lens, P, _p(local), _p(aggregate), aggregate.numel(),
+                                                           _stream(aggregate)), "onebit_decode_merge")
 
 
-def terngrad_decode_merge(compressed_list, aggregate):
+def terngrad_decode_merge(compressed_list, aggregate, local=None):
     _f32(aggregate, "aggregate")
     ptrs, lens, P = _peers(compressed_list, aggregate)
+    _local_of(local, aggregate)
     with _on(aggregate.device):
-        check(_lib.lib().hipress_terngrad_decode_merge(ptrs, lens, P, _p(aggregate), aggregate.numel(),
-                                                       _stream(aggregate)), "terngrad_decode_merge")
+        check(_lib.lib().hipress_terngrad_decode_merge_local(ptrs, lens, P, _p(local), _p(aggregate), aggregate.numel(),
+                                                             _stream(aggregate)), "terngrad_decode_merge")
 
 
-def dgc_decode_merge(compressed_list, aggregate, accumulator=None, out_compressed=None, ratio=0.001):
+def dgc_decode_merge(compressed_list, aggregate, accumulator=None, out_compressed=None, ratio=0.001, local=None):
     """Scatter-add of the peers' (index, value) pairs; with `accumulator` given the
     aggregate is re-sparsified into `out_compressed` (accumulator = aggregator residual),
-    and `aggregate` may then be None (only the re-encoded payload is produced)."""
+    and `aggregate` may then be None (only the re-encoded payload is produced).  With
+    `local` (fp32, the aggregator's own gradient) the sum starts from it instead of zero."""
     like = aggregate if aggregate is not None else accumulator
     if like is None:
         raise TypeError("aggregate may only be None when accumulator and out_compressed are given")
@@ -377,11 +390,12 @@ def dgc_decode_merge(compressed_list, aggregate, accumulator=None, out_compresse
     if accumulator is not None:
         _f32(accumulator, "accumulator", like); _u8(out_compressed, "out_compressed", like)
         _same_numel(like, accumulator, "aggregate", "accumulator")
+    _local_of(local, like)
     with _on(like.device):
         ws = _workspace(like, size(L.hipress_sparse_merge_workspace_bytes(n, P, float(ratio), int(accumulator is not None)),
                                    "sparse_merge_workspace_bytes"))
-        check(L.hipress_sparse_decode_merge(
-            ptrs, lens, P, _p(aggregate), n, _p(accumulator), _p(out_compressed),
+        check(L.hipress_sparse_decode_merge_local(
+            ptrs, lens, P, _p(local), _p(aggregate), n, _p(accumulator), _p(out_compressed),
             out_compressed.numel() if out_compressed is not None else 0, float(ratio),
             _p(ws), ws.numel() if ws is not None else 0, _stream(like)), "sparse_decode_merge")
 
@@ -465,7 +479,9 @@ class MergeBatch:
     ``aggregate``, and optionally ``state`` + ``out_compressed`` for the fused
     re-encode (tbq: aggregator residual; dgc/graddrop: aggregator accumulator).
     With the re-encode a chunk's ``aggregate`` may be None: the sum is then not
-    written as fp32, only the re-encoded payload and the state are produced.
+    written as fp32, only the re-encoded payload and the state are produced.  A chunk's
+    ``local`` (fp32, the aggregator's own gradient for that chunk) makes its sum start
+    from there instead of zero.
     """
 
     def __init__(self, alg, chunks, threshold=0.0, bucket=512, ratio=0.001):
@@ -493,6 +509,8 @@ class MergeBatch:
             if st is not None:
                 _f32(st, "state", like); _u8(oc, "out_compressed", like)
                 mc.state, mc.out_payload, mc.out_payload_bytes = st.data_ptr(), oc.data_ptr(), oc.numel()
+            loc = _local_of(c.get("local"), like)
+            mc.local = loc.data_ptr() if loc is not None else None
             mc.n = like.numel()
             arr[i] = mc
         self.device = dev
@@ -626,10 +644,11 @@ class PlannedMerge:
     payloads, as ``PlannedSet.compressed`` of the sending side holds them.  The object
     allocates and exposes by gradient name ``aggregate[name]`` (the fp32 sum, whole
     gradient), and with the re-encode ``state[name]`` and ``out_compressed[name]`` (one
-    payload per partition).
+    payload per partition).  ``local``: dict name -> the aggregator's own uncompressed
+    gradient; the sums of those gradients start from it instead of zero.
     """
 
-    def __init__(self, alg, plan, peers, reencode=False, threshold=0.0, bucket=512, ratio=0.001):
+    def __init__(self, alg, plan, peers, reencode=False, local=None, threshold=0.0, bucket=512, ratio=0.001):
         from . import planner
 
         if alg not in ALG_IDS or alg == "onebit_deferred":
@@ -661,8 +680,14 @@ class PlannedMerge:
             if reencode:
                 self.state[name] = torch.zeros(size_, device=dev)
                 self.out_compressed[name] = [torch.zeros(nbytes(ln), dtype=torch.uint8, device=dev) for _, ln in bounds]
+            mine = None
+            if local is not None and name in local:
+                mine = _f32(local[name], "local").view(-1)
+                _same_numel(agg, mine, name, "local")
             for i, (off, ln) in enumerate(bounds):
                 c = {"compressed": [peer[name][i] for peer in peers], "aggregate": agg[off:off + ln]}
+                if mine is not None:
+                    c["local"] = mine[off:off + ln]
                 if reencode:
                     c["state"] = self.state[name][off:off + ln]
                     c["out_compressed"] = self.out_compressed[name][i]
@@ -714,14 +739,14 @@ _SCHEMAS = {
     "compll_terngrad_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
     "TernGradEncode": "(Tensor gradient, Tensor(a!) compressed, int bitwidth=2, Tensor? uniform=None) -> ()",
     "TernGradDecode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
-    "onebit_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate) -> ()",
-    "terngrad_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate) -> ()",
+    "onebit_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate, Tensor? local=None) -> ()",
+    "terngrad_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate, Tensor? local=None) -> ()",
     "tbq_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate, Tensor(b!)? residual=None, "
-                        "Tensor(c!)? out_compressed=None, float threshold=0.0) -> ()",
+                        "Tensor(c!)? out_compressed=None, float threshold=0.0, Tensor? local=None) -> ()",
     "dgc_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate, Tensor(b!)? accumulator=None, "
-                        "Tensor(c!)? out_compressed=None, float ratio=0.001) -> ()",
+                        "Tensor(c!)? out_compressed=None, float ratio=0.001, Tensor? local=None) -> ()",
     "graddrop_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate, Tensor(b!)? accumulator=None, "
-                             "Tensor(c!)? out_compressed=None, float ratio=0.01) -> ()",
+                             "Tensor(c!)? out_compressed=None, float ratio=0.01, Tensor? local=None) -> ()",
 }
 _ALIAS_OF = {
     "OnebitEncode": "onebit_encode", "OnebitDecode": "onebit_decode", "TBQEncode": "tbq_encode",

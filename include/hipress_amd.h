@@ -208,6 +208,28 @@ int hipress_sparse_decode_merge(const void *const *payloads, const int64_t *payl
                                 void *out_payload, int64_t out_payload_bytes, double ratio,
                                 void *workspace, int64_t workspace_bytes, void *stream);
 
+/* The same merges starting from the aggregator's own uncompressed gradient instead of
+ * zero: aggregate[i] = ((local[i] + d_1[i]) + d_2[i]) + ..., peers added in order.  One
+ * hop of a ring (the payload that arrived, the local gradient, the re-encoded payload to
+ * send on), or a server that is also a worker and need not compress its own share.
+ * local = NULL is the plain merge; aggregate may be the same buffer as local.  No
+ * counterpart in the reference checkout (CaSync's sources are not part of it). */
+int hipress_tbq_decode_merge_local(const void *const *payloads, const int64_t *payload_bytes,
+                                   int32_t npeers, const float *local, float *aggregate, int64_t n,
+                                   float *residual, void *out_payload, int64_t out_payload_bytes,
+                                   float threshold, void *stream);
+int hipress_onebit_decode_merge_local(const void *const *payloads, const int64_t *payload_bytes,
+                                      int32_t npeers, const float *local, float *aggregate,
+                                      int64_t n, void *stream);
+int hipress_terngrad_decode_merge_local(const void *const *payloads, const int64_t *payload_bytes,
+                                        int32_t npeers, const float *local, float *aggregate,
+                                        int64_t n, void *stream);
+int hipress_sparse_decode_merge_local(const void *const *payloads, const int64_t *payload_bytes,
+                                      int32_t npeers, const float *local, float *aggregate,
+                                      int64_t n, float *accumulator, void *out_payload,
+                                      int64_t out_payload_bytes, double ratio, void *workspace,
+                                      int64_t workspace_bytes, void *stream);
+
 /* ---- batched launches over a whole gradient set ---------------------------- */
 /* A training step compresses every tensor of the model; a batch object holds a
  * device-resident table of the tensors so that one launch sequence covers all of
@@ -264,6 +286,7 @@ typedef struct hipress_merge_chunk {
     void *out_payload;   /* re-encoded payload when state != NULL */
     int64_t out_payload_bytes;
     int64_t n;
+    const float *local;  /* fp32[n] the sum starts from (the aggregator's own gradient), or NULL */
 } hipress_merge_chunk;
 
 typedef struct hipress_merge_batch hipress_merge_batch;

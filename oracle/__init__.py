@@ -81,6 +81,10 @@ _SIG = {
     "hpo_onebit_decode_merge": (None, [_ptr, ctypes.c_int, _ptr, _i64]),
     "hpo_terngrad_decode_merge": (None, [_ptr, ctypes.c_int, _ptr, _i64]),
     "hpo_sparse_decode_merge": (None, [_ptr, ctypes.c_int, _ptr, _i64, _ptr, _ptr, _f64]),
+    "hpo_tbq_decode_merge_local": (None, [_ptr, ctypes.c_int, _ptr, _ptr, _i64, _ptr, _ptr, _f32]),
+    "hpo_onebit_decode_merge_local": (None, [_ptr, ctypes.c_int, _ptr, _ptr, _i64]),
+    "hpo_terngrad_decode_merge_local": (None, [_ptr, ctypes.c_int, _ptr, _ptr, _i64]),
+    "hpo_sparse_decode_merge_local": (None, [_ptr, ctypes.c_int, _ptr, _ptr, _i64, _ptr, _ptr, _f64]),
     "hpo_compll_decode": (_i64, [_ptr, _i64, _ptr, _i64]),
     "hpo_compll_payload_bytes": (_i64, [_i64, ctypes.c_int]),
     "hpo_compll_encode": (_i64, [_ptr, _ptr, _i64, _ptr, ctypes.c_int]),
@@ -263,43 +267,56 @@ def sparse_unpack(payload):
 
 
 # -- decode-and-merge ----------------------------------------------------------
-def tbq_decode_merge(payloads, n, r=None, tau=0.0):
+def _local(local, n):
+    """The aggregator's own uncompressed gradient the sum starts from, or None (zero)."""
+    if local is None:
+        return None, None
+    local = _f32c(local)
+    assert local.size == n
+    return local, _p(local)
+
+
+def tbq_decode_merge(payloads, n, r=None, tau=0.0, local=None):
     """-> aggregate, or (aggregate, out_payload, residual') when r is given."""
     keep, arr = _peer_array(payloads)
     agg = np.empty(n, dtype=np.float32)
+    local, lp = _local(local, n)
     if r is None:
-        lib().hpo_tbq_decode_merge(arr, len(keep), _p(agg), n, None, None, tau)
+        lib().hpo_tbq_decode_merge_local(arr, len(keep), lp, _p(agg), n, None, None, tau)
         return agg
     r = _f32c(r).copy()
     out = _payload(tbq_payload_bytes(n))
-    lib().hpo_tbq_decode_merge(arr, len(keep), _p(agg), n, _p(r), _p(out), tau)
+    lib().hpo_tbq_decode_merge_local(arr, len(keep), lp, _p(agg), n, _p(r), _p(out), tau)
     return agg, out, r
 
 
-def onebit_decode_merge(payloads, n):
+def onebit_decode_merge(payloads, n, local=None):
     keep, arr = _peer_array(payloads)
     agg = np.empty(n, dtype=np.float32)
-    lib().hpo_onebit_decode_merge(arr, len(keep), _p(agg), n)
+    local, lp = _local(local, n)
+    lib().hpo_onebit_decode_merge_local(arr, len(keep), lp, _p(agg), n)
     return agg
 
 
-def terngrad_decode_merge(payloads, n):
+def terngrad_decode_merge(payloads, n, local=None):
     keep, arr = _peer_array(payloads)
     agg = np.empty(n, dtype=np.float32)
-    lib().hpo_terngrad_decode_merge(arr, len(keep), _p(agg), n)
+    local, lp = _local(local, n)
+    lib().hpo_terngrad_decode_merge_local(arr, len(keep), lp, _p(agg), n)
     return agg
 
 
-def sparse_decode_merge(payloads, n, acc=None, ratio=0.0):
+def sparse_decode_merge(payloads, n, acc=None, ratio=0.0, local=None):
     """-> aggregate, or (aggregate, out_payload, acc') when acc is given."""
     keep, arr = _peer_array(payloads)
     agg = np.empty(n, dtype=np.float32)
+    local, lp = _local(local, n)
     if acc is None:
-        lib().hpo_sparse_decode_merge(arr, len(keep), _p(agg), n, None, None, ratio)
+        lib().hpo_sparse_decode_merge_local(arr, len(keep), lp, _p(agg), n, None, None, ratio)
         return agg
     acc = _f32c(acc).copy()
     out = _payload(sparse_payload_bytes(n, ratio))
-    lib().hpo_sparse_decode_merge(arr, len(keep), _p(agg), n, _p(acc), _p(out), ratio)
+    lib().hpo_sparse_decode_merge_local(arr, len(keep), lp, _p(agg), n, _p(acc), _p(out), ratio)
     return agg, out, acc
 
 

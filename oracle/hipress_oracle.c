@@ -479,14 +479,22 @@ void hpo_sparse_decode(const uint8_t *payload, float *out, int64_t n)
 /* decode-and-merge                                                   */
 /* ------------------------------------------------------------------ */
 
-/* agg[i] = ((0 + d_1[i]) + d_2[i]) + ... in peer order, binary32.  If r is
- * not NULL the aggregate is re-encoded for the next hop with the
- * aggregator's own residual r and threshold tau into out_payload. */
-void hpo_tbq_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n, float *r,
-                          uint8_t *out_payload, float tau)
+/* The aggregate starts from zero, or from the aggregator's own uncompressed
+ * gradient `local` (a ring hop, a server that is also a worker); the peers are
+ * then added to it in peer order.  agg may be the same buffer as local. */
+static void merge_start(float *agg, const float *local, int64_t n)
 {
     HPO_PARALLEL_FOR
-    for (int64_t i = 0; i < n; ++i) agg[i] = 0.0f;
+    for (int64_t i = 0; i < n; ++i) agg[i] = local ? local[i] : 0.0f;
+}
+
+/* agg[i] = ((start + d_1[i]) + d_2[i]) + ... in peer order, binary32, start = 0
+ * or local[i].  If r is not NULL the aggregate is re-encoded for the next hop
+ * with the aggregator's own residual r and threshold tau into out_payload. */
+void hpo_tbq_decode_merge_local(const uint8_t *const *payloads, int npeers, const float *local, float *agg,
+                                int64_t n, float *r, uint8_t *out_payload, float tau)
+{
+    merge_start(agg, local, n);
     for (int p = 0; p < npeers; ++p) {
         float t;
         const uint32_t *w = (const uint32_t *)(payloads[p] + HPO_HEADER_BYTES);
@@ -497,10 +505,16 @@ void hpo_tbq_decode_merge(const uint8_t *const *payloads, int npeers, float *agg
     if (r) hpo_tbq_encode(agg, r, n, out_payload, tau);
 }
 
-void hpo_onebit_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n)
+void hpo_tbq_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n, float *r,
+                          uint8_t *out_payload, float tau)
 {
-    HPO_PARALLEL_FOR
-    for (int64_t i = 0; i < n; ++i) agg[i] = 0.0f;
+    hpo_tbq_decode_merge_local(payloads, npeers, NULL, agg, n, r, out_payload, tau);
+}
+
+void hpo_onebit_decode_merge_local(const uint8_t *const *payloads, int npeers, const float *local, float *agg,
+                                   int64_t n)
+{
+    merge_start(agg, local, n);
     for (int p = 0; p < npeers; ++p) {
         float s;
         const uint32_t *w = (const uint32_t *)(payloads[p] + HPO_HEADER_BYTES);
@@ -510,10 +524,15 @@ void hpo_onebit_decode_merge(const uint8_t *const *payloads, int npeers, float *
     }
 }
 
-void hpo_terngrad_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n)
+void hpo_onebit_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n)
 {
-    HPO_PARALLEL_FOR
-    for (int64_t i = 0; i < n; ++i) agg[i] = 0.0f;
+    hpo_onebit_decode_merge_local(payloads, npeers, NULL, agg, n);
+}
+
+void hpo_terngrad_decode_merge_local(const uint8_t *const *payloads, int npeers, const float *local, float *agg,
+                                     int64_t n)
+{
+    merge_start(agg, local, n);
     for (int p = 0; p < npeers; ++p) {
         const uint32_t *hdr = (const uint32_t *)payloads[p];
         int64_t bucket = hdr[1];
@@ -526,15 +545,19 @@ void hpo_terngrad_decode_merge(const uint8_t *const *payloads, int npeers, float
     }
 }
 
-/* Zero-fill, then scatter-ADD every peer's pairs in peer order and slot
- * order (duplicates across peers sum).  If acc is not NULL the aggregate is
- * re-sparsified for the next hop GradDrop-style with the aggregator's
- * residual acc: acc' = acc + agg, select, zero. */
-void hpo_sparse_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n,
-                             float *acc, uint8_t *out_payload, double ratio)
+void hpo_terngrad_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n)
 {
-    HPO_PARALLEL_FOR
-    for (int64_t i = 0; i < n; ++i) agg[i] = 0.0f;
+    hpo_terngrad_decode_merge_local(payloads, npeers, NULL, agg, n);
+}
+
+/* Start from zero or from `local`, then scatter-ADD every peer's pairs in peer
+ * order and slot order (duplicates across peers sum).  If acc is not NULL the
+ * aggregate is re-sparsified for the next hop GradDrop-style with the
+ * aggregator's residual acc: acc' = acc + agg, select, zero. */
+void hpo_sparse_decode_merge_local(const uint8_t *const *payloads, int npeers, const float *local, float *agg,
+                                   int64_t n, float *acc, uint8_t *out_payload, double ratio)
+{
+    merge_start(agg, local, n);
     for (int p = 0; p < npeers; ++p) {
         const uint32_t *hdr = (const uint32_t *)payloads[p];
         int64_t nnz = hdr[0], cap = hdr[2];
@@ -545,6 +568,12 @@ void hpo_sparse_decode_merge(const uint8_t *const *payloads, int npeers, float *
             if (idx[j] >= 0 && idx[j] < n) agg[idx[j]] = agg[idx[j]] + val[j];
     }
     if (acc) hpo_graddrop_encode(agg, acc, n, out_payload, ratio);
+}
+
+void hpo_sparse_decode_merge(const uint8_t *const *payloads, int npeers, float *agg, int64_t n,
+                             float *acc, uint8_t *out_payload, double ratio)
+{
+    hpo_sparse_decode_merge_local(payloads, npeers, NULL, agg, n, acc, out_payload, ratio);
 }
 
 /* ------------------------------------------------------------------ */

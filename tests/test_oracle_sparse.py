@@ -229,3 +229,43 @@ def test_sparse_merge_scatter_add_with_duplicates():
     want_pay, want_acc = oracle.graddrop_encode(agg, acc0, ratio)
     np.testing.assert_array_equal(out, want_pay)
     np.testing.assert_array_equal(acc, want_acc)
+
+
+def test_merges_that_start_from_a_local_gradient():
+    """A ring hop / a server that is also a worker: the sum starts from the aggregator's own
+    uncompressed gradient, the peers are added to it in peer order; independent restatement
+    with numpy float32 adds, element for element, and the re-encode sees that sum."""
+    n, P, tau, ratio = 7001, 3, F(0.05), 0.01
+    rng = np.random.default_rng(21)
+    local = rng.normal(0, 0.03, n).astype(F)
+    local[:4] = [0.0, -0.0, np.inf, 1e-40]
+    tb = [oracle.tbq_encode(rng.normal(0, 0.04, n).astype(F), np.zeros(n, F), tau)[0] for _ in range(P)]
+    ob = [oracle.onebit_encode(rng.normal(0, 1, n).astype(F), np.zeros(n, F))[0] for _ in range(P)]
+    tg = [oracle.terngrad_encode(rng.normal(0, 1, n).astype(F), rng.random(n, dtype=F), 512) for _ in range(P)]
+    sp = [oracle.graddrop_encode(rng.normal(0, 1e-3, n).astype(F), np.zeros(n, F), ratio)[0] for _ in range(P)]
+    for pays, dec, mrg in ((tb, oracle.tbq_decode, oracle.tbq_decode_merge), (ob, oracle.onebit_decode, oracle.onebit_decode_merge),
+                           (tg, oracle.terngrad_decode, oracle.terngrad_decode_merge),
+                           (sp, oracle.sparse_decode, oracle.sparse_decode_merge)):
+        seq = local.copy()
+        for p in pays:
+            d = dec(p, n)
+            if mrg is oracle.sparse_decode_merge:  # only the listed elements are touched: -0 and NaN patterns survive elsewhere
+                idx = oracle.sparse_unpack(p)[4]
+                seq[idx] = (seq[idx] + d[idx]).astype(F)
+            else:
+                seq = (seq + d).astype(F)
+        got = mrg(pays, n, local=local)
+        np.testing.assert_array_equal(got.view(np.uint32), seq.view(np.uint32))
+        # without a local gradient the start is +0
+        np.testing.assert_array_equal(mrg(pays, n, local=np.zeros(n, F)), mrg(pays, n))
+    r0 = rng.normal(0, 0.01, n).astype(F)
+    agg, out, r = oracle.tbq_decode_merge(tb, n, r0, tau, local=local)
+    finite = np.isfinite(agg)
+    want_pay, want_r = oracle.tbq_encode(agg, r0, tau)
+    np.testing.assert_array_equal(out, want_pay)
+    np.testing.assert_array_equal(r[finite], want_r[finite])
+    loc2 = np.where(np.isfinite(local), local, 0).astype(F)
+    agg, out, acc = oracle.sparse_decode_merge(sp, n, r0, ratio, local=loc2)
+    want_pay, want_acc = oracle.graddrop_encode(agg, r0, ratio)
+    np.testing.assert_array_equal(out, want_pay)
+    np.testing.assert_array_equal(acc, want_acc)
