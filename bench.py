@@ -265,14 +265,15 @@ class MergeWorkload:
     """Decode-and-merge of 8 peer payloads per 4 MB chunk of the VGG19 set, with the
     fused re-encode for the next hop."""
 
-    def __init__(self, name, alg, sizes, npeers=8, aggregate=True):
+    def __init__(self, name, alg, sizes, npeers=8, aggregate=True, local=False):
         self.name, self.alg, self.sizes, self.npeers = name, alg, sizes, npeers
         self.aggregate = aggregate  # False: only the re-encoded payload is produced (no fp32 sum written)
+        self.local = local          # True: every sum starts from the aggregator's own fp32 gradient (a ring hop)
         self.elements = sum(sizes)
         self.dominant_phase = 0
         self.nphases = 1
         self.rotate = 1
-        agg_bytes = 4.0 if aggregate else 0.0
+        agg_bytes = (4.0 if aggregate else 0.0) + (4.0 if local else 0.0)
         if alg == "tbq":
             self.enc_bytes, self.dec_bytes = 0.25 * npeers + agg_bytes + 8.25, 0.0
             self.dominant_kernel, self.dominant_bytes = "dense_merge_kernel", self.enc_bytes
@@ -295,6 +296,9 @@ class MergeWorkload:
                            "aggregate": torch.empty(n, device=dev) if self.aggregate else None,
                            "state": torch.zeros(n, device=dev),
                            "out_compressed": torch.zeros(nb, dtype=torch.uint8, device=dev)})
+        if self.local:
+            for c, g in zip(chunks, W.normal_set(self.sizes, dev, 0, sigma=0.02 if self.alg == "tbq" else 1e-3)):
+                c["local"] = g
         # peer p's payloads come from that peer's own gradients (seed p) through the encoders
         for p in range(self.npeers):
             if self.alg == "tbq":
@@ -342,16 +346,18 @@ class MergeWorkload:
             n = self.sizes[i]
             pays = [p.cpu().numpy() for p in self.chunks[i]["compressed"]]
             arr = (ctypes.c_void_p * P)(*[p.ctypes.data for p in pays])
+            loc = self.chunks[i]["local"].cpu().numpy() if self.local else None
             jobs.append((n, pays, arr, np.empty(n, np.float32), np.zeros(n, np.float32),
-                         np.zeros(self.chunks[i]["out_compressed"].numel(), np.uint8)))
+                         np.zeros(self.chunks[i]["out_compressed"].numel(), np.uint8), loc))
         total = sum(j[0] for j in jobs)
 
         def run(L):
-            for n, _, arr, agg, state, outp in jobs:
+            for n, _, arr, agg, state, outp, loc in jobs:
+                lp = _vp(loc) if loc is not None else None
                 if alg == "tbq":
-                    L.hpo_tbq_decode_merge(arr, P, _vp(agg), n, _vp(state), _vp(outp), 0.05)
+                    L.hpo_tbq_decode_merge_local(arr, P, lp, _vp(agg), n, _vp(state), _vp(outp), 0.05)
                 else:
-                    L.hpo_sparse_decode_merge(arr, P, _vp(agg), n, _vp(state), _vp(outp), ratio)
+                    L.hpo_sparse_decode_merge_local(arr, P, lp, _vp(agg), n, _vp(state), _vp(outp), ratio)
 
         what = (f"{alg} decode-and-merge of {P} peers + re-encode over the {len(jobs)} largest of "
                 f"{len(self.sizes)} chunks ({total:,} elements per pass)")
@@ -520,6 +526,8 @@ def make_workload(name):
         return MergeWorkload(name, "tbq", W.chunk_sizes(vgg), aggregate=False)
     if name == "merge_dgc_vgg19_payload_only":
         return MergeWorkload(name, "dgc", W.chunk_sizes(vgg), aggregate=False)
+    if name == "hop_tbq_vgg19":  # one hop of a ring: the payload that arrived + the node's own gradient -> the payload to send on
+        return MergeWorkload(name, "tbq", W.chunk_sizes(vgg), npeers=1, aggregate=False, local=True)
     raise SystemExit(f"unknown workload {name}")
 
 
@@ -528,7 +536,7 @@ ALL_WORKLOADS = [
     "tbq_vgg19", "dgc_vgg19", "onebit_vgg19", "terngrad_vgg19", "graddrop_vgg19", "onebit_deferred_vgg19",
     "tbq_262144", "tbq_262144_x512", "terngrad_resnet50", "dgc_bert_large", "graddrop_bert_large",
     "merge_tbq_vgg19", "merge_dgc_vgg19", "compll_b2_fc6", "compll_generated_b2_fc6", "tbq_fc6", "tbq_generated_fc6",
-    "merge_tbq_vgg19_payload_only", "merge_dgc_vgg19_payload_only", "tbq_vgg19_planned",
+    "merge_tbq_vgg19_payload_only", "merge_dgc_vgg19_payload_only", "tbq_vgg19_planned", "hop_tbq_vgg19",
 ]
 # any workload with the suffix _graph: the same step captured once into a HIP graph and replayed
 EXTRA_WORKLOADS = [w + "_graph" for w in ALL_WORKLOADS]
