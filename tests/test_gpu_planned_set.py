@@ -211,3 +211,26 @@ def test_planned_merge_sums_every_partition_in_peer_order_and_reencodes(hp, alg)
     pm.close()
     for s in senders:
         s.close()
+
+
+def test_planned_merge_with_the_aggregators_own_gradient(hp):
+    """A co-located server: two senders' payloads plus its own uncompressed gradients, partition by partition."""
+    senders = []
+    for p in range(2):
+        ps = hp.PlannedSet("tbq", PLAN, {k: torch.from_numpy(v).cuda() for k, v in gradients(60 + p).items()}, threshold=0.05)
+        ps.encode()
+        senders.append(ps)
+    mine = gradients(70)
+    pm = hp.PlannedMerge("tbq", PLAN, [s.compressed for s in senders], reencode=True, threshold=0.05,
+                         local={k: torch.from_numpy(v).cuda() for k, v in mine.items()})
+    pm.run()
+    for part in pm.parts:
+        name, i, off, ln = part["name"], part["index"], part["offset"], part["length"]
+        pays = [host(s.compressed[name][i]) for s in senders]
+        agg, out, r_new = oracle.tbq_decode_merge(pays, ln, np.zeros(ln, F), 0.05, local=mine[name][off:off + ln])
+        np.testing.assert_array_equal(host(pm.aggregate[name])[off:off + ln], agg)
+        np.testing.assert_array_equal(host(pm.out_compressed[name][i]), out)
+        np.testing.assert_array_equal(host(pm.state[name])[off:off + ln], r_new)
+    pm.close()
+    for s in senders:
+        s.close()
