@@ -172,6 +172,15 @@ __device__ __forceinline__ unsigned valid4(long long e, long long n) {
     return left >= 4 ? 0xfu : (left <= 0 ? 0u : ((1u << left) - 1u));
 }
 
+// ---- occupancy --------------------------------------------------------------------
+// The plain streaming kernels move most bytes with four wavefronts per SIMD, not with the
+// eight their few registers would allow.  Naming a high register as clobbered makes the
+// kernel claim 104 of the 512 vector registers of a SIMD lane, which is that limit; set
+// this way it is worth about 1 % over the same limit set with idle LDS at launch (TBQ
+// encode 270 -> 266 us on the VGG19 set), which the kernels that do better with five
+// workgroups per CU, or with a limit that depends on the launch's size, still use.
+__device__ __forceinline__ void four_waves_per_simd() { asm volatile("" ::: "v103"); }
+
 // ---- workgroup -> tile order ----------------------------------------------------
 // Consecutive workgroup ids are dealt to the eight XCDs in turn, so with the plain
 // order every XCD (and its L2) writes every eighth 16 KiB tile.  Kernels that mostly

@@ -79,6 +79,7 @@ __device__ __forceinline__ void tbq_encode_tile(const Seg& s, unsigned tile) {
 
 template <class Src>
 __global__ __launch_bounds__(kBlock) void tbq_encode_kernel(Src src) {
+    four_waves_per_simd();
     unsigned tile;
     const Seg s = src.get(tile, blockIdx.x);
     if (tile == 0 && threadIdx.x == 0) {
@@ -165,6 +166,7 @@ __device__ __forceinline__ float onebit_abs_tile(const Seg& s, unsigned tile) {
 
 template <class Src>
 __global__ __launch_bounds__(kBlock) void onebit_abs_kernel(Src src, float* partial) {
+    four_waves_per_simd();
     __shared__ float wsum[4];
     unsigned tile;
     const Seg s = src.get(tile, blockIdx.x);
@@ -262,6 +264,7 @@ __device__ __forceinline__ void onebit_quant_tile(const Seg& s, unsigned tile) {
 // |r+g| finished there and left its last tiles in L2 (xcd_reversed, l2_tail).
 template <class Src>
 __global__ __launch_bounds__(kBlock) void onebit_quant_kernel(Src src) {
+    four_waves_per_simd();
     unsigned tile;
     const Seg s = src.get(tile, xcd_reversed(blockIdx.x, gridDim.x));
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) onebit_quant_tile<true>(s, tile);
@@ -644,7 +647,7 @@ static unsigned decode_cap(const Launch& L, unsigned per_tile) {
     return (unsigned long long)L.ntiles * per_tile <= (192ull << 20) ? kLdsFor5 : 0u;
 }
 
-hipError_t launch_tbq_encode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_encode_kernel, kLdsFor5, L, st); }
+hipError_t launch_tbq_encode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_encode_kernel, 0u, L, st); }
 hipError_t launch_tbq_decode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_decode_kernel, decode_cap(L, kTile / 4), L, st); }
 hipError_t launch_onebit_decode(const Launch& L, hipStream_t st) {
     HP_LAUNCH(onebit_decode_kernel, decode_cap(L, kTile / 8), L, st);
@@ -656,9 +659,9 @@ hipError_t launch_terngrad_decode(const Launch& L, hipStream_t st) {
 }
 
 static hipError_t onebit_abs(const Launch& L, float* partial, hipStream_t st) {
-    HP_LAUNCH(onebit_abs_kernel, kLdsFor4, L, st, partial);
+    HP_LAUNCH(onebit_abs_kernel, 0u, L, st, partial);
 }
-static hipError_t onebit_quant(const Launch& L, hipStream_t st) { HP_LAUNCH(onebit_quant_kernel, kLdsFor4, L, st); }
+static hipError_t onebit_quant(const Launch& L, hipStream_t st) { HP_LAUNCH(onebit_quant_kernel, 0u, L, st); }
 
 static hipError_t onebit_scale(const Launch& L, const float* partial, hipStream_t st) {
     if (L.single) {

@@ -179,6 +179,7 @@ __device__ __forceinline__ void sparse_reset_select(const Seg& s, const SparseWs
 
 template <class Src, bool DGC>
 __global__ __launch_bounds__(kBlock) void sparse_accum_kernel(Src src, SparseWs ws) {
+    if (!DGC) four_waves_per_simd();  // with the momentum streams the kernel does best unlimited
     unsigned tile;
     const Seg s = src.get(tile, blockIdx.x);
     if (tile == 0) sparse_reset_select(s, ws);
@@ -1153,7 +1154,7 @@ static hipError_t sparse_encode_src(const Src& src, const Src& ssrc_tiles, const
             const unsigned cnt = ntiles - base < per ? ntiles - base : per;
             const Src part = offset_src(src, base);
             if (dgc) hipLaunchKernelGGL((sparse_accum_kernel<Src, true>), dim3(cnt), dim3(kBlock), 0, st, part, ws);
-            else hipLaunchKernelGGL((sparse_accum_kernel<Src, false>), dim3(cnt), dim3(kBlock), kLdsFor4, st, part, ws);
+            else hipLaunchKernelGGL((sparse_accum_kernel<Src, false>), dim3(cnt), dim3(kBlock), 0, st, part, ws);
         }
     }
     if (on(1) && nstiles) hipLaunchKernelGGL((sparse_select_kernel<Src, 0>), dim3(nstiles), dim3(kBlock), 0, st, ssrc_tiles, ws);
