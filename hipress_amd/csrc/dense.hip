@@ -130,6 +130,7 @@ __device__ __forceinline__ void tbq_decode_tile(const Seg& s, unsigned tile) {
 
 template <class Src>
 __global__ __launch_bounds__(kBlock) void tbq_decode_kernel(Src src) {
+    four_waves_per_simd();
     unsigned tile;
     const Seg s = src.get(tile, xcd_grouped(blockIdx.x, gridDim.x));
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) tbq_decode_tile<true>(s, tile);
@@ -387,6 +388,7 @@ __device__ __forceinline__ void onebit_decode_tile(const Seg& s, unsigned tile) 
 
 template <class Src>
 __global__ __launch_bounds__(kBlock) void onebit_decode_kernel(Src src) {
+    four_waves_per_simd();
     unsigned tile;
     const Seg s = src.get(tile, xcd_grouped(blockIdx.x, gridDim.x));
     if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) onebit_decode_tile<true>(s, tile);
@@ -638,19 +640,20 @@ __global__ __launch_bounds__(kBlock) void terngrad_decode_kernel(Src src) {
         return hipGetLastError();                                                             \
     } while (0)
 
-// The decoders' cap pays while the payload they read (per_tile bytes for every 4096
-// elements) still fits the 256 MiB memory-side cache, where the encoder left it; once it
-// no longer does, the decoders run at about 5 instead of 6.5 TB/s and the cap costs
-// another 15 % (measured on sets of 0.8 to 1.6 G elements: the step in tbq decode lies
-// between 268 and 302 MB of payload, in onebit decode beyond 200 MB).
+// The TBQ and onebit decoders limit themselves to four wavefronts per SIMD by the registers
+// they claim, at every size (92 -> 80 us on the VGG19 set behind their encoders; at 1.5 and
+// 3 G elements the same as unlimited or 10 % better).  The TernGrad table decode does better
+// with five workgroups per CU, set with idle LDS, and only while the payload it reads
+// (per_tile bytes for every 4096 elements) still fits the 256 MiB memory-side cache, where
+// the encoder left it: beyond that such a cap costs 15 %.
 static unsigned decode_cap(const Launch& L, unsigned per_tile) {
     return (unsigned long long)L.ntiles * per_tile <= (192ull << 20) ? kLdsFor5 : 0u;
 }
 
 hipError_t launch_tbq_encode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_encode_kernel, 0u, L, st); }
-hipError_t launch_tbq_decode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_decode_kernel, decode_cap(L, kTile / 4), L, st); }
+hipError_t launch_tbq_decode(const Launch& L, hipStream_t st) { HP_LAUNCH(tbq_decode_kernel, 0u, L, st); }
 hipError_t launch_onebit_decode(const Launch& L, hipStream_t st) {
-    HP_LAUNCH(onebit_decode_kernel, decode_cap(L, kTile / 8), L, st);
+    HP_LAUNCH(onebit_decode_kernel, 0u, L, st);
 }
 // A single-tensor call learns the bucket size from the header on the device, a chain of
 // dependent loads that wants full occupancy; a table launch carries it in the descriptors.
