@@ -30,6 +30,7 @@ __device__ __forceinline__ void store_f32_bytes(uint8_t* p, float x) {
 
 template <class Src>
 __global__ __launch_bounds__(kBlock) void compll_minmax_kernel(Src src, float* partial) {
+    four_waves_per_simd();  // a read-only sweep: 61 -> 57 us on 102.8 M elements
     __shared__ float wmx[4], wmn[4];
     unsigned tile;
     const Seg s = src.get(tile, blockIdx.x);
