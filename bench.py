@@ -10,16 +10,24 @@ compressor / configuration (DGC over the same set first).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others] [--no-cpu]
 
-Prints ONE JSON line.  value = 4 * elements * steps / elapsed over exactly K
-steps bracketed by device synchronisation, in GB/s of fp32 gradient through
-encode+decode; `median_ms_per_step` is the median of the same steps timed one by
-one with events in a second run.  `roofline` describes the dominant kernel:
-algorithmic bytes per launch over its mean duration, measured with events on the
-launch stream in a third run that issues the encode sequence launch by launch,
-against the 8 TB/s HBM peak.  Every entry carries `cpu_baseline`: the scalar CPU
-oracle (one thread, the execution model of the reference's registered CPU
-operator) on a bounded sample of the same tensors, and the same source built with
-OpenMP on all host cores beside it.
+Prints ONE compact JSON line (under 4 KB) on stdout; the full per-workload records go to
+gpurun_out/bench_detail.json (path named in the line as `detail`) and, one JSON
+object per workload, to stderr.  value = 4 * elements * steps / elapsed over
+exactly K steps bracketed by device synchronisation, in GB/s of fp32 gradient
+through encode+decode; `median_ms_per_step` is the median of the same steps timed
+one by one with events in a second run.  `roofline` describes the dominant kernel:
+algorithmic bytes per launch over its mean duration against the 8 TB/s HBM peak.
+Two durations are carried: `kernel_ms_events`, measured live with events on the
+launch stream in a third run that issues the encode sequence launch by launch, and
+`kernel_ms_profile`, the kernel's average in the committed rocprofv3 summary of the
+same command (profiles/<workload>.md).  `frac` and `achieved` use the profile's
+duration when the summary exists (anyone can re-derive them from the committed
+table; `kernel_ms_source` names the file), the live one otherwise; `frac_events` is
+always the live figure.  `traffic` is the HBM bytes per launch from the same
+summary's counters and `traffic_ratio` its ratio to the algorithmic bytes.  Every
+entry carries `cpu_baseline`: the scalar CPU oracle (one thread, the execution model
+of the reference's registered CPU operator) on a bounded sample of the same
+tensors, and the same source built with OpenMP on all host cores beside it.
 """
 import argparse
 import ctypes
@@ -56,6 +64,56 @@ def measured_traffic(workload, kernel):
             except ValueError:
                 return None, None
     return None, None
+
+
+def profile_kernel_us(workload, kernel):
+    """Average duration in microseconds of `kernel` in the "Kernel statistics" table of
+    profiles/<workload>.md (rocprofv3 --kernel-trace --stats of `bench.py --workload
+    <workload>`): the first row of that table whose name holds `kernel`, or None when there
+    is no summary or no such row.  -> (microseconds, source path)"""
+    path = os.path.join(ROOT, "profiles", workload + ".md")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, None
+    sect = text.split("Kernel statistics", 1)
+    if len(sect) < 2:
+        return None, None
+    for line in sect[1].split("HBM traffic per dispatch", 1)[0].splitlines():
+        cells = [c.strip() for c in line.split("|")]
+        if len(cells) >= 6 and kernel in cells[1]:
+            try:
+                return float(cells[3].replace(",", "")), os.path.relpath(path, ROOT)
+            except ValueError:
+                return None, None
+    return None, None
+
+
+def launches_per_step(w):
+    """Launches of the dominant kernel in one step: the library issues a very long accumulate
+    pass in equal parts of at most 49,152 tiles; everything else is one launch."""
+    if w.dominant_kernel == "sparse_accum_kernel":
+        return -(-sum(-(-n // 4096) for n in w.sizes) // 49152)
+    return 1
+
+
+def roofline_of(workload, kernel, bytes_per_launch, launches, events_ms):
+    """The roofline record of one workload's dominant kernel.  bytes_per_launch: algorithmic
+    bytes one launch moves; events_ms: its live mean duration per launch (None when the
+    workload's calls do not expose the kernel on its own)."""
+    prof_us, prof_src = profile_kernel_us(workload, kernel)
+    traffic, traffic_src = measured_traffic(workload, kernel)
+    ms = prof_us * 1e-3 if prof_us else events_ms
+    if not ms:
+        return None
+    ach = bytes_per_launch / (ms * 1e-3) / 1e9
+    return {"bound": "hbm", "kernel": kernel, "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": ach / HBM_PEAK_GBS, "traffic": traffic,
+            "traffic_ratio": traffic / bytes_per_launch if traffic else None, "traffic_source": traffic_src,
+            "kernel_ms_source": prof_src if prof_us else "hipEvent",
+            "kernel_ms_profile": prof_us * 1e-3 if prof_us else None, "kernel_ms_events": events_ms,
+            "frac_events": bytes_per_launch / (events_ms * 1e-3) / 1e9 / HBM_PEAK_GBS if events_ms else None,
+            "launches_per_step": launches, "algorithmic_bytes_per_launch": bytes_per_launch}
 
 
 def _events(n):
@@ -558,7 +616,8 @@ def cpu_baseline(job, budget_s):
 
     passes, el = run(oracle.lib(), budget_s)
     out = {"value": 4.0 * job.elements * passes / el / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-           "sample": f"{job.sample}, {passes} passes, {el:.1f} s, scalar C oracle (gcc -O3, one thread)"}
+           "sample": f"{job.sample}, {passes} passes, {el:.1f} s, scalar C oracle (gcc -O3, one thread)",
+           "sample_short": f"front of the same tensors, {job.elements:,} elements/pass x {passes} passes, {el:.1f} s, scalar C oracle"}
     try:
         Lo = oracle.omp_lib()
         threads = int(Lo.hpo_threads())
@@ -672,17 +731,11 @@ def measure(name, steps, warmup, cpu_budget_s=0.0, min_warmup_s=0.25):
         "pct_of_hbm_roofline": 100.0 * alg_gbs / HBM_PEAK_GBS,
         **extra,
     }
-    if dom_ms:
-        # the library issues a very long accumulate pass in equal parts (49,152 tiles at most): figures per launch
-        launches = 1
-        if w.dominant_kernel == "sparse_accum_kernel":
-            launches = -(-sum(-(-n // 4096) for n in w.sizes) // 49152)
-        ach = dom_b * w.elements / (dom_ms * 1e-3) / 1e9
-        traffic, source = measured_traffic(name, w.dominant_kernel)
-        res["roofline"] = {"bound": "hbm", "kernel": w.dominant_kernel, "achieved": ach, "peak": HBM_PEAK_GBS,
-                           "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": source,
-                           "kernel_ms": dom_ms / launches, "launches_per_step": launches,
-                           "algorithmic_bytes_per_launch": dom_b * w.elements / launches}
+    launches = launches_per_step(w)
+    roof = roofline_of(name[: -len("_graph")] if graph else name, w.dominant_kernel,
+                       dom_b * w.elements / launches, launches, dom_ms / launches if dom_ms else None)
+    if roof:
+        res["roofline"] = roof
     if name == "tbq_262144":
         res["c_level"] = c_level_latency()
     if cpu_budget_s > 0 and hasattr(w, "cpu_job") and not graph:
@@ -697,6 +750,77 @@ def measure(name, steps, warmup, cpu_budget_s=0.0, min_warmup_s=0.25):
     del w
     torch.cuda.empty_cache()
     return res
+
+
+METRIC = "fp32 grad GB/s through encode+decode, % of HBM roofline; VGG19 TBQ, DGC"
+DETAIL_PATH = os.path.join("gpurun_out", "bench_detail.json")
+MAX_LINE_BYTES = 4096  # the final stdout line stays below this, whatever the number of workloads
+
+
+def _sig(x, digits=4):
+    """x rounded to `digits` significant digits (None stays None): keeps the line short."""
+    if x is None or isinstance(x, (str, bool)):
+        return x
+    return float(f"{x:.{digits}g}")
+
+
+def _short_roofline(r):
+    keep = ("bound", "kernel", "achieved", "peak", "unit", "frac", "traffic", "traffic_ratio", "kernel_ms_source",
+            "kernel_ms_profile", "kernel_ms_events", "frac_events", "launches_per_step", "algorithmic_bytes_per_launch")
+    out = {k: r.get(k) for k in keep}
+    for k in ("achieved", "frac", "traffic_ratio", "kernel_ms_profile", "kernel_ms_events", "frac_events"):
+        out[k] = _sig(out[k])
+    out["algorithmic_bytes_per_launch"] = int(out["algorithmic_bytes_per_launch"])
+    return out
+
+
+def _short_cpu(c):
+    """cpu_baseline without prose beyond one short `sample` string."""
+    out = {"value": _sig(c["value"]), "unit": c["unit"], "cores": c["cores"], "kind": c["kind"],
+           "sample": c.get("sample_short", c["sample"])[:120]}
+    ac = c.get("all_cores") or {}
+    if "value" in ac:
+        out["all_cores"] = {"value": _sig(ac["value"]), "cores": ac["cores"]}
+    return out
+
+
+def compact_line(main_res, others, steps, warmup):
+    """The one JSON object bench.py prints on stdout: the headline workload in full (metric,
+    value, timing, config, roofline, cpu_baseline) and every other workload reduced to
+    {workload, value, ms_per_step, pct, frac, cpu1, cpuN}.  Stays below MAX_LINE_BYTES."""
+    line = {
+        "metric": METRIC,
+        "value": _sig(main_res["value"], 6),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": _sig(main_res["ms_per_step"], 6),
+        "median_ms_per_step": _sig(main_res["median_ms_per_step"], 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": main_res["workload"], "elements": main_res["elements"], "tensors": main_res["tensors"],
+                   "algorithmic_bytes_per_element": _sig(main_res["algorithmic_bytes_per_element"], 6)},
+        "pct_of_hbm_roofline": _sig(main_res["pct_of_hbm_roofline"]),
+    }
+    if main_res.get("roofline"):
+        line["roofline"] = _short_roofline(main_res["roofline"])
+    if "cpu_baseline" in main_res:
+        line["cpu_baseline"] = _short_cpu(main_res["cpu_baseline"])
+    if "density" in main_res:
+        line["density"] = _sig(main_res["density"])
+    line["detail"] = DETAIL_PATH
+    if others:
+        line["others"] = []
+        for r in others:
+            cpu = r.get("cpu_baseline") or {}
+            line["others"].append({"workload": r["workload"], "value": _sig(r["value"]), "ms_per_step": _sig(r["ms_per_step"]),
+                                   "pct": _sig(r["pct_of_hbm_roofline"], 3), "frac": _sig((r.get("roofline") or {}).get("frac"), 3),
+                                   "cpu1": _sig(cpu.get("value"), 3), "cpuN": _sig((cpu.get("all_cores") or {}).get("value"), 3)})
+    return line
 
 
 def main():
@@ -737,42 +861,28 @@ def main():
                           "launches": args.steps}))
         return
 
-    main_res = measure(args.workload, args.steps, args.warmup, 0.0 if args.no_cpu else args.cpu_seconds,
-                       args.min_warmup_ms * 1e-3)
+    def record(r):  # the full record of each workload goes to stderr as soon as it is measured
+        sys.stderr.write(json.dumps(r) + "\n")
+        sys.stderr.flush()
+        return r
+
+    main_res = record(measure(args.workload, args.steps, args.warmup, 0.0 if args.no_cpu else args.cpu_seconds,
+                              args.min_warmup_ms * 1e-3))
     others = []
     if not args.no_others:
         for name in ALL_WORKLOADS:
             if name != args.workload:
-                others.append(measure(name, args.others_steps, 3, 0.0 if args.no_cpu else args.others_cpu_seconds,
-                                      args.min_warmup_ms * 1e-3))
-    line = {
-        "metric": "fp32 grad GB/s through encode+decode, % of HBM roofline; VGG19 TBQ, DGC",
-        "value": main_res["value"],
-        "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "warmup_steps_run": main_res["warmup_steps_run"],
-        "ms_per_step": main_res["ms_per_step"],
-        "median_ms_per_step": main_res["median_ms_per_step"],
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic (counter-based generator, seed 0; values as the configuration states them)",
-        "config": {"workload": args.workload, "elements": main_res["elements"], "tensors": main_res["tensors"],
-                   "algorithmic_bytes_per_element": main_res["algorithmic_bytes_per_element"]},
-        "pct_of_hbm_roofline": main_res["pct_of_hbm_roofline"],
-        "roofline": {k: v for k, v in main_res.get("roofline", {}).items()},
-    }
-    if "cpu_baseline" in main_res:
-        line["cpu_baseline"] = main_res["cpu_baseline"]
-    for k in ("density", "c_level"):
-        if k in main_res:
-            line[k] = main_res[k]
-    if others:
-        line["others"] = others
-    print(json.dumps(line))
+                others.append(record(measure(name, args.others_steps, 3, 0.0 if args.no_cpu else args.others_cpu_seconds,
+                                             args.min_warmup_ms * 1e-3)))
+    line = compact_line(main_res, others, args.steps, args.warmup)
+    detail = {"headline": main_res, "others": others}
+    try:  # the full records also go to a file next to the other run outputs
+        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        with open(os.path.join(ROOT, DETAIL_PATH), "w") as f:
+            json.dump(detail, f, indent=1)
+    except OSError as exc:
+        line["detail"] = f"not written: {exc}"
+    print(json.dumps(line, separators=(",", ":")), flush=True)
 
 
 if __name__ == "__main__":

@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <atomic>
 #include <cmath>
+#include <cstdint>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -458,12 +459,22 @@ int hipress_onebit_encode(const float* grad, float* residual, int64_t n, void* p
 // be cleared.
 constexpr int kStaticMaxDevices = 64;
 constexpr int64_t kStaticTiles = HIPRESS_ONEBIT_STATIC_MAX_N / kTile;
+static_assert(HIPRESS_ONEBIT_STATIC_MAX_N % kTile == 0 && kStaticTiles == 65536,
+              "a tensor of HIPRESS_ONEBIT_STATIC_MAX_N elements fills the array exactly");
 static __device__ __align__(256) float scratch[kStaticTiles];
 static std::atomic<float*> scratch_ptr[kStaticMaxDevices];
 
-static int static_scratch(float** out) {
+// The array of the CURRENT device; a stream that belongs to another device is refused
+// (its kernels would run where this pointer means nothing).
+static int static_scratch(hipStream_t stream, float** out) {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kStaticMaxDevices) return HIPRESS_ERR_HIP;
+    // 0, 1 and 2 are the default, legacy and per-thread stream handles: always the current device's
+    if (reinterpret_cast<uintptr_t>(stream) > 2) {
+        int sdev = -1;
+        if (hipStreamGetDevice(stream, &sdev) != hipSuccess) return HIPRESS_ERR_HIP;
+        if (sdev != dev) return HIPRESS_ERR_PARAM;
+    }
     float* p = scratch_ptr[dev].load(std::memory_order_acquire);
     if (!p) {
         if (hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch)) != hipSuccess || !p) return HIPRESS_ERR_HIP;
@@ -482,7 +493,7 @@ int hipress_onebit_encode_static(const float* grad, float* residual, int64_t n, 
     int rc = build_encode_seg(HIPRESS_ONEBIT, t, pr, &s);
     if (rc) return rc;
     float* partial = nullptr;
-    if ((rc = static_scratch(&partial))) return rc;
+    if ((rc = static_scratch(static_cast<hipStream_t>(stream), &partial))) return rc;
     return hiperr(launch_onebit_encode(single_launch(s), partial, -1, static_cast<hipStream_t>(stream)));
 }
 

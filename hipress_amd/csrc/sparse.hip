@@ -27,6 +27,7 @@
 //                   being zeroed at those places.
 // |x| is handled as the integer key bits(x) & 0x7fffffff, which orders like |x|.
 #include "common.h"
+#include "flat_pairs.h"
 #include "launch.h"
 
 namespace hp {
@@ -1078,15 +1079,17 @@ __global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs
         pcnt[threadIdx.x] = run.end > run.idx ? (unsigned)(run.end - run.idx) : 0u;
     }
     __syncthreads();
-    unsigned total = 0;
-    for (int p = 0; p < npeers; ++p) total += pcnt[p];
-    // The pairs of all peers, flattened peer by peer, are dealt out one per thread, so a
-    // whole round is one memory round trip; they are then added peer by peer (sums must
-    // follow the peer order; within a peer the indices are distinct).
-    for (unsigned base = 0; base < total; base += kBlock) {
-        const unsigned f = base + threadIdx.x;
-        unsigned myp = 0, before = 0;
-        while (myp + 1 < (unsigned)npeers && f >= before + pcnt[myp]) before += pcnt[myp++];
+    // The pairs of all peers, flattened peer by peer (64-bit positions: flat_pairs.h), are
+    // dealt out one per thread, so a whole round is one memory round trip; they are then
+    // added peer by peer (sums must follow the peer order; within a peer the indices are
+    // distinct).
+    using u64 = unsigned long long;
+    const u64 total = flat_total(pcnt, (unsigned)npeers);
+    for (u64 base = 0; base < total; base += kBlock) {
+        const u64 f = base + threadIdx.x;
+        unsigned myp = 0;
+        u64 before = 0;
+        flat_advance(pcnt, (unsigned)npeers, f, myp, before);
         const bool have = f < total;
         long long i = -1;
         float v = 0.f;
@@ -1096,11 +1099,13 @@ __global__ __launch_bounds__(kBlock) void sparse_merge_kernel(MSrc src, SparseWs
         }
         const bool inside = have && i >= t_lo && i < t_hi;
         // peers present in this round (uniform): first and last flat entry of the round
-        unsigned pfirst = 0, acc0 = 0;
-        while (pfirst + 1 < (unsigned)npeers && base >= acc0 + pcnt[pfirst]) acc0 += pcnt[pfirst++];
-        const unsigned lastf = (base + kBlock < total ? base + kBlock : total) - 1;
-        unsigned plast = pfirst, acc1 = acc0;
-        while (plast + 1 < (unsigned)npeers && lastf >= acc1 + pcnt[plast]) acc1 += pcnt[plast++];
+        unsigned pfirst = 0;
+        u64 acc0 = 0;
+        flat_advance(pcnt, (unsigned)npeers, base, pfirst, acc0);
+        const u64 lastf = (base + kBlock < total ? base + kBlock : total) - 1;
+        unsigned plast = pfirst;
+        u64 acc1 = acc0;
+        flat_advance(pcnt, (unsigned)npeers, lastf, plast, acc1);
         for (unsigned p = pfirst; p <= plast; ++p) {
             if (inside && myp == p) atomicAdd(&lds[i - t_lo], v);
             __syncthreads();

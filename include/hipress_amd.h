@@ -110,7 +110,10 @@ int hipress_onebit_decode(const void *payload, int64_t payload_bytes, float *out
  * held until the process ends), which limits n to HIPRESS_ONEBIT_STATIC_MAX_N
  * (larger n: HIPRESS_ERR_SIZE).  The call allocates and frees nothing; the first call
  * on a device looks up that device's copy of the array (hipGetSymbolAddress), so make
- * it once before a capture begins.  All calls on one GPU share the array: calls that
+ * it once before a capture begins.  The array used is the one of the CURRENT device
+ * (hipGetDevice at the time of the call): `stream` must belong to that device, and a
+ * stream of another device is refused with HIPRESS_ERR_PARAM before anything is
+ * enqueued.  All calls on one GPU share the array: calls that
  * overlap there (different streams without ordering) race; calls on one stream, or
  * ordered by events, are safe.  No counterpart in the reference. */
 #define HIPRESS_ONEBIT_STATIC_MAX_N 268435456LL /* 2^28 elements = 65,536 tiles of 4096 */

@@ -298,6 +298,75 @@ def untouched_outside(bufs, n):
         assert (b[:off] == -99.0).all() and (b[off + n:] == -99.0).all(), "wrote outside the view"
 
 
+def _deferred_steps_against_two_pass_oracle(hp, n, grads, r0, state, sstate, res, check_scale):
+    """Runs the deferred-residual onebit pair (hipress_onebit_encode_deferred +
+    hipress_onebit_residual, per-tensor entry points) over consecutive steps and holds every
+    payload and every materialised residual against the two-pass oracle, which is given the
+    GPU's scale of that step."""
+    r_ref = r0
+    for step, g in enumerate(grads):
+        pay = payload(hp.onebit_payload_bytes(n))
+        hp.onebit_encode_deferred(g[0], state, sstate, pay)
+        got = host(pay)
+        s = got[:4].view(F)[0]
+        check_scale(step, s, oracle.onebit_scale(g[1], r_ref))
+        want, r_ref = oracle.onebit_encode(g[1], r_ref, scale=s)
+        np.testing.assert_array_equal(got[4:], want[4:], err_msg=f"payload step {step}")
+        assert host(sstate).view(np.uint32)[0] == got[:4].view(np.uint32)[0]
+        hp.onebit_residual(state, sstate, res)
+        feq(host(res), r_ref, f"residual step {step}")
+        out = torch.full((n,), 7.0, device="cuda")
+        hp.onebit_decode(pay, out)
+        feq(host(out), oracle.onebit_decode(got, n), f"decode step {step}")
+
+
+@pytest.mark.parametrize("kind", ["finite", "inf", "nan"])
+def test_onebit_deferred_special_values_three_steps(hp, kind):
+    """The one-pass variant on NaN, infinities, signed zeros, denormals and FLT_MAX: what it
+    defers (r = v - d of the step before, formed on the fly) must come out as the two-pass
+    operator stores it, also once the scale is infinite or no number."""
+    n = 70001
+    rng = np.random.default_rng(11)
+    specials = {"finite": FINITE_SPECIALS[FINITE_SPECIALS != -FLT_MAX], "inf": SPECIALS[1:], "nan": SPECIALS}[kind]
+    grads = []
+    for step in range(3):
+        g = sprinkle(rng, n, 1e-3, np.roll(specials, step), every=4001 if kind == "finite" else 97)
+        if kind == "finite":
+            g[np.abs(g) == FLT_MAX] = 0.0
+            if step == 0:
+                g[12345] = FLT_MAX  # a single one: the sum stays finite in any order
+        grads.append((dev(g), g))
+    r0 = rng.normal(0, 1e-3, n).astype(F)
+
+    def check_scale(step, s, s_ref):
+        if kind == "finite":
+            assert np.isfinite(s) and abs(float(s) - float(s_ref)) <= 1e-5 * float(s_ref), (step, s, s_ref)
+        elif kind == "inf" and step == 0:
+            assert s == np.inf and s_ref == np.inf
+        else:  # a NaN input, or inf - inf from the step before: no number on both sides
+            assert np.isnan(s) == np.isnan(s_ref) and (np.isnan(s) or s == s_ref), (step, s, s_ref)
+
+    _deferred_steps_against_two_pass_oracle(hp, n, grads, r0, dev(r0), torch.zeros(1, device="cuda"),
+                                            torch.empty(n, device="cuda"), check_scale)
+
+
+@pytest.mark.parametrize("n", [9001, 70003])
+def test_onebit_deferred_unaligned_views_three_steps(hp, n):
+    """Gradient, state and residual output only 4-byte aligned (the element-wise path of the
+    one-pass kernel and of hipress_onebit_residual), three steps with the state carried."""
+    rng = np.random.default_rng(n + 1)
+    r0 = rng.normal(0, 1e-3, n).astype(F)
+    gs = [rng.normal(0, 1e-3, n).astype(F) for _ in range(3)]
+    (g0, g1, g2, sv, resv), bufs = views(n, gs[0], gs[1], gs[2], r0, None)
+
+    def check_scale(step, s, s_ref):
+        assert abs(float(s) - float(s_ref)) <= 1e-5 * float(s_ref), (step, s, s_ref)
+
+    _deferred_steps_against_two_pass_oracle(hp, n, list(zip((g0, g1, g2), gs)), r0, sv, torch.zeros(1, device="cuda"), resv,
+                                            check_scale)
+    untouched_outside(bufs, n)
+
+
 @pytest.mark.parametrize("n", [9001, 70003])
 def test_onebit_unaligned_views(hp, n):
     rng = np.random.default_rng(n)

@@ -92,6 +92,34 @@ def test_tbq_config1_full_size(hp):
     np.testing.assert_array_equal(host(out), oracle.tbq_decode(want_pay, n))
 
 
+def test_tbq_config1_three_steps_on_the_generated_tensor(hp):
+    """The first configuration as it is measured: one gradient of 262,144 elements, N(0, 0.02),
+    from the library's own counter-based generator with seed 0 (the tensor bench.py times),
+    threshold 0.05, residual zeros, three consecutive steps with the residual carried: payload,
+    residual and decoded tensor bit for bit against the oracle at every step."""
+    from hipress_amd import workloads
+
+    n = 262144
+    g_dev = workloads.normal_set([n], torch.device("cuda:0"), 0, sigma=0.02)[0]
+    g = host(g_dev)
+    assert g.dtype == F and abs(float(g.std()) - 0.02) < 5e-4 and abs(float(g.mean())) < 2e-4
+    r_gpu, r_ref = torch.zeros(n, device="cuda"), np.zeros(n, F)
+    seen = []
+    for step in range(3):
+        pay = payload(hp.tbq_payload_bytes(n))
+        hp.tbq_encode(g_dev, r_gpu, pay, 0.05)
+        want_pay, r_ref = oracle.tbq_encode(g, r_ref, 0.05)
+        np.testing.assert_array_equal(host(pay), want_pay, err_msg=f"payload step {step}")
+        np.testing.assert_array_equal(host(r_gpu).view(np.uint32), r_ref.view(np.uint32), err_msg=f"residual step {step}")
+        out = torch.full((n,), 7.0, device="cuda")
+        hp.tbq_decode(pay, out)
+        want_out = oracle.tbq_decode(want_pay, n)
+        np.testing.assert_array_equal(host(out).view(np.uint32), want_out.view(np.uint32), err_msg=f"decode step {step}")
+        seen.append(int(np.count_nonzero(want_out)))
+    # the carried residual matters: with sigma = 0.02 and tau = 0.05 later steps send more than the first
+    assert seen[0] > 0 and seen[1] > seen[0] and seen[2] > seen[0], seen
+
+
 # ---------------------------------------------------------------- onebit
 @pytest.mark.parametrize("n", SIZES)
 def test_onebit_encode_decode(hp, n):

@@ -87,3 +87,61 @@ def test_static_scratch_encode_rejects_what_its_array_cannot_hold():
     assert L.hipress_onebit_encode_static(fake, fake, big, fake, 16 + 4 * ((big + 31) // 32), None) == -2
     assert _lib.strerror(-2).startswith("element count")
     assert L.hipress_onebit_encode_static(None, None, 16, None, 100, None) == -1
+
+
+def test_static_scratch_encode_under_stream_capture():
+    """What the entry point is for: the first call is made eagerly (it looks up the device's
+    array), then the same call is captured into a HIP graph and replayed several times with the
+    program's own eager work between the replays; every replay must leave what the eager
+    workspace encoder leaves for the same gradient and residual."""
+    import torch
+
+    from hipress_amd import _lib
+
+    L = _lib.lib()
+    n = 300007
+    nbytes = int(L.hipress_onebit_payload_bytes(n))
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    g = torch.randn(n, generator=gen, device="cuda") * 0.01
+    r = torch.zeros(n, device="cuda")
+    pay = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    assert L.hipress_onebit_encode_static(g.data_ptr(), r.data_ptr(), n, pay.data_ptr(), nbytes,
+                                          torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    r.zero_()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            rc = L.hipress_onebit_encode_static(g.data_ptr(), r.data_ptr(), n, pay.data_ptr(), nbytes, side.cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    r.zero_()  # whatever the capture did or did not run, the replays start from a zero residual
+    ws = torch.empty(int(L.hipress_onebit_workspace_bytes(n)), dtype=torch.uint8, device="cuda")
+    r_ref = torch.zeros(n, device="cuda")
+    p_ref = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    for replay in range(4):
+        g.copy_(torch.randn(n, generator=gen, device="cuda") * 0.01)  # new gradient in the captured buffer
+        pay.fill_(0xAB)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert L.hipress_onebit_encode(g.data_ptr(), r_ref.data_ptr(), n, p_ref.data_ptr(), nbytes, ws.data_ptr(), ws.numel(),
+                                       torch.cuda.current_stream().cuda_stream) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(pay, p_ref), f"payload differs in replay {replay}"
+        assert torch.equal(r.view(torch.int32), r_ref.view(torch.int32)), f"residual differs in replay {replay}"
+
+
+def test_static_scratch_array_holds_exactly_the_largest_tensor():
+    """Host arithmetic only: the largest n the entry point takes is 65,536 tiles of 4096, the
+    size of its array (a static_assert in the library says the same), and one more element is
+    one tile too many."""
+    from hipress_amd import _lib
+
+    L = _lib.lib()
+    assert STATIC_MAX_N % 4096 == 0 and STATIC_MAX_N // 4096 == 65536
+    # the workspace encoder asks for one float per tile: the array is that size at the limit
+    assert int(L.hipress_onebit_workspace_bytes(STATIC_MAX_N)) >= 65536 * 4
+    fake = ctypes.c_void_p(1 << 20)
+    assert L.hipress_onebit_encode_static(fake, fake, STATIC_MAX_N + 1, fake, 16 + 4 * ((STATIC_MAX_N + 32) // 32), None) == -2
