@@ -96,7 +96,10 @@ int hipress_tbq_decode(const void *payload, int64_t payload_bytes, float *out, i
 /* ---- onebit: sign bits, per-tensor mean-magnitude scale, error feedback --- */
 /* Replaces <Func>_body for "onebit" (/root/reference/README.md:9).  Where the
  * reference body blocks the host on each thrust::reduce result
- * (TernGradEncode_body.h:115-116), the scale here stays on the device. */
+ * (TernGradEncode_body.h:115-116), the scale here stays on the device.  The scale is
+ * mean|r + g|, summed per 4096-element tile in fp32 (fixed order: the same bits on
+ * every run) and over the tiles in fp64; a tile whose magnitudes sum beyond FLT_MAX
+ * therefore yields an infinite scale where an fp64 sum would still be finite. */
 int hipress_onebit_encode(const float *grad, float *residual, int64_t n, void *payload,
                           int64_t payload_bytes, void *workspace, int64_t workspace_bytes,
                           void *stream);
