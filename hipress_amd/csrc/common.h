@@ -192,19 +192,32 @@ __device__ __forceinline__ unsigned xcd_grouped(unsigned b, unsigned nblocks) {
 }
 
 // Two-pass operators (a reduction over the tensor, then the pass that needs its result) read
-// the same arrays twice.  The second pass walks the launch backwards so that it begins where
-// the first one ended, and it does so in groups of eight so that workgroup b still runs on
-// the XCD that ran workgroup b' = b (mod 8) of the first pass: every XCD has its own L2, and
-// only the lines it fetched itself are in it.  A permutation of [0, nblocks).
+// the same arrays twice.  What the first pass read last can still be on the chip when the
+// second pass starts: not in the L2s (the counter of L2-to-fabric read traffic, FETCH_SIZE,
+// reads the same with and without what follows) but in the memory-side Infinity Cache behind
+// them (256 MiB, shared by all XCDs), which a streamed (non-temporal) load passes by and a
+// plain load fills.  So the first pass reads the last tiles of its launch with plain loads
+// (cache_tail) and the second pass walks the launch backwards (xcd_reversed), in groups of
+// eight so that consecutive workgroups still go to the eight XCDs in turn.  Both halves are
+// needed: on the same GPU, alternating libraries, the quantise pass of onebit over the VGG19
+// set takes 259 us with both, 263 us with only the reversed order and 263 us with neither;
+// the code pass of the min/max quantiser over 102.8 M elements 133 / 136 / 136 us.
+// How much to leave behind depends on what the second pass does besides re-reading.  After
+// one read stream (the min/max quantiser) the gain grows up to the cache's size: tails of
+// 32 / 64 / 128 / 192 / 256 / 384 MiB take min/max + code pass from 190.4 to 189.3 / 187.9 /
+// 185.9 / 185.3 / 186.7 us (the plain loads cost the first pass 1 us per 64 MiB, the second
+// pass gains 2.5).  After two read streams whose second pass also writes one of them back
+// (onebit) nothing is gained beyond 32 MiB: what the second pass saves, the first one loses.
+// A permutation of [0, nblocks).
 __device__ __forceinline__ unsigned xcd_reversed(unsigned b, unsigned nblocks) {
     const unsigned groups = nblocks >> 3, g = b >> 3;
     return g < groups ? (groups - 1 - g) * 8 + (b & 7u) : b;
 }
-// The first pass reads the last tiles of a launch with plain loads so that they stay in L2
-// for the second pass (a streamed load marks its line for early eviction): as many tiles as
-// the eight 4 MiB L2s hold of `streams` fp32 arrays.
-__device__ __forceinline__ bool l2_tail(unsigned b, unsigned nblocks, unsigned streams) {
-    return b + (32u << 20) / (streams * kTile * 4u) >= nblocks;
+constexpr unsigned kCacheTailOneStream = 256u << 20, kCacheTailTwoStreams = 32u << 20;  // bytes, all streams together
+// True for the last tiles of a launch that reads `streams` fp32 arrays: plain loads there.
+__device__ __forceinline__ bool cache_tail(unsigned b, unsigned nblocks, unsigned streams) {
+    const unsigned bytes = streams <= 1u ? kCacheTailOneStream : kCacheTailTwoStreams;
+    return b + bytes / ((streams ? streams : 1u) * kTile * 4u) >= nblocks;
 }
 // (The empty statement keeps the compiler from folding a branch of such loads into an
 // otherwise identical branch of streamed ones, which would make all of them plain.)

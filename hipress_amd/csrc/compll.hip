@@ -38,7 +38,7 @@ __global__ __launch_bounds__(kBlock) void compll_minmax_kernel(Src src, float* p
     const long long n = (long long)s.n;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
     const bool fast = s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n;
-    const bool keep = fast && l2_tail(blockIdx.x, gridDim.x, 1);  // left in L2 for the quantise pass
+    const bool keep = fast && cache_tail(blockIdx.x, gridDim.x, 1);  // left on the chip for the code pass
     float mx = kMaxInit, mn = kMinInit;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {

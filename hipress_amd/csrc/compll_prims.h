@@ -93,7 +93,7 @@ __global__ void serial_kernel(Args a, Dev* d) {
 // ---- streamed operands ---------------------------------------------------------------------
 // A lane owns four consecutive indices of each of four rows of 256 of its
 // wavefront's 1024.  Fn::stream(a, k), k < Fn::NS, are the float vectors a lambda
-// reads at its own index; they are loaded as 16-byte vectors, whole rows per wavefront.
+// KEEP: plain loads, which leave their lines on the chip for the sweep that follows; the others are
 // KEEP: plain loads, which leave their lines in L2 for the sweep that follows; the others are
 // streamed.  (The empty statement keeps the compiler from folding the two otherwise identical
 // branches into one, which would drop the streaming hint from both.)
@@ -129,16 +129,20 @@ __device__ __forceinline__ void load_streams(const Args& a, long long base, long
     else load_streams_as<Args, Fn, false>(a, base, count, x);
 }
 
-// A sweep that follows a reduce over the same vectors walks its tiles backwards, in groups of
-// eight so that workgroup b stays on the XCD (b mod 8) whose L2 holds what workgroup b' = b
-// (mod 8) of the reduce read last; the reduce reads as many of its last tiles with plain
-// loads as the eight 4 MiB L2s hold.
+// A sweep that follows a reduce over the same vectors walks its tiles backwards (in groups of
+// eight, so that consecutive workgroups still go to the eight XCDs in turn), and the reduce
+// reads its last tiles with plain loads: a plain load leaves its line in the memory-side
+// Infinity Cache (256 MiB), which a streamed load passes by, so the sweep begins with data
+// that is still on the chip.  After a reduce over one vector the tail is as large as that
+// cache; with more vectors 32 MiB in all (beyond that the plain loads cost the reduce what
+// the sweep gains).
 __device__ __forceinline__ unsigned tile_reversed(unsigned b, unsigned nblocks) {
     const unsigned groups = nblocks >> 3, g = b >> 3;
     return g < groups ? (groups - 1 - g) * 8 + (b & 7u) : b;
 }
-__device__ __forceinline__ bool in_l2_tail(unsigned b, unsigned nblocks, unsigned streams) {
-    return b + (32u << 20) / ((streams ? streams : 1u) * (unsigned)kTile * 4u) >= nblocks;
+__device__ __forceinline__ bool in_cache_tail(unsigned b, unsigned nblocks, unsigned streams) {
+    const unsigned bytes = streams <= 1u ? (256u << 20) : (32u << 20);
+    return b + bytes / ((streams ? streams : 1u) * (unsigned)kTile * 4u) >= nblocks;
 }
 
 // ---- reduce --------------------------------------------------------------------------------
@@ -161,7 +165,7 @@ __global__ __launch_bounds__(kBlock) void reduce_tiles_kernel(Args a, const Dev*
     const long long n = Src::count(a, *d);
     const long long base = (long long)blockIdx.x * kTile + wave * 1024 + lane * 4;
     f4 in[Src::NS > 0 ? Src::NS : 1][4];
-    load_streams<Args, Src>(a, base, n, in, in_l2_tail(blockIdx.x, gridDim.x, Src::NS));
+    load_streams<Args, Src>(a, base, n, in, in_cache_tail(blockIdx.x, gridDim.x, Src::NS));
     f4 x[4];
     unsigned ok[4];
 #pragma unroll

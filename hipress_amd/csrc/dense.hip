@@ -146,7 +146,7 @@ __device__ __forceinline__ float abs4sum(f4 v) {
 }
 
 // Pass 1: one partial sum of |r+g| per tile, in a fixed order (deterministic).
-// KEEP: plain loads, for the tiles the quantise pass is to find in L2.
+// KEEP: plain loads, for the tiles the quantise pass is to find on the chip (cache_tail).
 template <bool FAST, bool KEEP = false>
 __device__ __forceinline__ float onebit_abs_tile(const Seg& s, unsigned tile) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(kBlock) void onebit_abs_kernel(Src src, float* part
     const Seg s = src.get(tile, blockIdx.x);
     float a;
     const bool whole = s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n;
-    if (whole && l2_tail(blockIdx.x, gridDim.x, 2)) a = onebit_abs_tile<true, true>(s, tile);
+    if (whole && cache_tail(blockIdx.x, gridDim.x, 2)) a = onebit_abs_tile<true, true>(s, tile);
     else if (whole) a = onebit_abs_tile<true>(s, tile);
     else a = onebit_abs_tile<false>(s, tile);
     a = wave_sum(a);
@@ -261,8 +261,8 @@ __device__ __forceinline__ void onebit_quant_tile(const Seg& s, unsigned tile) {
     if ((lane & 7u) < 4u && (FAST || widx < (long long)((n + 31) >> 5))) words[widx] = myword;
 }
 
-// The launch is walked from its end towards its start, XCD by XCD: the pass that summed
-// |r+g| finished there and left its last tiles in L2 (xcd_reversed, l2_tail).
+// The launch is walked from its end towards its start: the pass that summed |r+g| finished
+// there and left its last tiles in the Infinity Cache (xcd_reversed, cache_tail).
 template <class Src>
 __global__ __launch_bounds__(kBlock) void onebit_quant_kernel(Src src) {
     four_waves_per_simd();
