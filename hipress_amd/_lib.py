@@ -7,7 +7,9 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libhipress_amd.so")
+# HIPRESS_AMD_LIB names another build of the same library (a variant made with
+# `python -m hipress_amd.build --define ... --output ...` for an A/B measurement)
+LIB_PATH = os.environ.get("HIPRESS_AMD_LIB") or os.path.join(_HERE, "libhipress_amd.so")
 
 ONEBIT, TBQ, TERNGRAD, DGC, GRADDROP, ONEBIT_DEFERRED = range(6)
 ALG_IDS = {"onebit": ONEBIT, "tbq": TBQ, "terngrad": TERNGRAD, "dgc": DGC, "graddrop": GRADDROP,

@@ -208,16 +208,29 @@ __device__ __forceinline__ unsigned xcd_grouped(unsigned b, unsigned nblocks) {
 // 185.9 / 185.3 / 186.7 us (the plain loads cost the first pass 1 us per 64 MiB, the second
 // pass gains 2.5).  After two read streams whose second pass also writes one of them back
 // (onebit) nothing is gained beyond 32 MiB: what the second pass saves, the first one loses.
+//
+// Tuning constants, overridable at build time for A/B measurements
+// (python -m hipress_amd.build --define HP_CACHE_TAIL_ONE_MIB=0 ...): MiB read with plain loads
+// at the end of a first pass over one / over several fp32 arrays (0 = none), and whether the
+// second pass is walked backwards.
+#ifndef HP_CACHE_TAIL_ONE_MIB
+#define HP_CACHE_TAIL_ONE_MIB 256
+#endif
+#ifndef HP_CACHE_TAIL_MANY_MIB
+#define HP_CACHE_TAIL_MANY_MIB 32
+#endif
+#ifndef HP_SECOND_PASS_REVERSED
+#define HP_SECOND_PASS_REVERSED 1
+#endif
 // A permutation of [0, nblocks).
 __device__ __forceinline__ unsigned xcd_reversed(unsigned b, unsigned nblocks) {
     const unsigned groups = nblocks >> 3, g = b >> 3;
-    return g < groups ? (groups - 1 - g) * 8 + (b & 7u) : b;
+    return (HP_SECOND_PASS_REVERSED) && g < groups ? (groups - 1 - g) * 8 + (b & 7u) : b;
 }
-constexpr unsigned kCacheTailOneStream = 256u << 20, kCacheTailTwoStreams = 32u << 20;  // bytes, all streams together
 // True for the last tiles of a launch that reads `streams` fp32 arrays: plain loads there.
 __device__ __forceinline__ bool cache_tail(unsigned b, unsigned nblocks, unsigned streams) {
-    const unsigned bytes = streams <= 1u ? kCacheTailOneStream : kCacheTailTwoStreams;
-    return b + bytes / ((streams ? streams : 1u) * kTile * 4u) >= nblocks;
+    const unsigned bytes = (streams <= 1u ? (unsigned)HP_CACHE_TAIL_ONE_MIB : (unsigned)HP_CACHE_TAIL_MANY_MIB) << 20;
+    return b + bytes / ((streams ? streams : 1u) * kTile * 4u) >= nblocks && bytes != 0u;
 }
 // (The empty statement keeps the compiler from folding a branch of such loads into an
 // otherwise identical branch of streamed ones, which would make all of them plain.)

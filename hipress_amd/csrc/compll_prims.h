@@ -136,13 +136,23 @@ __device__ __forceinline__ void load_streams(const Args& a, long long base, long
 // that is still on the chip.  After a reduce over one vector the tail is as large as that
 // cache; with more vectors 32 MiB in all (beyond that the plain loads cost the reduce what
 // the sweep gains).
+// (Build-time overrides for A/B measurements, as in common.h of the hand-written kernels.)
+#ifndef HP_CACHE_TAIL_ONE_MIB
+#define HP_CACHE_TAIL_ONE_MIB 256
+#endif
+#ifndef HP_CACHE_TAIL_MANY_MIB
+#define HP_CACHE_TAIL_MANY_MIB 32
+#endif
+#ifndef HP_SECOND_PASS_REVERSED
+#define HP_SECOND_PASS_REVERSED 1
+#endif
 __device__ __forceinline__ unsigned tile_reversed(unsigned b, unsigned nblocks) {
     const unsigned groups = nblocks >> 3, g = b >> 3;
-    return g < groups ? (groups - 1 - g) * 8 + (b & 7u) : b;
+    return (HP_SECOND_PASS_REVERSED) && g < groups ? (groups - 1 - g) * 8 + (b & 7u) : b;
 }
 __device__ __forceinline__ bool in_cache_tail(unsigned b, unsigned nblocks, unsigned streams) {
-    const unsigned bytes = streams <= 1u ? (256u << 20) : (32u << 20);
-    return b + bytes / ((streams ? streams : 1u) * (unsigned)kTile * 4u) >= nblocks;
+    const unsigned bytes = (streams <= 1u ? (unsigned)HP_CACHE_TAIL_ONE_MIB : (unsigned)HP_CACHE_TAIL_MANY_MIB) << 20;
+    return b + bytes / ((streams ? streams : 1u) * (unsigned)kTile * 4u) >= nblocks && bytes != 0u;
 }
 
 // ---- reduce --------------------------------------------------------------------------------
