@@ -814,6 +814,9 @@ def compact_line(main_res, others, steps, warmup):
         line["density"] = _sig(main_res["density"])
     line["detail"] = DETAIL_PATH
     if others:
+        # cpu1 / cpuN of every entry: GB/s of the scalar oracle on one thread / on this many threads
+        cores = [(r.get("cpu_baseline") or {}).get("all_cores", {}).get("cores") for r in others]
+        line["others_cpu_cores"] = {"cpu1": 1, "cpuN": next((c for c in cores if c), None)}
         line["others"] = []
         for r in others:
             cpu = r.get("cpu_baseline") or {}

@@ -11,7 +11,11 @@
  * Every call only enqueues work on `stream` and returns; nothing here
  * synchronises with the host or allocates device memory, except
  * hipress_batch_create / hipress_merge_batch_create (set-up time) and their
- * destroy calls.
+ * destroy calls.  Like the reference's bodies, the library starts no threads and keeps
+ * no state between calls beyond what the caller passes in (two atomic counters and
+ * the array of hipress_onebit_encode_static aside): calls from different host
+ * threads may overlap as long as their buffers, workspaces and batch objects are
+ * distinct.
  *
  * The per-tensor entry points replace the reference's generated operator body
  *   void <Func>_body<policy_t>(float* gradient, int32 _gradient_size,

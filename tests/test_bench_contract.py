@@ -108,6 +108,7 @@ def test_the_printed_line_is_compact_and_complete():
     cpu = back["cpu_baseline"]
     assert cpu["value"] > 0 and cpu["cores"] == 1 and cpu["kind"] == "port" and len(cpu["sample"]) <= 120
     assert cpu["all_cores"]["cores"] == 16
+    assert back["others_cpu_cores"] == {"cpu1": 1, "cpuN": 16}
     assert [o["workload"] for o in back["others"]] == bench.ALL_WORKLOADS[1:]
     for o in back["others"]:
         assert set(o) == {"workload", "value", "ms_per_step", "pct", "frac", "cpu1", "cpuN"}
