@@ -11,8 +11,8 @@ compressor / configuration (DGC over the same set first).
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-others] [--no-cpu]
 
 Prints ONE compact JSON line (under 4 KB) on stdout; the full per-workload records go to
-gpurun_out/bench_detail.json (path named in the line as `detail`) and, one JSON
-object per workload, to stderr.  value = 4 * elements * steps / elapsed over
+a JSON file beside the other run outputs (its path is in the line as `detail`) and, one
+JSON object per workload, to stderr.  value = 4 * elements * steps / elapsed over
 exactly K steps bracketed by device synchronisation, in GB/s of fp32 gradient
 through encode+decode; `median_ms_per_step` is the median of the same steps timed
 one by one with events in a second run.  `roofline` describes the dominant kernel:
