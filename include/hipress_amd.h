@@ -222,8 +222,12 @@ int hipress_sparse_decode_merge(const void *const *payloads, const int64_t *payl
  * zero: aggregate[i] = ((local[i] + d_1[i]) + d_2[i]) + ..., peers added in order.  One
  * hop of a ring (the payload that arrived, the local gradient, the re-encoded payload to
  * send on), or a server that is also a worker and need not compress its own share.
- * local = NULL is the plain merge; aggregate may be the same buffer as local.  No
- * counterpart in the reference checkout (CaSync's sources are not part of it). */
+ * local = NULL is the plain merge; aggregate may be the same buffer as local.  More
+ * than HIPRESS_MAX_PEERS payloads are merged by several calls, each after the first
+ * with local = the aggregate so far (and only the last with the re-encode): the
+ * additions happen in the same order as in one sum over all peers, so the result is
+ * the same bit for bit.  No counterpart in the reference checkout (CaSync's sources
+ * are not part of it). */
 int hipress_tbq_decode_merge_local(const void *const *payloads, const int64_t *payload_bytes,
                                    int32_t npeers, const float *local, float *aggregate, int64_t n,
                                    float *residual, void *out_payload, int64_t out_payload_bytes,

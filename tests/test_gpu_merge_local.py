@@ -162,3 +162,37 @@ def test_empty_chunk_and_argument_checks(hp):
     with pytest.raises(TypeError):
         hp.onebit_decode_merge([torch.zeros(hp.onebit_payload_bytes(8), dtype=torch.uint8, device="cuda")],
                                torch.empty(8, device="cuda"), local=torch.empty(8, device="cuda", dtype=torch.float64))
+
+
+@pytest.mark.parametrize("n", [100003, (1 << 20) + 5])
+def test_more_peers_than_one_call_takes_are_merged_in_two_calls(hp, n):
+    """One call takes at most 16 peers.  Twenty are merged by two calls, the second starting
+    from the first one's aggregate (`local`) and carrying the re-encode: the additions happen
+    in the same order as in one sum over all twenty, so aggregate, re-encoded payload and state
+    equal the oracle's for twenty peers bit for bit - dense (TBQ) and sparse."""
+    rng = np.random.default_rng(n)
+    P, first = 20, 16
+    tau = F(0.05)
+    pays = [oracle.tbq_encode(rng.normal(0, 0.04, n).astype(F), np.zeros(n, F), tau)[0] for _ in range(P)]
+    r0 = rng.normal(0, 0.01, n).astype(F)
+    want_agg, want_out, want_r = oracle.tbq_decode_merge(pays, n, r0, tau)
+    d = [dev(p) for p in pays]
+    agg, res = torch.empty(n, device="cuda"), dev(r0)
+    outp = torch.zeros(hp.tbq_payload_bytes(n), dtype=torch.uint8, device="cuda")
+    hp.tbq_decode_merge(d[:first], agg)
+    hp.tbq_decode_merge(d[first:], agg, res, outp, tau, local=agg)  # aggregate may be the same buffer as local
+    np.testing.assert_array_equal(host(agg), want_agg)
+    np.testing.assert_array_equal(host(outp), want_out)
+    np.testing.assert_array_equal(host(res), want_r)
+    # sparse: twenty GradDrop payloads, re-encoded at 1 %
+    sp = [oracle.graddrop_encode(rng.normal(0, 1e-3, n).astype(F), np.zeros(n, F), 0.01)[0] for _ in range(P)]
+    a0 = rng.normal(0, 1e-4, n).astype(F)
+    want_agg, want_out, want_acc = oracle.sparse_decode_merge(sp, n, a0, 0.01)
+    d = [dev(p) for p in sp]
+    agg, acc = torch.empty(n, device="cuda"), dev(a0)
+    outp = torch.zeros(hp.sparse_payload_bytes(n, 0.01), dtype=torch.uint8, device="cuda")
+    hp.dgc_decode_merge(d[:first], agg)
+    hp.dgc_decode_merge(d[first:], agg, acc, outp, 0.01, local=agg)
+    np.testing.assert_array_equal(host(agg), want_agg)
+    np.testing.assert_array_equal(host(acc), want_acc)
+    same_pairs(host(outp), want_out)
