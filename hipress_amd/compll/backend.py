@@ -47,6 +47,12 @@ def _rerunnable(lines) -> bool:
     return True
 
 
+def _local(name: str) -> str:
+    """A lambda's parameter or local variable as it is spelt in the generated source: prefixed,
+    so that a program's own names (`a`, `d`, `s`, `i` ...) never meet the generator's."""
+    return "l_" + name
+
+
 def _unparen(code: str) -> str:
     """Drops one pair of parentheses that encloses the whole expression."""
     if code.startswith("(") and code.endswith(")"):
@@ -200,7 +206,7 @@ class FunctionGen:
             return Value(e.text, "int", "host")
         if isinstance(e, F.Name):
             if e.id in scope:
-                return Value(e.id, scope[e.id], "host")
+                return Value(_local(e.id), scope[e.id], "host")
             s = self.scalar(e.id, e.line)
             if s.cls is None:
                 raise CompileError(f"{e.id!r} is used before it has a value", e.line)
@@ -253,7 +259,7 @@ class FunctionGen:
             self.needs_uniform = True
             if self.streams is not None:
                 return Value(f"cl::uniform_from(s[{self._stream('a.uniform')}], (float)({lo.code}), (float)({hi.code}))", "float", "dev")
-            return Value(f"cl::uniform_draw(a.uniform, {index_name}, (float)({lo.code}), (float)({hi.code}))", "float", "dev")
+            return Value(f"cl::uniform_draw(a.uniform, {_local(index_name)}, (float)({lo.code}), (float)({hi.code}))", "float", "dev")
         if isinstance(e, F.Call):
             args = [self.expr(x, scope, index_name) for x in e.args]
             cls = "dev" if any(x.cls == "dev" for x in args) else "host"
@@ -317,7 +323,7 @@ class FunctionGen:
         kind = self.lambda_kind(lam)
         ret = {"float": "float", "int": "long long"}[kind]
         index_name = lam.params[0].name if len(lam.params) == 1 and self._kind_of(lam.params[0].type) == "int" else None
-        params = ", ".join(("float " if self._kind_of(p.type) == "float" else "long long ") + p.name for p in lam.params)
+        params = ", ".join(("float " if self._kind_of(p.type) == "float" else "long long ") + _local(p.name) for p in lam.params)
         scope = self._lambda_scope(lam)
         lines = [f"static __device__ __forceinline__ {ret} fn_{name}(const Args& a, const Dev& d, {params}) {{"]
         lines += self.lambda_body(lam.body, scope, index_name, ret, 1)
@@ -429,7 +435,7 @@ class FunctionGen:
         ret = {"float": "float", "int": "long long"}[kind]
         index_name = lam.params[0].name
         self.streams = None if self._assigns(lam.body, index_name) else []
-        lines = [f"static __device__ __forceinline__ {ret} mfn_{name}(const Args& a, const Dev& d, long long {index_name}, const float* s) {{"]
+        lines = [f"static __device__ __forceinline__ {ret} mfn_{name}(const Args& a, const Dev& d, long long {_local(index_name)}, const float* s) {{"]
         lines += self.lambda_body(lam.body, self._lambda_scope(lam), index_name, ret, 1)
         lines.append(f"    return ({ret})0;")
         lines.append("}")
@@ -447,18 +453,18 @@ class FunctionGen:
                     raise CompileError("vectors cannot be declared inside a lambda", st.line)
                 ctype = "float" if st.type.base == "float" else "long long"
                 if st.value is None:
-                    out.append(f"{pad}{ctype} {st.name} = 0;")
+                    out.append(f"{pad}{ctype} {_local(st.name)} = 0;")
                 else:
                     if not isinstance(st.value, F.Expr) or isinstance(st.value, (F.Reduce, F.Map, F.Concat)):
                         raise CompileError("vector primitives cannot be used inside a lambda", st.line)
                     v = self.expr(st.value, scope, index_name)
-                    out.append(f"{pad}{ctype} {st.name} = ({ctype})({v.code});")
+                    out.append(f"{pad}{ctype} {_local(st.name)} = ({ctype})({v.code});")
                 scope[st.name] = "float" if ctype == "float" else "int"
             elif isinstance(st, F.Assign):
                 if st.name not in scope:
                     raise CompileError(f"a lambda may only assign its own variables ({st.name!r})", st.line)
                 v = self.expr(st.value, scope, index_name)
-                out.append(f"{pad}{st.name} = {v.code};")
+                out.append(f"{pad}{_local(st.name)} = {v.code};")
             elif isinstance(st, F.If):
                 c = self.expr(st.cond, scope, index_name)
                 out.append(f"{pad}if ({_unparen(c.code)}) {{")

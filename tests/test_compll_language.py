@@ -192,3 +192,37 @@ def test_maps_share_a_sweep_only_when_that_is_what_the_program_says():
         compll.compile_text(FEEDBACK % ("i", "r = map(range(g.size), carry); out = concat(t, codes);"))
     with pytest.raises(F.CompileError, match="only once"):
         compll.compile_text("void Op(float* g, uint8* o, uint8 b) { int k = b + 1; k = 2; }")
+
+
+REFERENCE_PSE = "/root/reference/src/CompLL/GCGen/pse"
+
+
+@pytest.mark.skipif(not os.path.isdir(REFERENCE_PSE), reason="the reference checkout is not on this machine")
+def test_the_reference_checkout_s_own_programs_compile_unmodified(tmp_path):
+    """A user of the reference's generator brings programs written for it.  The two it ships
+    (TernGradEncode.pse, TernGradDecode.pse: read here where they lie, never copied) go through
+    this compiler as they are - commented-out `param` block, `else` branches, `uint<bitwidth>`,
+    `concat` / `extract`, `.size`, `random<float>` - give the same launch plan as the restated
+    program the GPU tests run, and the HIP they turn into compiles for gfx950."""
+    import subprocess
+
+    from hipress_amd import build as hb
+
+    plans = {}
+    for name in ("TernGradEncode", "TernGradDecode"):
+        text = open(os.path.join(REFERENCE_PSE, name + ".pse")).read()
+        source, manifest = compll.compile_text(text)
+        assert [m["name"] for m in manifest] == [name]
+        plans[name] = manifest[0]
+        assert f'extern "C" int {name}(' in source and f'extern "C" int64_t {name}_workspace_bytes(' in source
+        src = tmp_path / (name + ".hip")
+        src.write_text(source)
+        r = subprocess.run([os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), *hb.FLAGS, "-I", os.path.join(os.path.dirname(hb.CSRC), "csrc"),
+                            "--cuda-device-only", "-c", str(src), "-o", os.devnull], capture_output=True, text=True, timeout=600)
+        assert r.returncode == 0, r.stderr[-3000:]
+    ours = manifests()
+    assert plans["TernGradEncode"]["launches"] == ours["MinMaxQuantEncode"]["launches"] == ["reduce", "map_packed"]
+    assert plans["TernGradDecode"]["launches"] == ours["MinMaxQuantDecode"]["launches"] == ["map_float"]
+    # same operator surface as the reference registers: (gradient, compressed, bitwidth) / (compressed, gradient)
+    assert [p["name"] for p in plans["TernGradEncode"]["params"]][:3] == ["gradient", "compressed", "bitwidth"]
+    assert [p["name"] for p in plans["TernGradDecode"]["params"]][:2] == ["compressed", "gradient"]
