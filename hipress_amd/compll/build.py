@@ -2,6 +2,8 @@
 hipress_amd/libhipress_compll_gen.so for gfx950 (cross-compiles without a GPU).
 
 Usage: python -m hipress_amd.compll.build
+A program of one's own: python -m hipress_amd.compll my.pse --library my_ops.so, then
+hipress_amd.compll.runtime.Operators("my_ops.so").
 """
 import glob
 import os
@@ -33,18 +35,29 @@ def manifests():
     return out
 
 
-def build(verbose=False):
+def build_library(paths, output, workdir=None, verbose=False):
+    """Generates HIP from the operator programs `paths`, compiles it for gfx950 and links
+    `output` (a shared library with one C entry point per operator); the operators'
+    parameter lists go to `output + ".json"`, which runtime.Operators reads to bind them."""
+    import json
+
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    os.makedirs(GENERATED, exist_ok=True)
-    objs, procs = [], []
-    for path in programs():
+    output = os.path.abspath(output)
+    workdir = workdir or output + ".build"
+    os.makedirs(workdir, exist_ok=True)
+    objs, procs, manifest = [], [], {}
+    for path in paths:
         stem = os.path.splitext(os.path.basename(path))[0]
         with open(path) as f:
-            source, _ = compile_text(f.read())
-        hip = os.path.join(GENERATED, stem + ".hip")
+            source, man = compile_text(f.read())
+        for m in man:
+            if m["name"] in manifest:
+                raise RuntimeError(f"operator {m['name']!r} is defined twice ({path})")
+            manifest[m["name"]] = m
+        hip = os.path.join(workdir, stem + ".hip")
         with open(hip, "w") as f:
             f.write(source)
-        obj = os.path.join(GENERATED, stem + ".o")
+        obj = os.path.join(workdir, stem + ".o")
         cmd = [hipcc, *FLAGS, "-c", hip, "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
@@ -61,9 +74,34 @@ def build(verbose=False):
             sys.stderr.write(f"--- {stem} ---\n{out}\n")
     if failed:
         raise RuntimeError("hipcc failed on generated code")
-    subprocess.check_call([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs])
-    return LIB
+    subprocess.check_call([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", output, *objs])
+    with open(output + ".json", "w") as f:
+        json.dump(manifest, f, indent=1)
+    return output
+
+
+def build(verbose=False):
+    """The shipped programs -> hipress_amd/libhipress_compll_gen.so."""
+    return build_library(programs(), LIB, workdir=GENERATED, verbose=verbose)
+
+
+# The two programs the reference checkout ships for its own generator.  Where that checkout is
+# present they are compiled as they are, read in place, into a library of their own (kept out
+# of version control like every built file), so that a GPU test can run the operators a user of
+# the reference would bring.
+REFERENCE_PROGRAMS = "/root/reference/src/CompLL/GCGen/pse"
+REFERENCE_LIB = os.path.join(GENERATED, "reference_programs", "libreference_programs.so")
+
+
+def build_reference_programs(verbose=False):
+    """-> the library's path, or None when the reference checkout is not on this machine."""
+    paths = sorted(glob.glob(os.path.join(REFERENCE_PROGRAMS, "*.pse")))
+    if not paths:
+        return None
+    os.makedirs(os.path.dirname(REFERENCE_LIB), exist_ok=True)
+    return build_library(paths, REFERENCE_LIB, verbose=verbose)
 
 
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_reference_programs(verbose=True) or "no reference checkout here: its programs are not built")

@@ -22,12 +22,27 @@ class GeneratedOpError(RuntimeError):
 
 
 class Operators:
-    def __init__(self, path=LIB):
+    """The operators of a generated library as Python callables.  path: the library
+    (default: the one built from the shipped programs); manifest: name -> parameter list,
+    by default the file `path + ".json"` that the build writes beside the library."""
+
+    def __init__(self, path=LIB, manifest=None):
         if not os.path.exists(path):
-            raise GeneratedOpError(f"{path} is missing: run `python -m hipress_amd.compll.build`")
+            raise GeneratedOpError(f"{path} is missing: run `python -m hipress_amd.compll.build` "
+                                   "(or `python -m hipress_amd.compll prog.pse --library {path}` for a program of your own)")
         self._lib = ctypes.CDLL(path)
         self._workspaces = {}
-        self.manifest = manifests()
+        if manifest is None:
+            if os.path.exists(path + ".json"):
+                import json
+
+                with open(path + ".json") as f:
+                    manifest = json.load(f)
+            elif os.path.abspath(path) == os.path.abspath(LIB):
+                manifest = manifests()
+            else:
+                raise GeneratedOpError(f"{path}.json (the operators' parameter lists) is missing")
+        self.manifest = manifest
         for name, m in self.manifest.items():
             fn = getattr(self._lib, name)
             argtypes = []

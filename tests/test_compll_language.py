@@ -226,3 +226,41 @@ def test_the_reference_checkout_s_own_programs_compile_unmodified(tmp_path):
     # same operator surface as the reference registers: (gradient, compressed, bitwidth) / (compressed, gradient)
     assert [p["name"] for p in plans["TernGradEncode"]["params"]][:3] == ["gradient", "compressed", "bitwidth"]
     assert [p["name"] for p in plans["TernGradDecode"]["params"]][:2] == ["compressed", "gradient"]
+
+
+def test_a_program_of_one_s_own_becomes_a_loadable_library(tmp_path):
+    """The whole way a user of the reference's generator goes: program in, library out
+    (`python -m hipress_amd.compll prog.pse -b --library ops.so`), operators bound from the
+    manifest the build leaves beside it.  No GPU call is made."""
+    import json
+    import subprocess
+    import sys
+
+    from hipress_amd.compll import runtime
+
+    prog = tmp_path / "clip.pse"
+    prog.write_text("""
+void ClipScale(float* gradient, float* clipped, float bound) {
+    lambda_func keep = [&](int index) -> float {
+        float a = gradient[index];
+        if (a > bound) { return bound; }
+        if (a < 0 - bound) { return 0 - bound; }
+        return a;
+    }
+    clipped = map(range(gradient.size), keep);
+}
+""")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib = tmp_path / "clip_ops.so"
+    r = subprocess.run([sys.executable, "-m", "hipress_amd.compll", str(prog), "-b", "--library", str(lib)], cwd=root,
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-3000:]
+    assert lib.exists() and json.loads((tmp_path / "clip_ops.so.json").read_text())["ClipScale"]["launches"] == ["map_float"]
+    ops = runtime.Operators(str(lib))
+    assert callable(ops.ClipScale) and [p["name"] for p in ops.manifest["ClipScale"]["params"]] == ["gradient", "clipped", "bound"]
+    with pytest.raises(TypeError):
+        ops.ClipScale(1, 2, 3, 4)  # argument checks come before anything touches a GPU
+    # the reference's wrapper / registration flags have nothing to generate here and say so
+    r = subprocess.run([sys.executable, "-m", "hipress_amd.compll", str(prog), "-w", "-r", "-f", "mxnet"], cwd=root,
+                       capture_output=True, text=True)
+    assert r.returncode == 2 and "Operators" in r.stderr

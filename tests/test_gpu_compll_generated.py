@@ -193,3 +193,42 @@ def test_generated_ops_report_errors(ops):
     out = torch.full((50,), 7.0, device="cuda")
     ops.MinMaxQuantDecode(bad, out)
     assert (host(out) == 7.0).all()
+
+
+# ---------------------------------------------------------------- the reference's own programs
+@pytest.fixture(scope="module")
+def reference_ops():
+    """The operators compiled from the reference checkout's own two programs, unmodified
+    (built on the machine that holds the checkout; the library travels, the checkout does not)."""
+    import os
+
+    from hipress_amd.compll import runtime
+    from hipress_amd.compll.build import REFERENCE_LIB
+
+    if not os.path.exists(REFERENCE_LIB):
+        pytest.skip("the reference checkout's programs were not built on this tree")
+    return runtime.Operators(REFERENCE_LIB)
+
+
+@pytest.mark.parametrize("b", [1, 2, 4, 8])
+@pytest.mark.parametrize("n", [1, 5, 4097, 262144, 1000003])
+def test_the_reference_s_own_programs_match_the_oracle(reference_ops, n, b):
+    """TernGradEncode(gradient, compressed, bitwidth) / TernGradDecode(compressed, gradient) as
+    the reference's generator registers them, generated here from its own program text: payload
+    byte for byte against the oracle (which follows the same program), decode value for value."""
+    import hipress_amd as hp
+
+    rng = np.random.default_rng(77 * b + n)
+    g = rng.normal(0, 1e-3, n).astype(F)
+    u = rng.random(n, dtype=F)
+    want = oracle.compll_encode(g, u, b)
+    pay = torch.full((want.size,), 0xAB, dtype=torch.uint8, device="cuda")
+    reference_ops.TernGradEncode(dev(g), pay, b, uniform=dev(u))
+    np.testing.assert_array_equal(host(pay), want)
+    out = torch.full((n,), 7.0, device="cuda")
+    reference_ops.TernGradDecode(pay, out)
+    dec = oracle.compll_decode(want, n)
+    k = hp.compll_decoded_count(n, b)
+    assert dec.size == k
+    np.testing.assert_array_equal(host(out)[:k], dec)
+    assert (host(out)[k:] == 7.0).all()
