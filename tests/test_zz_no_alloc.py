@@ -145,3 +145,32 @@ def test_static_scratch_array_holds_exactly_the_largest_tensor():
     assert int(L.hipress_onebit_workspace_bytes(STATIC_MAX_N)) >= 65536 * 4
     fake = ctypes.c_void_p(1 << 20)
     assert L.hipress_onebit_encode_static(fake, fake, STATIC_MAX_N + 1, fake, 16 + 4 * ((STATIC_MAX_N + 32) // 32), None) == -2
+
+
+def test_static_scratch_encode_at_the_largest_size_its_array_holds():
+    """n = 2^28: all 65,536 words of the array are in use (the last tile's sum is its last
+    word).  Payload and residual equal the workspace encoder's; one more element is refused."""
+    import torch
+
+    from hipress_amd import _lib
+
+    L = _lib.lib()
+    n = STATIC_MAX_N
+    nbytes = int(L.hipress_onebit_payload_bytes(n))
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    g = torch.randn(n, generator=gen, device="cuda") * 0.01
+    g[-4096:] *= 50.0  # the last tile carries weight in the scale: leaving its word out would show
+    r_ref, r_new = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    p_ref = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    p_new = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    ws = torch.empty(int(L.hipress_onebit_workspace_bytes(n)), dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    assert L.hipress_onebit_encode(g.data_ptr(), r_ref.data_ptr(), n, p_ref.data_ptr(), nbytes, ws.data_ptr(), ws.numel(), stream) == 0
+    assert L.hipress_onebit_encode_static(g.data_ptr(), r_new.data_ptr(), n, p_new.data_ptr(), nbytes, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(p_ref, p_new)
+    assert torch.equal(r_ref.view(torch.int32), r_new.view(torch.int32))
+    scale = float(p_new[:4].view(torch.float32).item())
+    want = float(g.abs().double().mean().item())
+    assert abs(scale - want) <= 1e-5 * want
+    assert L.hipress_onebit_encode_static(g.data_ptr(), r_new.data_ptr(), n + 1, p_new.data_ptr(), nbytes + 4, stream) == -2
