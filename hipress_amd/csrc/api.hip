@@ -21,7 +21,9 @@ namespace {
 constexpr int64_t kSampleTile = 4096;    // sample keys per workgroup of the select passes
 
 inline bool mis(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
-inline bool al16(const void* p) { return !mis(p, 16); }
+// The 16-byte vector path of the kernels needs dword alignment only (common.h: f4u), which
+// every fp32 pointer has once it has passed the 4-byte check.
+inline bool vec_ok(const void* p) { return !mis(p, 4); }
 inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 inline unsigned tiles_of(int64_t n) { return n <= 0 ? 1u : (unsigned)((n + kTile - 1) / kTile); }
 inline bool bad_n(int64_t n) { return n < 0 || n > HIPRESS_MAX_N; }
@@ -166,20 +168,20 @@ int build_encode_seg(int alg, const hipress_tensor& t, const hipress_params& pr,
     s->pay = static_cast<uint8_t*>(t.payload);
     s->n = (unsigned long long)t.n;
     s->ntiles = tiles_of(t.n);
-    s->aligned = al16(t.grad);
+    s->aligned = vec_ok(t.grad);
     switch (alg) {
         case HIPRESS_ONEBIT:
         case HIPRESS_ONEBIT_DEFERRED:
         case HIPRESS_TBQ:
             s->s0 = t.state0;
             s->s1 = alg == HIPRESS_ONEBIT_DEFERRED ? t.state1 : nullptr;
-            s->aligned = s->aligned && al16(t.state0);
+            s->aligned = s->aligned && vec_ok(t.state0);
             s->f0 = pr.threshold;
             s->words_off = HIPRESS_HEADER_BYTES;
             break;
         case HIPRESS_TERNGRAD: {
             s->u = t.uniform;
-            s->aligned = s->aligned && al16(t.uniform);
+            s->aligned = s->aligned && vec_ok(t.uniform);
             s->bucket = (unsigned)pr.bucket;
             int64_t off = HIPRESS_HEADER_BYTES + tg_scale_bytes(t.n, pr.bucket);
             if (off > 0xffffffffLL) return HIPRESS_ERR_SIZE;
@@ -192,11 +194,11 @@ int build_encode_seg(int alg, const hipress_tensor& t, const hipress_params& pr,
                 s->s0 = t.state0;
                 s->s1 = t.state1;
                 s->f0 = pr.momentum_factor;
-                s->aligned = s->aligned && al16(t.state0) && al16(t.state1);
+                s->aligned = s->aligned && vec_ok(t.state0) && vec_ok(t.state1);
             } else {
                 s->s0 = nullptr;
                 s->s1 = t.state0;
-                s->aligned = s->aligned && al16(t.state0);
+                s->aligned = s->aligned && vec_ok(t.state0);
             }
             SparsePlan p = sparse_plan(t.n, pr.ratio);
             s->cap = (unsigned)p.cap;
@@ -221,7 +223,7 @@ int build_decode_seg(int alg, const void* payload, int64_t payload_bytes, float*
     s->out = out;
     s->n = (unsigned long long)n;
     s->ntiles = tiles_of(n);
-    s->aligned = al16(out);
+    s->aligned = vec_ok(out);
     s->words_off = HIPRESS_HEADER_BYTES;
     switch (alg) {
         case HIPRESS_ONEBIT:
@@ -594,7 +596,7 @@ int hipress_compll_encode(const float* grad, const float* uniform, int64_t n, vo
     s.pay = static_cast<uint8_t*>(compressed);
     s.n = (unsigned long long)n;
     s.ntiles = tiles_of(n);
-    s.aligned = al16(grad) && al16(uniform);
+    s.aligned = vec_ok(grad) && vec_ok(uniform);
     s.bucket = (unsigned)bitwidth;
     return hiperr(launch_compll_encode(single_launch(s), bitwidth, static_cast<float*>(workspace),
                                        static_cast<hipStream_t>(stream)));
@@ -612,7 +614,7 @@ int hipress_compll_decode(const void* compressed, int64_t compressed_bytes, floa
     s.out = out;
     s.n = (unsigned long long)n;
     s.ntiles = tiles_of(n);
-    s.aligned = al16(out);
+    s.aligned = vec_ok(out);
     return hiperr(launch_compll_decode(single_launch(s), static_cast<hipStream_t>(stream)));
 }
 
@@ -683,7 +685,7 @@ static int build_merge_seg(int alg, const void* const* payloads, const int64_t* 
     m->s.out = aggregate;
     m->s.n = (unsigned long long)n;
     m->s.ntiles = tiles_of(n);
-    m->s.aligned = al16(aggregate) && al16(local);
+    m->s.aligned = vec_ok(aggregate) && vec_ok(local);
     return HIPRESS_OK;
 }
 
@@ -715,7 +717,7 @@ static int add_tbq_reencode(MergeSeg* m, float* residual, void* out_payload, int
     m->s.s0 = residual;
     m->s.pay = static_cast<uint8_t*>(out_payload);
     m->s.f0 = threshold;
-    m->s.aligned = m->s.aligned && al16(residual);
+    m->s.aligned = m->s.aligned && vec_ok(residual);
     return HIPRESS_OK;
 }
 

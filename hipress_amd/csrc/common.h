@@ -43,7 +43,7 @@ struct Seg {
     unsigned int ntiles;     // tiles of this tensor
     unsigned int words_off;  // byte offset of the packed words from the payload base
     unsigned int bucket;     // terngrad bucket size
-    unsigned int aligned;    // 1 when every pointer used is 16-byte aligned
+    unsigned int aligned;    // 1 when the 16-byte vector path may be used (every fp32 pointer a multiple of 4)
     unsigned int cap;        // sparse capacity
     float f0;                // tbq threshold | dgc momentum factor
     unsigned int ks;         // sparse: rank of the threshold inside the sample
@@ -134,14 +134,19 @@ struct MergeBatchSrc {
 #ifdef __HIPCC__
 // ---- memory access ---------------------------------------------------------
 // Streaming data is touched exactly once, so loads and stores carry the
-// non-temporal hint.
+// non-temporal hint.  The fp32 arrays need only be 4-byte aligned: a 16-byte access to
+// global memory is one instruction at any dword address (the vector type below says
+// "aligned to 4", and the compiler emits the same global_load_dwordx4 / global_store_dwordx4
+// for it as for a 16-byte aligned one), so a view that starts a few floats into an
+// allocation takes the same path as the allocation itself.
+typedef f4 f4u __attribute__((aligned(4)));
 __device__ __forceinline__ f4 ld4(const float* p) {
-    return __builtin_nontemporal_load(reinterpret_cast<const f4*>(p));
+    return __builtin_nontemporal_load(reinterpret_cast<const f4u*>(p));
 }
 __device__ __forceinline__ void st4(float* p, f4 v) {
-    __builtin_nontemporal_store(v, reinterpret_cast<f4*>(p));
+    __builtin_nontemporal_store(v, reinterpret_cast<f4u*>(p));
 }
-// Element-wise variants for partial tiles and pointers that are only 4-byte aligned.
+// Element-wise variants for partial tiles.
 __device__ __forceinline__ f4 ld4_guard(const float* p, long long e, long long n) {
     f4 v = {0.f, 0.f, 0.f, 0.f};
     if (e < n) v.x = p[e];
@@ -236,7 +241,7 @@ __device__ __forceinline__ bool cache_tail(unsigned b, unsigned nblocks, unsigne
 // otherwise identical branch of streamed ones, which would make all of them plain.)
 __device__ __forceinline__ f4 ld4_keep(const float* p) {
     asm volatile("");
-    return *reinterpret_cast<const f4*>(p);
+    return *reinterpret_cast<const f4u*>(p);
 }
 
 // ---- cross-lane -------------------------------------------------------------

@@ -22,6 +22,9 @@
 namespace cl {
 
 typedef float f4 __attribute__((ext_vector_type(4)));
+// 16 bytes at any dword address: one global_load_dwordx4 / global_store_dwordx4 either way,
+// so float vectors need only the alignment of a float
+typedef f4 f4u __attribute__((aligned(4)));
 
 constexpr int kBlock = 256;   // threads per workgroup (four wave64 wavefronts)
 constexpr int kTile = 4096;   // elements per workgroup in the sweeps
@@ -102,16 +105,16 @@ __device__ __forceinline__ void load_streams_as(const Args& a, long long base, l
 #pragma unroll
     for (int k = 0; k < Fn::NS; ++k) {
         const float* p = Fn::stream(a, k);
-        const bool vec_ok = (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+        const bool vec_ok = (reinterpret_cast<uintptr_t>(p) & 3u) == 0;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const long long e = base + j * 256;
             if (e + 3 < count && vec_ok) {
                 if (KEEP) {
                     asm volatile("");
-                    x[k][j] = *reinterpret_cast<const f4*>(p + e);
+                    x[k][j] = *reinterpret_cast<const f4u*>(p + e);
                 } else {
-                    x[k][j] = __builtin_nontemporal_load(reinterpret_cast<const f4*>(p + e));
+                    x[k][j] = __builtin_nontemporal_load(reinterpret_cast<const f4u*>(p + e));
                 }
             } else {
                 x[k][j].x = e < count ? p[e] : 0.f;
@@ -369,7 +372,7 @@ __global__ __launch_bounds__(kBlock) void map_float_kernel(Args a, Dev* dglobal,
     if (count > cap) count = cap;
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long base = (long long)blockIdx.x * kTile + wave * 1024 + lane * 4;
-    const bool vec_ok = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
+    const bool vec_ok = (reinterpret_cast<uintptr_t>(out) & 3u) == 0;
     f4 x[Fn::NS > 0 ? Fn::NS : 1][4];
     load_streams<Args, Fn>(a, base, count, x);
 #pragma unroll
@@ -386,7 +389,7 @@ __global__ __launch_bounds__(kBlock) void map_float_kernel(Args a, Dev* dglobal,
             q.y = Fn::call(a, *d, e + 1, s[1]);
             q.z = Fn::call(a, *d, e + 2, s[2]);
             q.w = Fn::call(a, *d, e + 3, s[3]);
-            __builtin_nontemporal_store(q, reinterpret_cast<f4*>(out + e));
+            __builtin_nontemporal_store(q, reinterpret_cast<f4u*>(out + e));
         } else {
             for (int c = 0; c < 4; ++c)
                 if (e + c < count) out[e + c] = Fn::call(a, *d, e + c, s[c]);
@@ -457,7 +460,7 @@ __global__ __launch_bounds__(kBlock) void map_fused_kernel(Args a, Dev* dglobal,
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long base = (long long)tile_reversed(blockIdx.x, gridDim.x) * kTile + wave * 1024 + lane * 4;
     if (base - lane * 4 >= count) return;  // the whole wavefront leaves together
-    const bool vec_ok = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
+    const bool vec_ok = (reinterpret_cast<uintptr_t>(out) & 3u) == 0;
     f4 x[Fn::NS > 0 ? Fn::NS : 1][4];
     load_streams<Args, Fn>(a, base, count, x);
 #pragma unroll
@@ -478,7 +481,7 @@ __global__ __launch_bounds__(kBlock) void map_fused_kernel(Args a, Dev* dglobal,
             q.z = Fn::call_values(a, *d, e + 2, s[2]);
             q.w = Fn::call_values(a, *d, e + 3, s[3]);
             if (vec_ok) {
-                __builtin_nontemporal_store(q, reinterpret_cast<f4*>(out + e));
+                __builtin_nontemporal_store(q, reinterpret_cast<f4u*>(out + e));
             } else {
                 out[e] = q.x;
                 out[e + 1] = q.y;

@@ -306,7 +306,7 @@ __global__ __launch_bounds__(kBlock) void sparse_select_kernel(Src src, SparseWs
 // The 16 lanes of a DPP row read one 64-element group as 16-byte vectors; a
 // wavefront therefore works on four flagged groups per load instruction.
 __device__ __forceinline__ f4 load_group4(const float* p, long long e, long long n, bool aligned) {
-    if (aligned && e + 3 < n) return *reinterpret_cast<const f4*>(p + e);
+    if (aligned && e + 3 < n) return *reinterpret_cast<const f4u*>(p + e);
     return ld4_guard(p, e, n);
 }
 
@@ -680,11 +680,11 @@ __global__ __launch_bounds__(kBlock) void sparse_emit_kernel(Src src, SparseWs w
                 if (s2) { idx[p] = (int32_t)(e + 2); val[p] = v.z; keep.z = 0.f; ++p; }
                 if (s3) { idx[p] = (int32_t)(e + 3); val[p] = v.w; keep.w = 0.f; ++p; }
                 if (aligned && e + 3 < n) {
-                    *reinterpret_cast<f4*>(s.s1 + e) = keep;
+                    *reinterpret_cast<f4u*>(s.s1 + e) = keep;
                     if (s.s0) {
-                        f4 m = *reinterpret_cast<const f4*>(s.s0 + e);
+                        f4 m = *reinterpret_cast<const f4u*>(s.s0 + e);
                         m.x = s0 ? 0.f : m.x; m.y = s1 ? 0.f : m.y; m.z = s2 ? 0.f : m.z; m.w = s3 ? 0.f : m.w;
-                        *reinterpret_cast<f4*>(s.s0 + e) = m;
+                        *reinterpret_cast<f4u*>(s.s0 + e) = m;
                     }
                 } else {
                     if (s0) { clear_element<STREAM>(&s.s1[e]); if (s.s0) clear_element<STREAM>(&s.s0[e]); }

@@ -3,7 +3,9 @@
  *
  * One shared library, libhipress_amd.so, exports everything declared here with
  * C linkage.  All pointers named grad/residual/momentum/accumulator/uniform/
- * payload/out/aggregate/workspace are DEVICE pointers owned by the caller;
+ * payload/out/aggregate/workspace are DEVICE pointers owned by the caller (fp32
+ * arrays 4-byte aligned - a view a few floats into a flat buffer runs on the same
+ * 16-byte vector path as the buffer itself; payloads and workspaces 16-byte aligned);
  * `stream` is a hipStream_t passed as void* (NULL = the default stream), the
  * way the reference carries its stream
  * (/root/reference/src/CompLL/GCGen/output/get_policy_general.h:125-133,

@@ -1,6 +1,6 @@
 """GPU parity on the inputs a gradient set does not normally hold: NaN, +-Inf, +-0,
 denormals and FLT_MAX mixed into ordinary data, buckets whose elements are all equal,
-pointers that are only 4-byte aligned (every guarded code path), and empty tensors -
+pointers that are only 4-byte aligned (16-byte vector accesses at dword addresses), and empty tensors -
 each compressor and both merges against the CPU oracle, through the C ABI.
 
 Floats are compared value for value with NaN equal to NaN (the bits of a NaN that an
@@ -355,8 +355,9 @@ def test_onebit_deferred_special_values_three_steps(hp, kind):
 
 @pytest.mark.parametrize("n", [9001, 70003])
 def test_onebit_deferred_unaligned_views_three_steps(hp, n):
-    """Gradient, state and residual output only 4-byte aligned (the element-wise path of the
-    one-pass kernel and of hipress_onebit_residual), three steps with the state carried."""
+    """Gradient, state and residual output only 4-byte aligned (16-byte accesses at dword
+    addresses in the one-pass kernel and in hipress_onebit_residual), three steps with the
+    state carried."""
     rng = np.random.default_rng(n + 1)
     r0 = rng.normal(0, 1e-3, n).astype(F)
     gs = [rng.normal(0, 1e-3, n).astype(F) for _ in range(3)]
