@@ -656,17 +656,23 @@ def _warm_up(w, warmup, min_seconds):
             w.step()
             done += 1
         torch.cuda.synchronize()
-    return done
+    return done, time.perf_counter() - t0
 
 
-def measure(name, steps, warmup, cpu_budget_s=0.0, min_warmup_s=0.25):
+def measure(name, steps, warmup, cpu_budget_s=0.0, min_warmup_s=0.25, min_timed_s=0.0):
+    """One workload's record.  The timed region is exactly `steps` steps; with min_timed_s the
+    number of steps is raised until the region lasts about that long (judged by the warm-up's
+    rate), so that the two synchronisations around it, tens of microseconds, do not decide the
+    figure of a workload whose step takes a few microseconds."""
     import torch
 
     dev = torch.device("cuda:0")
     graph = name.endswith("_graph")
     w = make_workload(name[: -len("_graph")] if graph else name)
     w.setup(dev)
-    warm_steps = _warm_up(w, warmup, min_warmup_s)
+    warm_steps, warm_s = _warm_up(w, warmup, min_warmup_s)
+    if min_timed_s > 0 and warm_steps and warm_s > 0:
+        steps = max(steps, min(5000, -(-int(min_timed_s * 1e6) // max(1, int(warm_s / warm_steps * 1e6)))))
     captured = None
     if graph:  # one step captured on a side stream; every later step is one graph launch
         side = torch.cuda.Stream()
@@ -720,6 +726,7 @@ def measure(name, steps, warmup, cpu_budget_s=0.0, min_warmup_s=0.25):
     alg_gbs = (enc_b + dec_b) * w.elements * steps / elapsed / 1e9
     res = {
         "workload": name,
+        "steps": steps,
         "warmup_steps_run": warm_steps,
         "value": gbs,
         "ms_per_step": elapsed / steps * 1e3,
@@ -839,6 +846,9 @@ def main():
     ap.add_argument("--others-cpu-seconds", type=float, default=2.0, help="one-thread CPU budget of every other workload")
     ap.add_argument("--min-warmup-ms", type=float, default=250.0,
                     help="keep warming up (beyond --warmup steps) until the GPU has been busy this long")
+    ap.add_argument("--others-min-timed-ms", type=float, default=2.0,
+                    help="every other workload is timed over at least --others-steps steps and about this long "
+                         "(the headline over exactly --steps)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 1 GiB device-to-device copy (a kernel of known traffic: 1 GiB read, "
                          "1 GiB written) so that rocprofv3 FETCH_SIZE / WRITE_SIZE can be scaled against it")
@@ -876,7 +886,7 @@ def main():
         for name in ALL_WORKLOADS:
             if name != args.workload:
                 others.append(record(measure(name, args.others_steps, 3, 0.0 if args.no_cpu else args.others_cpu_seconds,
-                                             args.min_warmup_ms * 1e-3)))
+                                             args.min_warmup_ms * 1e-3, min_timed_s=args.others_min_timed_ms * 1e-3)))
     line = compact_line(main_res, others, args.steps, args.warmup)
     detail = {"headline": main_res, "others": others}
     try:  # the full records also go to a file next to the other run outputs
