@@ -1041,6 +1041,9 @@ static int merge_batch_create_impl(hipress_merge_batch** out, int32_t alg, const
         const hipress_merge_chunk& c = chunks[i];
         MergeSeg m;
         if ((rc = build_merge_seg(alg, c.payloads, c.payload_bytes, npeers, c.local, c.aggregate, c.n, b->reencode, &m))) return fail(rc);
+        // terngrad: the bucket size the peers are expected to have used lets the kernel ask for their
+        // words before it has seen their headers (which still decide when they say otherwise)
+        if (alg == HIPRESS_TERNGRAD && params->bucket >= 1) m.s.bucket = (unsigned)params->bucket;
         if (b->reencode && alg == HIPRESS_TBQ) {
             if ((rc = add_tbq_reencode(&m, c.state, c.out_payload, c.out_payload_bytes, params->threshold))) return fail(rc);
         }

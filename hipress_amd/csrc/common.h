@@ -244,6 +244,31 @@ __device__ __forceinline__ f4 ld4_keep(const float* p) {
     return *reinterpret_cast<const f4u*>(p);
 }
 
+// ---- bucket arithmetic --------------------------------------------------------
+// Element first + off (off < 8192) lies in bucket q, at place r inside it, given that element
+// `first` lies in bucket q0 at place r0 and buckets hold B elements: a 32-bit division, or a
+// comparison when a bucket is longer than the stretch looked at.  The 64-bit division that
+// places `first` is done once per wavefront on uniform values; per element it would cost more
+// than everything else a decoder does.
+struct BucketPos {
+    long long q;
+    unsigned long long r;
+};
+__device__ __forceinline__ BucketPos bucket_pos(long long q0, unsigned long long r0, unsigned off, unsigned long long B) {
+    const unsigned long long x = r0 + off;
+    BucketPos p;
+    if (B <= 8192ull) {
+        const unsigned xq = (unsigned)x / (unsigned)B;
+        p.q = q0 + xq;
+        p.r = x - (unsigned long long)xq * B;
+    } else {
+        const bool over = x >= B;
+        p.q = q0 + (over ? 1 : 0);
+        p.r = over ? x - B : x;
+    }
+    return p;
+}
+
 // ---- cross-lane -------------------------------------------------------------
 // quad_perm broadcast of lane k of every group of four lanes (DPP, no LDS traffic)
 template <int K>

@@ -480,7 +480,116 @@ __global__ __launch_bounds__(kBlock) void terngrad_encode_kernel(Src src) {
     else terngrad_encode_tile<false, BPW>(s, tile);
 }
 
-// Any other bucket size: one wavefront per bucket writes the scale ...
+// Any other bucket size up to a tile (4096): still a single pass.  A tile's elements lie in
+// the buckets b_first .. b_last; the first of them may have begun in the tile before and the
+// last may end in the tile behind, by less than a bucket each, so the workgroup also reads
+// those two stretches of the gradient (nothing else of the neighbours) and so knows the
+// maximum of every bucket its own elements need.  Maxima meet in LDS as integer keys (the
+// bit pattern of |g| orders like |g|; values that are no number leave no key, as fmaxf
+// passes them over).  A bucket's scale is written by the tile it begins in.
+constexpr unsigned kAnyBucketMax = kTile;
+constexpr unsigned kAnyBuckets = kTile + 2;  // bucket size 1: every element its own, plus none hanging over
+
+__device__ __forceinline__ unsigned absmax_key(float x) {
+    const unsigned k = __float_as_uint(x) & 0x7fffffffu;
+    return k > 0x7f800000u ? 0u : k;  // NaN contributes nothing
+}
+
+template <bool FAST>
+__device__ __forceinline__ void terngrad_encode_any_tile(const Seg& s, unsigned tile, unsigned* mx) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const unsigned B = s.bucket;
+    const long long t0 = (long long)tile * kTile, t1 = t0 + kTile < n ? t0 + kTile : n;
+    const long long b_first = t0 / B, b_last = (t1 - 1) / B;
+    const long long start = b_first * B;                                         // <= t0
+    const long long end = (b_last + 1) * B < n ? (b_last + 1) * B : n;           // >= t1
+    const unsigned nb = (unsigned)(b_last - b_first + 1);
+    const unsigned head = (unsigned)(t0 - start);                                // elements of bucket b_first in front of the tile
+    float* scales = reinterpret_cast<float*>(s.pay + kHeaderBytes);
+    uint32_t* words = reinterpret_cast<uint32_t*>(s.pay + s.words_off);
+    for (unsigned i = threadIdx.x; i < nb; i += kBlock) mx[i] = 0u;
+    // the tile's own elements, requested before anything waits
+    const long long base = t0 + wave * kWaveTile;
+    f4 g[4], u[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const long long e = base + j * 256 + lane * 4;
+        g[j] = load4<FAST>(s.g, e, n);
+        u[j] = load4<FAST>(s.u, e, n);
+    }
+    __syncthreads();
+    // what hangs over from the neighbours: fewer than B elements on either side
+    for (long long i = start + threadIdx.x; i < t0; i += kBlock) atomicMax(&mx[0], absmax_key(s.g[i]));
+    for (long long i = t1 + threadIdx.x; i < end; i += kBlock) atomicMax(&mx[nb - 1], absmax_key(s.g[i]));
+    // local bucket and place inside it of each step's first element: one 32-bit division per step
+    unsigned lb[4], rem[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const unsigned x = head + wave * kWaveTile + j * 256 + lane * 4;  // < 2 * kTile
+        lb[j] = x / B;
+        rem[j] = x - lb[j] * B;
+        const float v[4] = {g[j].x, g[j].y, g[j].z, g[j].w};
+        const long long e = base + j * 256 + lane * 4;
+        if (rem[j] + 3u < B) {  // the four elements share a bucket
+            if (e < n) atomicMax(&mx[lb[j]], absmax_key(absmax4(g[j])));  // elements beyond n were loaded as zero
+        } else {
+            unsigned b = lb[j], r = rem[j];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                if (e + k < n) atomicMax(&mx[b], absmax_key(v[k]));
+                if (++r == B) { r = 0; ++b; }
+            }
+        }
+    }
+    __syncthreads();
+    // scales of the buckets that begin in this tile
+    for (unsigned i = (head ? 1u : 0u) + threadIdx.x; i < nb; i += kBlock) scales[b_first + i] = __uint_as_float(mx[i]);
+    if (base >= n) return;
+    unsigned myword = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        unsigned byte;
+        if (rem[j] + 3u < B) {
+            byte = tern_code4(g[j], u[j], __uint_as_float(mx[lb[j]]));  // pad elements are 0: u*s < 0 is false
+        } else {
+            const float gv[4] = {g[j].x, g[j].y, g[j].z, g[j].w}, uv[4] = {u[j].x, u[j].y, u[j].z, u[j].w};
+            unsigned b = lb[j], r = rem[j];
+            byte = 0;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                // a pad element may index one bucket past the last: its code is 0 whatever the scale
+                const float sc = b < nb ? __uint_as_float(mx[b]) : 0.f;
+                byte |= tern_code(gv[k], uv[k], sc) << (2 * k);
+                if (++r == B) { r = 0; ++b; }
+            }
+        }
+        const unsigned w = quad_pack8(byte);
+        myword = ((lane & 3u) == (unsigned)j) ? w : myword;
+    }
+    const long long widx = (base >> 4) + (lane & 3u) * 16 + (lane >> 2);
+    if (FAST || widx < (long long)((n + 15) >> 4)) words[widx] = myword;
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void terngrad_encode_any_kernel(Src src) {
+    __shared__ unsigned mx[kAnyBuckets];
+    unsigned tile;
+    const Seg s = src.get(tile, blockIdx.x);
+    if (tile == 0 && threadIdx.x == 0) {
+        uint32_t* h = reinterpret_cast<uint32_t*>(s.pay);
+        h[0] = (uint32_t)s.n;
+        h[1] = s.bucket;
+        h[2] = 0;
+        h[3] = 0;
+    }
+    terngrad_zero_scale_pad(s, tile);
+    if ((unsigned long long)tile * kTile >= s.n) return;  // an empty tensor has one tile and nothing in it
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) terngrad_encode_any_tile<true>(s, tile, mx);
+    else terngrad_encode_any_tile<false>(s, tile, mx);
+}
+
+// Bucket sizes beyond a tile: one wavefront per bucket writes the scale ...
 template <class Src>
 __global__ __launch_bounds__(kBlock) void terngrad_scale_generic_kernel(Src src) {
     // grid: tiles of the tensor; each workgroup walks the buckets that START in its tile
@@ -561,6 +670,10 @@ __device__ __forceinline__ void terngrad_decode_tile(const Seg& s, unsigned tile
         b[j] = (w >> (8 * (lane & 3u))) & 0xffu;
     }
     float sc4[4] = {0.f, 0.f, 0.f, 0.f};
+    // the tile's first element: its bucket and its place in it (not needed when every step lies in one bucket)
+    const long long tile0 = (long long)tile * kTile;
+    const long long tq0 = BUCKET256 ? 0 : tile0 / B;
+    const unsigned long long tr0 = BUCKET256 ? 0ull : (unsigned long long)(tile0 - tq0 * B);
     if (BUCKET256) {
         // one division per wavefront: the four steps start 0, 256, 512, 768 elements
         // further on and B >= 256, so each step is at most three buckets ahead
@@ -580,10 +693,18 @@ __device__ __forceinline__ void terngrad_decode_tile(const Seg& s, unsigned tile
         if (BUCKET256) {
             o = expand2(b[j], sc4[j]);
         } else {
-            o.x = (e < n && b[j]) ? code_value(b[j] & 3u, scales[e / B]) : 0.f;
-            o.y = (e + 1 < n && b[j]) ? code_value((b[j] >> 2) & 3u, scales[(e + 1) / B]) : 0.f;
-            o.z = (e + 2 < n && b[j]) ? code_value((b[j] >> 4) & 3u, scales[(e + 2) / B]) : 0.f;
-            o.w = (e + 3 < n && b[j]) ? code_value((b[j] >> 6) & 3u, scales[(e + 3) / B]) : 0.f;
+            // bucket of the lane's first element from the tile's; the other three follow by counting
+            const BucketPos bp = bucket_pos(tq0, tr0, (unsigned)(wave * kWaveTile + j * 256 + lane * 4), (unsigned long long)B);
+            long long q = bp.q;
+            unsigned long long r = bp.r;
+            float ov[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const unsigned c = (b[j] >> (2 * k)) & 3u;
+                ov[k] = (e + k < n && c) ? code_value(c, scales[q]) : 0.f;
+                if (++r == (unsigned long long)B) { r = 0; ++q; }
+            }
+            o.x = ov[0]; o.y = ov[1]; o.z = ov[2]; o.w = ov[3];
         }
         store4<FAST>(s.out, e, n, o);
     }
@@ -618,6 +739,7 @@ __global__ __launch_bounds__(kBlock) void terngrad_decode_kernel(Src src) {
     const bool b256 = (B & 255) == 0;
     if (fast && b256) terngrad_decode_tile<true, true>(s, tile, B, words, false);
     else if (b256) terngrad_decode_tile<false, true>(s, tile, B, words, false);
+    else if (fast) terngrad_decode_tile<true, false>(s, tile, B, words, false);
     else terngrad_decode_tile<false, false>(s, tile, B, words, false);
 }
 
@@ -716,6 +838,7 @@ static hipError_t terngrad_encode_src(const Src& src, unsigned ntiles, unsigned 
     if (bucket == 256) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 4>), dim3(ntiles), dim3(kBlock), kLdsFor5, st, src);
     else if (bucket == 512) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 2>), dim3(ntiles), dim3(kBlock), kLdsFor5, st, src);
     else if (bucket == 1024) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 1>), dim3(ntiles), dim3(kBlock), kLdsFor5, st, src);
+    else if (bucket <= kAnyBucketMax) hipLaunchKernelGGL((terngrad_encode_any_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);
     else {
         hipLaunchKernelGGL((terngrad_scale_generic_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);
         hipLaunchKernelGGL((terngrad_quant_generic_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);

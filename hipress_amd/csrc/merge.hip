@@ -51,15 +51,11 @@ __device__ __forceinline__ void merge_tile(const MergeSeg& m, unsigned tile, int
     for (int p0 = 0; p0 < npeers; p0 += kPeerChunk) {
         uint32_t wq[kPeerChunk];
         float sc[kPeerChunk];                // onebit: scale, tbq: threshold
-        const float* scales[kPeerChunk];     // terngrad
-        long long bucket[kPeerChunk];
         bool use[kPeerChunk];
 #pragma unroll
         for (int q = 0; q < kPeerChunk; ++q) {
             wq[q] = 0u;
             sc[q] = 0.f;
-            scales[q] = nullptr;
-            bucket[q] = 1;
             use[q] = p0 + q < npeers;
             if (!use[q]) continue;
             const uint8_t* pay = m.peer[p0 + q];
@@ -76,17 +72,8 @@ __device__ __forceinline__ void merge_tile(const MergeSeg& m, unsigned tile, int
                     sc[q] = __uint_as_float(h[0]);
                     words = reinterpret_cast<const uint32_t*>(pay + kHeaderBytes);
                 } else {
-                    // bucket size from the header; a header that does not fit the buffer adds nothing
-                    const long long B = h[1];
-                    const unsigned long long nb = B >= 1 ? ((unsigned long long)n + B - 1) / B : 0;
-                    const unsigned long long off = kHeaderBytes + ((4 * nb + 15) & ~15ull);
-                    if (B < 1 || off + 4 * (unsigned long long)nwords > m.peer_bytes[p0 + q]) {
-                        use[q] = false;
-                        continue;
-                    }
-                    bucket[q] = B;
-                    scales[q] = reinterpret_cast<const float*>(pay + kHeaderBytes);
-                    words = reinterpret_cast<const uint32_t*>(pay + off);
+                    static_assert(ALG != HIPRESS_TERNGRAD, "terngrad has a tile function of its own");
+                    words = nullptr;
                 }
                 const long long widx = (base >> 4) + lane;
                 if (FAST || widx < nwords) wq[q] = words[widx];
@@ -111,14 +98,6 @@ __device__ __forceinline__ void merge_tile(const MergeSeg& m, unsigned tile, int
                     const unsigned byte = (w >> (8 * (lane & 3u))) & 0xffu;
                     if (ALG == HIPRESS_TBQ) {
                         agg[j] = agg[j] + expand_codes(byte, sc[q]);
-                    } else {
-                        const long long e = base + j * 256 + lane * 4, B = bucket[q];
-                        f4 d;
-                        d.x = e < n ? code_val(byte & 3u, scales[q][e / B]) : 0.f;
-                        d.y = e + 1 < n ? code_val((byte >> 2) & 3u, scales[q][(e + 1) / B]) : 0.f;
-                        d.z = e + 2 < n ? code_val((byte >> 4) & 3u, scales[q][(e + 2) / B]) : 0.f;
-                        d.w = e + 3 < n ? code_val((byte >> 6) & 3u, scales[q][(e + 3) / B]) : 0.f;
-                        agg[j] = agg[j] + d;
                     }
                 }
             }
@@ -156,6 +135,179 @@ __device__ __forceinline__ void merge_tile(const MergeSeg& m, unsigned tile, int
     }
 }
 
+// ---- TernGrad peers --------------------------------------------------------------------
+// A TernGrad payload keeps one scale per bucket between its header and its words, so where the
+// words start, and which scale an element takes, follow from the bucket size in the header.
+// Everything here is arranged so that this costs one round trip to memory and a handful of
+// instructions per wavefront and tile, not per peer or per element:
+//  * n and the bucket size are 32-bit quantities; a power of two divides by shifting;
+//  * the peers of a launch normally share one bucket size.  The launch may name it
+//    (Seg::bucket; otherwise the first peer's header does), the geometry for it - where the words
+//    start, which bucket and place the wavefront's and each lane's first elements have - is
+//    worked out once, and words and scales of all peers are asked for from it straight away,
+//    together with the headers.  A header that names another size decides: that peer alone is
+//    set up again from its own header.
+struct TgGeom {
+    unsigned long long words_off;  // byte offset of the packed words from the payload base
+    unsigned q0, r0;               // bucket of the wavefront's first element, and that element's place in it
+    bool ok;                       // the bucket size is usable
+};
+
+__device__ __forceinline__ TgGeom tg_geom(unsigned B, unsigned n32, unsigned b32) {
+    TgGeom g;
+    g.ok = B >= 1u;
+    unsigned nb = 0u;
+    g.q0 = g.r0 = 0u;
+    if (g.ok) {
+        if ((B & (B - 1u)) == 0u) {
+            const unsigned sh = (unsigned)__ffs((int)B) - 1u;
+            nb = (n32 >> sh) + ((n32 & (B - 1u)) != 0u);
+            g.q0 = b32 >> sh;
+            g.r0 = b32 & (B - 1u);
+        } else {
+            nb = n32 / B + (n32 % B != 0u);
+            g.q0 = b32 / B;
+            g.r0 = b32 - g.q0 * B;
+        }
+    }
+    g.words_off = kHeaderBytes + ((4ull * nb + 15ull) & ~15ull);
+    return g;
+}
+
+// Bucket (pq) and place in it (pr) of the lane's first element in each of the four steps.
+__device__ __forceinline__ void tg_positions(const TgGeom& g, unsigned B, unsigned lane, unsigned (&pq)[4], unsigned (&pr)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if ((B & 255u) == 0u) {
+            // a step of 256 aligned elements lies inside one bucket, at most three on from the wavefront's first
+            const unsigned long long x = (unsigned long long)g.r0 + (unsigned)(j * 256);
+            pq[j] = g.q0 + (unsigned)(x >= B) + (unsigned)(x >= 2ull * B) + (unsigned)(x >= 3ull * B);
+            pr[j] = 0u;  // not used: every element of the step shares the bucket
+        } else {
+            const BucketPos bp = bucket_pos(g.q0, g.r0, (unsigned)(j * 256) + lane * 4u, B);
+            pq[j] = (unsigned)bp.q;
+            pr[j] = (unsigned)bp.r;
+        }
+    }
+}
+
+// Asks for one peer's word and for the scales of the lane's first elements; false when the
+// payload cannot hold what its bucket size implies (such a peer adds nothing).
+template <bool FAST>
+__device__ __forceinline__ bool tg_request(const uint8_t* pay, unsigned long long pay_bytes, const TgGeom& g,
+                                           const unsigned (&pq)[4], long long n, long long base, unsigned lane,
+                                           uint32_t& word, float (&sc)[4]) {
+    const long long nwords = (n + 15) >> 4;
+    word = 0u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sc[j] = 0.f;
+    if (!g.ok || g.words_off + 4ull * (unsigned long long)nwords > pay_bytes) return false;
+    const uint32_t* words = reinterpret_cast<const uint32_t*>(pay + g.words_off);
+    const float* scales = reinterpret_cast<const float*>(pay + kHeaderBytes);
+    const long long widx = (base >> 4) + lane;
+    if (FAST || widx < nwords) word = words[widx];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        if (base + j * 256 + lane * 4 < n) sc[j] = scales[pq[j]];
+    return true;
+}
+
+template <bool FAST, bool LOCAL>
+__device__ __forceinline__ void merge_tile_terngrad(const MergeSeg& m, unsigned tile, int npeers) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const Seg s = m.s;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    if (base >= n) return;
+    const unsigned n32 = (unsigned)n, b32 = (unsigned)base;
+    f4 agg[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        agg[j] = (f4){0.f, 0.f, 0.f, 0.f};
+        if (LOCAL && s.g) agg[j] = load4<FAST>(s.g, base + j * 256 + lane * 4, n);
+    }
+    constexpr int kPeerChunk = 8;  // two or four at a time are no faster: the adds, not the loads, bound this kernel
+    for (int p0 = 0; p0 < npeers; p0 += kPeerChunk) {
+        unsigned hb[kPeerChunk];  // bucket sizes as the headers have them
+#pragma unroll
+        for (int q = 0; q < kPeerChunk; ++q) {
+            hb[q] = 0u;
+            if (p0 + q < npeers) hb[q] = reinterpret_cast<const uint32_t*>(m.peer[p0 + q])[1];
+        }
+        // the size the peers are expected to share: named by the launch, else the first header's
+        const unsigned B0 = s.bucket ? s.bucket : (unsigned)__builtin_amdgcn_readfirstlane((int)hb[0]);
+        const TgGeom g0 = tg_geom(B0, n32, b32);
+        unsigned pq0[4], pr0[4];
+        tg_positions(g0, B0 ? B0 : 1u, lane, pq0, pr0);
+        uint32_t wq[kPeerChunk];
+        float tsc[kPeerChunk][4];
+        unsigned usemask = 0u;
+#pragma unroll
+        for (int q = 0; q < kPeerChunk; ++q) {
+            wq[q] = 0u;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) tsc[q][j] = 0.f;
+            if (p0 + q < npeers && tg_request<FAST>(m.peer[p0 + q], m.peer_bytes[p0 + q], g0, pq0, n, base, lane, wq[q], tsc[q]))
+                usemask |= 1u << q;
+        }
+        // the headers have their say: a peer of another bucket size is set up again from its own
+        unsigned ownmask = 0u;
+#pragma unroll
+        for (int q = 0; q < kPeerChunk; ++q) {
+            if (p0 + q < npeers && hb[q] != B0) {  // wavefront-uniform, rare
+                const TgGeom g = tg_geom(hb[q], n32, b32);
+                unsigned pq[4], pr[4];
+                tg_positions(g, hb[q] ? hb[q] : 1u, lane, pq, pr);
+                usemask &= ~(1u << q);
+                if (tg_request<FAST>(m.peer[p0 + q], m.peer_bytes[p0 + q], g, pq, n, base, lane, wq[q], tsc[q])) usemask |= 1u << q;
+                ownmask |= 1u << q;
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < kPeerChunk; ++q) {
+            if (!((usemask >> q) & 1u)) continue;  // wavefront-uniform
+            const bool own = (ownmask >> q) & 1u;
+            const unsigned B = own ? hb[q] : B0;
+            unsigned pq[4], pr[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                pq[j] = pq0[j];
+                pr[j] = pr0[j];
+            }
+            if (own) tg_positions(tg_geom(B, n32, b32), B, lane, pq, pr);
+            const float* scales = reinterpret_cast<const float*>(m.peer[p0 + q] + kHeaderBytes);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t w = (uint32_t)__shfl((int)wq[q], j * 16 + (int)(lane >> 2), 64);
+                const unsigned byte = (w >> (8 * (lane & 3u))) & 0xffu;
+                if ((B & 255u) == 0u || (unsigned long long)pr[j] + 3ull < B) {
+                    // the lane's four elements share a bucket (codes beyond n are 0)
+                    agg[j] = agg[j] + expand_codes(byte, tsc[q][j]);
+                } else {
+                    const long long e = base + j * 256 + lane * 4;
+                    unsigned bq = pq[j], br = pr[j];
+                    float sck = tsc[q][j], dv[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const unsigned c = (byte >> (2 * k)) & 3u;
+                        dv[k] = (e + k < n && c) ? code_val(c, sck) : 0.f;
+                        if (++br == B) {  // the next element begins a bucket: its scale is looked up here
+                            br = 0u;
+                            ++bq;
+                            if (k < 3 && e + k + 1 < n) sck = scales[bq];
+                        }
+                    }
+                    f4 d;
+                    d.x = dv[0]; d.y = dv[1]; d.z = dv[2]; d.w = dv[3];
+                    agg[j] = agg[j] + d;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) store4<FAST>(s.out, base + j * 256 + lane * 4, n, agg[j]);
+}
+
 template <class MSrc, int ALG, bool REENC, bool LOCAL>
 __global__ __launch_bounds__(kBlock) void dense_merge_kernel(MSrc src, int npeers) {
     unsigned tile;
@@ -167,8 +319,14 @@ __global__ __launch_bounds__(kBlock) void dense_merge_kernel(MSrc src, int npeer
         h[2] = 0;
         h[3] = 0;
     }
-    if (m.s.aligned && (unsigned long long)(tile + 1) * kTile <= m.s.n) merge_tile<true, ALG, REENC, LOCAL>(m, tile, npeers);
-    else merge_tile<false, ALG, REENC, LOCAL>(m, tile, npeers);
+    const bool fast = m.s.aligned && (unsigned long long)(tile + 1) * kTile <= m.s.n;
+    if constexpr (ALG == HIPRESS_TERNGRAD) {
+        if (fast) merge_tile_terngrad<true, LOCAL>(m, tile, npeers);
+        else merge_tile_terngrad<false, LOCAL>(m, tile, npeers);
+    } else {
+        if (fast) merge_tile<true, ALG, REENC, LOCAL>(m, tile, npeers);
+        else merge_tile<false, ALG, REENC, LOCAL>(m, tile, npeers);
+    }
 }
 
 template <class MSrc, bool LOCAL>

@@ -197,7 +197,11 @@ def test_onebit_zero_tensor(hp):
 
 
 # ---------------------------------------------------------------- TernGrad
-@pytest.mark.parametrize("bucket", [512, 256, 1024, 100, 16, 2048])
+# 256 / 512 / 1024: the bucket maximum is a wavefront reduction; every other size up to a tile
+# (1, 3, 16, 100, 2048, 4095, 4096) goes through the single-pass encoder whose maxima meet in
+# LDS, buckets hanging over into the neighbouring tiles included; beyond a tile (4097, 5000,
+# 70000: a bucket longer than most of these tensors) two passes.
+@pytest.mark.parametrize("bucket", [512, 256, 1024, 100, 16, 2048, 1, 3, 4095, 4096, 4097, 5000, 70000])
 @pytest.mark.parametrize("n", [1, 17, 511, 512, 513, 4097, 70001, 1000003])
 def test_terngrad_encode_decode(hp, n, bucket):
     rng = np.random.default_rng(n * 7 + bucket)
@@ -212,6 +216,36 @@ def test_terngrad_encode_decode(hp, n, bucket):
     out = torch.full((n,), 7.0, device="cuda")
     hp.terngrad_decode(pay, out)
     np.testing.assert_array_equal(host(out), oracle.terngrad_decode(want, n))
+
+
+@pytest.mark.parametrize("bucket", [100, 3000, 4096, 6000])
+def test_terngrad_any_bucket_with_special_values_and_batches(hp, bucket):
+    """The LDS maxima of the single-pass encoder on values fmaxf treats specially (NaN is
+    passed over, infinities and signed zeros are not), through a batch whose tensors begin at
+    odd tile counts, against the oracle."""
+    rng = np.random.default_rng(bucket)
+    sizes = [4096 * 3 + 17, 1, 4096, 12345, 4095, 70001]
+    tensors, want = [], []
+    for k, n in enumerate(sizes):
+        g = rng.normal(0, 1e-3, n).astype(F)
+        if n > 100:
+            idx = rng.choice(n, size=min(n // 50, 40), replace=False)
+            g[idx] = rng.choice(np.array([np.nan, np.inf, -np.inf, 0.0, -0.0, 1e-40, 3e38, -3e38], F), size=idx.size)
+            g[bucket - 1 if bucket - 1 < n else 0] = np.nan        # last element of the first bucket
+            g[min(n - 1, 4096)] = -np.inf                          # first element behind a tile border
+        u = rng.random(n, dtype=F)
+        tensors.append({"gradient": dev(g), "uniform": dev(u), "out": torch.full((n,), 7.0, device="cuda"),
+                        "compressed": payload(hp.terngrad_payload_bytes(n, bucket))})
+        want.append(oracle.terngrad_encode(g, u, bucket))
+    b = hp.Batch("terngrad", tensors, bucket=bucket)
+    b.encode()
+    b.decode()
+    for t, w, n in zip(tensors, want, sizes):
+        np.testing.assert_array_equal(host(t["compressed"]), w, err_msg=f"payload n={n}")
+        got, ref = host(t["out"]), oracle.terngrad_decode(w, n)
+        np.testing.assert_array_equal(np.isnan(got), np.isnan(ref))
+        np.testing.assert_array_equal(got[~np.isnan(ref)], ref[~np.isnan(ref)], err_msg=f"decode n={n}")
+    b.close()
 
 
 def test_terngrad_decode_rejects_header_that_overruns_buffer(hp):
@@ -381,6 +415,44 @@ def test_terngrad_decode_merge_skips_a_peer_whose_header_does_not_fit(hp):
     for bad in (zero_bucket, tiny_bucket):
         hp.terngrad_decode_merge([dev(tg[0]), dev(bad), dev(tg[2])], agg)
         np.testing.assert_array_equal(host(agg), oracle.terngrad_decode_merge([tg[0], tg[2]], n))
+
+
+@pytest.mark.parametrize("expected", [512, 100, 4096, 3])
+def test_terngrad_merge_batch_with_peers_of_other_bucket_sizes(hp, expected):
+    """A merge batch names the bucket size its peers are expected to have used and asks for
+    their words from that before it has seen their headers; a header that names another size
+    still decides.  Nine peers per chunk (two rounds of the kernel's eight): most with the
+    expected size, the others with sizes of every kind (a multiple of 256, a power of two below
+    it, neither, longer than a tile, 1), and one whose header is unusable.  Against the oracle,
+    which reads every header."""
+    rng = np.random.default_rng(expected)
+    others = [256, 64, 100, 6000, 1, expected, expected, expected, expected]
+    sizes = [4096 * 2 + 17, 100003, 5, 4096]
+    chunks, want = [], []
+    for n in sizes:
+        pays = [oracle.terngrad_encode(rng.normal(0, 1, n).astype(F), rng.random(n, dtype=F), b) for b in others]
+        broken = pays[6].copy()
+        broken[4:8] = 0  # bucket size 0: this peer adds nothing
+        pays[6] = broken
+        # every buffer as large as the largest layout, so that a wrong guess still reads inside it
+        room = max(p.size for p in pays)
+        bufs = []
+        for p in pays:
+            t = torch.zeros(room, dtype=torch.uint8, device="cuda")
+            t[: p.size] = dev(p)
+            bufs.append(t)
+        chunks.append({"compressed": bufs, "aggregate": torch.full((n,), 7.0, device="cuda")})
+        want.append(oracle.terngrad_decode_merge([p for k, p in enumerate(pays) if k != 6], n))
+    mb = hp.MergeBatch("terngrad", chunks, bucket=expected)
+    mb.run()
+    for c, w, n in zip(chunks, want, sizes):
+        np.testing.assert_array_equal(host(c["aggregate"]), w, err_msg=f"n={n}")
+    # and peer by peer through the per-tensor call, which has no expectation to start from
+    for c, w, n in zip(chunks, want, sizes):
+        agg = torch.full((n,), 7.0, device="cuda")
+        hp.terngrad_decode_merge(c["compressed"], agg)
+        np.testing.assert_array_equal(host(agg), w, err_msg=f"per-tensor n={n}")
+    mb.close()
 
 
 @pytest.mark.parametrize("n", [1000, 1048576])
