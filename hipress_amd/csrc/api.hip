@@ -554,7 +554,7 @@ int hipress_terngrad_decode(const void* payload, int64_t payload_bytes, float* o
     int rc = build_decode_seg(HIPRESS_TERNGRAD, payload, payload_bytes, out, n, &s);
     if (rc) return rc;
     if (payload_bytes < HIPRESS_HEADER_BYTES + words_bytes(n, 2)) return HIPRESS_ERR_SIZE;
-    return hiperr(launch_terngrad_decode(single_launch(s), static_cast<hipStream_t>(stream)));
+    return hiperr(launch_terngrad_decode(single_launch(s), 0u, static_cast<hipStream_t>(stream)));
 }
 
 // ---- the in-tree CompLL operator -------------------------------------------------------
@@ -986,7 +986,7 @@ int hipress_batch_decode(hipress_batch* b, void* stream) {
         case HIPRESS_ONEBIT:
         case HIPRESS_ONEBIT_DEFERRED: return hiperr(launch_onebit_decode(L, st));
         case HIPRESS_TBQ: return hiperr(launch_tbq_decode(L, st));
-        case HIPRESS_TERNGRAD: return hiperr(launch_terngrad_decode(L, st));
+        case HIPRESS_TERNGRAD: return hiperr(launch_terngrad_decode(L, (unsigned)b->params.bucket, st));
         case HIPRESS_DGC:
         case HIPRESS_GRADDROP:
             if (++b->epoch == 0) b->epoch = 1;  // the flags start at 0, which no call uses

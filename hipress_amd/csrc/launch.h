@@ -11,7 +11,7 @@ hipError_t launch_onebit_decode(const Launch& L, hipStream_t st);
 hipError_t launch_onebit_encode_deferred(const Launch& L, float* partial, int phase, hipStream_t st);
 hipError_t launch_onebit_materialize(const Launch& L, hipStream_t st);
 hipError_t launch_terngrad_encode(const Launch& L, unsigned bucket, hipStream_t st);
-hipError_t launch_terngrad_decode(const Launch& L, hipStream_t st);
+hipError_t launch_terngrad_decode(const Launch& L, unsigned bucket, hipStream_t st);  // bucket: what the launch's descriptors name, 0 = unknown
 
 // The in-tree CompLL operator (10-byte header, b-bit min/max quantiser).
 hipError_t launch_compll_encode(const Launch& L, int bitwidth, float* partial, hipStream_t st);
