@@ -530,6 +530,7 @@ int hipress_onebit_residual(const float* state, const float* scale_state, int64_
     s.out = residual;
     s.n = (unsigned long long)n;
     s.ntiles = tiles_of(n);
+    s.aligned = vec_ok(state) && vec_ok(residual);
     return hiperr(launch_onebit_materialize(single_launch(s), static_cast<hipStream_t>(stream)));
 }
 

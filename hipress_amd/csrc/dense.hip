@@ -339,25 +339,32 @@ __global__ __launch_bounds__(kBlock) void onebit_deferred_kernel(Src src, float*
 }
 
 // out = v - d(v, scale): the residual the two-pass operator holds after the same steps.
-template <class Src>
-__global__ __launch_bounds__(kBlock) void onebit_materialize_kernel(Src src) {
-    unsigned tile;
-    const Seg s = src.get(tile, blockIdx.x);
+template <bool FAST>
+__device__ __forceinline__ void onebit_materialize_tile(const Seg& s, unsigned tile) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long n = (long long)s.n;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
     const float sp = *s.s1;
+    f4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = load4<FAST>(s.s0, base + j * 256 + lane * 4, n);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        long long e = base + j * 256 + lane * 4;
-        f4 v = ld4_guard(s.s0, e, n);
         f4 r;
-        r.x = v.x - (v.x >= 0.f ? sp : -sp);
-        r.y = v.y - (v.y >= 0.f ? sp : -sp);
-        r.z = v.z - (v.z >= 0.f ? sp : -sp);
-        r.w = v.w - (v.w >= 0.f ? sp : -sp);
-        st4_guard(s.out, e, n, r);
+        r.x = v[j].x - (v[j].x >= 0.f ? sp : -sp);
+        r.y = v[j].y - (v[j].y >= 0.f ? sp : -sp);
+        r.z = v[j].z - (v[j].z >= 0.f ? sp : -sp);
+        r.w = v[j].w - (v[j].w >= 0.f ? sp : -sp);
+        store4<FAST>(s.out, base + j * 256 + lane * 4, n, r);
     }
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void onebit_materialize_kernel(Src src) {
+    unsigned tile;
+    const Seg s = src.get(tile, blockIdx.x);
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) onebit_materialize_tile<true>(s, tile);
+    else onebit_materialize_tile<false>(s, tile);
 }
 
 template <bool FAST>
