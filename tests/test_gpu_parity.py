@@ -417,8 +417,9 @@ def test_terngrad_decode_merge_skips_a_peer_whose_header_does_not_fit(hp):
         np.testing.assert_array_equal(host(agg), oracle.terngrad_decode_merge([tg[0], tg[2]], n))
 
 
+@pytest.mark.parametrize("roomy", [True, False])
 @pytest.mark.parametrize("expected", [512, 100, 4096, 3])
-def test_terngrad_merge_batch_with_peers_of_other_bucket_sizes(hp, expected):
+def test_terngrad_merge_batch_with_peers_of_other_bucket_sizes(hp, expected, roomy):
     """A merge batch names the bucket size its peers are expected to have used and asks for
     their words from that before it has seen their headers; a header that names another size
     still decides.  Nine peers per chunk (two rounds of the kernel's eight): most with the
@@ -434,11 +435,14 @@ def test_terngrad_merge_batch_with_peers_of_other_bucket_sizes(hp, expected):
         broken = pays[6].copy()
         broken[4:8] = 0  # bucket size 0: this peer adds nothing
         pays[6] = broken
-        # every buffer as large as the largest layout, so that a wrong guess still reads inside it
+        # roomy: every buffer as large as the largest layout, so that the expected layout fits all
+        # of them and is read before the header corrects it; otherwise every buffer exactly as large
+        # as its own layout, so that for some peers the expected layout does not fit and nothing
+        # may be read from it
         room = max(p.size for p in pays)
         bufs = []
         for p in pays:
-            t = torch.zeros(room, dtype=torch.uint8, device="cuda")
+            t = torch.zeros(room if roomy else p.size, dtype=torch.uint8, device="cuda")
             t[: p.size] = dev(p)
             bufs.append(t)
         chunks.append({"compressed": bufs, "aggregate": torch.full((n,), 7.0, device="cuda")})
