@@ -555,7 +555,9 @@ def make_workload(name):
     if name == "graddrop_vgg19":
         return SetWorkload(name, "graddrop", vgg, "vgg", {"ratio": 0.01}, 12.0, 4.0, 0, "sparse_accum_kernel", 12.0, nphases=7)
     if name == "tbq_262144":
-        return SetWorkload(name, "tbq", [262144], "n0.02", {"threshold": 0.05}, 12.25, 4.25, 0, "tbq_encode_kernel", 12.25)
+        # 128 buffer sets in turn (400 MB in all): one 3 MB set alone would be served from the caches
+        return SetWorkload(name, "tbq", [262144], "n0.02", {"threshold": 0.05}, 12.25, 4.25, 0, "tbq_encode_kernel", 12.25,
+                           rotate=128)
     if name == "tbq_262144_x512":
         return SetWorkload(name, "tbq", [262144] * 512, "n0.02", {"threshold": 0.05}, 12.25, 4.25, 0, "tbq_encode_kernel", 12.25)
     if name == "terngrad_resnet50":
