@@ -1,7 +1,10 @@
 """Seeded random configurations of every operator against the oracle: sizes that fall
 anywhere relative to word, bucket, group, tile and sample boundaries, parameters over their
 whole range, state carried over two steps.  The cases are fixed by the seed, so a failure
-names its case and repeats."""
+names its case and repeats.  HIPRESS_TEST_SEED=k in the environment shifts every seed by
+7919*k for a sweep over other cases (the suite itself runs k = 0)."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -10,6 +13,11 @@ import oracle
 
 pytestmark = pytest.mark.gpu
 F = np.float32
+SHIFT = 7919 * int(os.environ.get("HIPRESS_TEST_SEED", "0"))
+
+
+def seeded(seed):
+    return np.random.default_rng(seed + SHIFT)
 
 
 @pytest.fixture(scope="module")
@@ -53,7 +61,7 @@ def check_sparse(got_pay, want_pay, where):
 
 
 def test_dense_quantisers_random_cases(hp):
-    rng = np.random.default_rng(2024)
+    rng = seeded(2024)
     for case, n in enumerate(sizes(rng, 150)):
         sigma = 10 ** rng.uniform(-4, 0)
         tau = float(F(sigma * rng.uniform(0.2, 4.0)))
@@ -90,7 +98,7 @@ def test_dense_quantisers_random_cases(hp):
 
 
 def test_sparsifiers_random_cases(hp):
-    rng = np.random.default_rng(2025)
+    rng = seeded(2025)
     for case, n in enumerate(sizes(rng, 150, top=1_500_000)):
         ratio = float(10 ** rng.uniform(-3.3, -0.5))
         m = float(F(rng.uniform(0.0, 0.99)))
@@ -119,7 +127,7 @@ def test_sparsifiers_random_cases(hp):
 
 
 def test_merges_random_cases(hp):
-    rng = np.random.default_rng(2026)
+    rng = seeded(2026)
     for case, n in enumerate(sizes(rng, 80, top=1_200_000)):
         P = int(rng.integers(1, 17))
         tau = float(F(rng.uniform(0.01, 0.1)))
@@ -145,7 +153,7 @@ def test_merges_random_cases(hp):
 
 
 def test_batches_of_random_tensor_tables(hp):
-    rng = np.random.default_rng(2027)
+    rng = seeded(2027)
     for alg in ("tbq", "terngrad", "dgc", "graddrop"):
         for table in range(8):
             ns = sizes(rng, int(rng.integers(2, 25)), top=600_000)
@@ -191,3 +199,88 @@ def test_batches_of_random_tensor_tables(hp):
                     ref = oracle.sparse_decode(want, n)
                 np.testing.assert_array_equal(host(t["out"]), ref, err_msg="decode " + where)
             b.close()
+
+
+def test_views_buckets_and_dense_merges_random_cases(hp):
+    """What the cases above hold fixed: fp32 tensors that start 0-3 elements into their
+    allocation (4-byte aligned only), TernGrad bucket sizes of any value, dense merges of
+    1-16 peers with and without a local gradient (TernGrad peers partly with bucket sizes of
+    their own), and the min/max quantiser at every bit width."""
+    rng = seeded(2028)
+    for case, n in enumerate(sizes(rng, 60, top=700_000)):
+        bucket = int(rng.choice([int(rng.integers(1, 6000)), 256, 512, 768, 1024, 4096, 8192,
+                                 int(rng.integers(6000, 200000))]))
+        P = int(rng.integers(1, 17))
+        off = int(rng.integers(0, 4))
+        where = f"case {case}: n={n} bucket={bucket} peers={P} offset={off}"
+
+        def view(a):
+            t = torch.empty(n + off, device="cuda")
+            v = t[off:]
+            v.copy_(torch.from_numpy(np.ascontiguousarray(a, dtype=F)))
+            return v
+
+        g, u = rng.normal(0, 1e-3, n).astype(F), rng.random(n, dtype=F)
+        pay = payload(hp.terngrad_payload_bytes(n, bucket))
+        hp.terngrad_encode(view(g), view(u), pay, bucket)
+        want = oracle.terngrad_encode(g, u, bucket)
+        np.testing.assert_array_equal(host(pay), want, err_msg="terngrad " + where)
+        out = view(np.full(n, 7, F))
+        hp.terngrad_decode(pay, out)
+        np.testing.assert_array_equal(host(out), oracle.terngrad_decode(want, n), err_msg="terngrad decode " + where)
+
+        pays = []
+        for _ in range(P):
+            b = bucket if rng.random() < 0.8 else int(rng.integers(1, 3000))
+            pays.append(oracle.terngrad_encode(rng.normal(0, 1e-3, n).astype(F), rng.random(n, dtype=F), b))
+        local = rng.normal(0, 1e-3, n).astype(F) if rng.random() < 0.5 else None
+        loc = (lambda: None if local is None else view(local))
+        agg = view(np.full(n, 7, F))
+        hp.terngrad_decode_merge([dev(p) for p in pays], agg, local=loc())
+        np.testing.assert_array_equal(host(agg), oracle.terngrad_decode_merge(pays, n, local=local),
+                                      err_msg="terngrad merge " + where)
+        z = np.zeros(n, F)
+        pays = [oracle.onebit_encode(rng.normal(0, 10 ** rng.uniform(-4, 0), n).astype(F), z)[0] for _ in range(P)]
+        agg = view(np.full(n, 7, F))
+        hp.onebit_decode_merge([dev(p) for p in pays], agg, local=loc())
+        np.testing.assert_array_equal(host(agg), oracle.onebit_decode_merge(pays, n, local=local),
+                                      err_msg="onebit merge " + where)
+        tau = float(F(rng.uniform(0.01, 0.1)))
+        pays = [oracle.tbq_encode(rng.normal(0, 0.04, n).astype(F), z, tau)[0] for _ in range(P)]
+        agg = view(np.full(n, 7, F))
+        hp.tbq_decode_merge([dev(p) for p in pays], agg, local=loc())
+        np.testing.assert_array_equal(host(agg), oracle.tbq_decode_merge(pays, n, None, 0.0, local=local),
+                                      err_msg="tbq merge " + where)
+
+        b = int(rng.choice([1, 2, 4, 8]))
+        pay = payload(hp.compll_payload_bytes(n, b))
+        hp.compll_terngrad_encode(view(g), view(u), pay, b)
+        want = oracle.compll_encode(g, u, b)
+        np.testing.assert_array_equal(host(pay), want, err_msg=f"min/max quantiser b={b} " + where)
+        count = hp.compll_decoded_count(n, b)
+        out = torch.full((count + off + 1,), 7.0, device="cuda")[off:off + count]
+        hp.compll_terngrad_decode(pay, out)
+        ref = oracle.compll_decode(want, count)
+        assert len(ref) == count, (len(ref), count, where)
+        np.testing.assert_array_equal(host(out), ref, err_msg=f"min/max decode b={b} " + where)
+
+        ratio = float(10 ** rng.uniform(-3, -1))
+        m = float(F(rng.uniform(0.0, 0.99)))
+        mom0, acc0 = rng.normal(0, 1e-3, n).astype(F), rng.normal(0, 1e-3, n).astype(F)
+        mom, acc = view(mom0), view(acc0)
+        pay = payload(hp.sparse_payload_bytes(n, ratio))
+        hp.dgc_encode(view(g), mom, acc, pay, m, ratio)
+        want, mom_ref, acc_ref = oracle.dgc_encode(g, mom0, acc0, m, ratio)
+        check_sparse(host(pay), want, "dgc " + where)
+        np.testing.assert_array_equal(host(mom), mom_ref, err_msg="dgc momentum " + where)
+        np.testing.assert_array_equal(host(acc), acc_ref, err_msg="dgc accumulator " + where)
+        out = view(np.full(n, 7, F))
+        hp.dgc_decode(pay, out)
+        np.testing.assert_array_equal(host(out), oracle.sparse_decode(want, n), err_msg="sparse decode " + where)
+        sp = [oracle.graddrop_encode(rng.normal(0, 1e-3, n).astype(F), z, ratio)[0] for _ in range(P)]
+        agg, acc, outp = view(np.full(n, 7, F)), view(acc0), payload(hp.sparse_payload_bytes(n, ratio))
+        hp.dgc_decode_merge([dev(p) for p in sp], agg, acc, outp, ratio, local=loc())
+        want_agg, want_out, want_acc = oracle.sparse_decode_merge(sp, n, acc0, ratio, local=local)
+        np.testing.assert_array_equal(host(agg), want_agg, err_msg="sparse merge " + where)
+        check_sparse(host(outp), want_out, "sparse merge payload " + where)
+        np.testing.assert_array_equal(host(acc), want_acc, err_msg="sparse merge accumulator " + where)
