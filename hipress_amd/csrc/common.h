@@ -205,14 +205,15 @@ __device__ __forceinline__ unsigned xcd_grouped(unsigned b, unsigned nblocks) {
 // (cache_tail) and the second pass walks the launch backwards (xcd_reversed), in groups of
 // eight so that consecutive workgroups still go to the eight XCDs in turn.  Both halves are
 // needed: on the same GPU, alternating libraries, the quantise pass of onebit over the VGG19
-// set takes 259 us with both, 263 us with only the reversed order and 263 us with neither;
-// the code pass of the min/max quantiser over 102.8 M elements 133 / 136 / 136 us.
+// set takes 256.8 us with both, 262.6 us with only the reversed order and 259.7 us with
+// neither; the code pass of the min/max quantiser over 102.8 M elements 133.0 us with a
+// 32 MiB tail and the reversed order, 136.2 us with the order alone, 134.8 us with neither.
 // How much to leave behind depends on what the second pass does besides re-reading.  After
 // one read stream (the min/max quantiser) the gain grows up to the cache's size: tails of
-// 32 / 64 / 128 / 192 / 256 / 384 MiB take min/max + code pass from 190.4 to 189.3 / 187.9 /
-// 185.9 / 185.3 / 186.7 us (the plain loads cost the first pass 1 us per 64 MiB, the second
-// pass gains 2.5).  After two read streams whose second pass also writes one of them back
-// (onebit) nothing is gained beyond 32 MiB: what the second pass saves, the first one loses.
+// 0 / 32 / 64 / 128 / 192 / 256 / 384 MiB take min/max + code pass 192.7 / 190.3 / 189.3 /
+// 187.9 / 186.3 / 185.3 / 186.7 us (the plain loads cost the first pass 1 us per 64 MiB, the
+// second pass gains 2.5).  After two read streams whose second pass also writes one of them
+// back (onebit) nothing is gained beyond 32 MiB: what the second pass saves, the first loses.
 //
 // Tuning constants, overridable at build time for A/B measurements
 // (python -m hipress_amd.build --define HP_CACHE_TAIL_ONE_MIB=0 ...): MiB read with plain loads
