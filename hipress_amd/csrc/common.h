@@ -328,6 +328,22 @@ __device__ __forceinline__ unsigned wave_incl_scan_u(unsigned x) {
     return x;
 }
 // Sum over the 64 lanes, the same value (wavefront-uniform) in every lane.
+// The same for unsigned keys.
+__device__ __forceinline__ unsigned wave_umax(unsigned x) {
+#define HP_UMAX_STEP(CTRL, ROWS)                                                                       \
+    {                                                                                                 \
+        const unsigned y = (unsigned)__builtin_amdgcn_update_dpp((int)x, (int)x, CTRL, ROWS, 0xf, false); \
+        x = y > x ? y : x;                                                                            \
+    }
+    HP_UMAX_STEP(0xB1, 0xf)   // quad_perm [1,0,3,2]
+    HP_UMAX_STEP(0x4E, 0xf)   // quad_perm [2,3,0,1]
+    HP_UMAX_STEP(0x141, 0xf)  // row_half_mirror
+    HP_UMAX_STEP(0x140, 0xf)  // row_mirror
+    HP_UMAX_STEP(0x142, 0xa)  // row_bcast:15 into rows 1, 3
+    HP_UMAX_STEP(0x143, 0xc)  // row_bcast:31 into rows 2, 3
+#undef HP_UMAX_STEP
+    return (unsigned)__builtin_amdgcn_readlane((int)x, 63);
+}
 __device__ __forceinline__ unsigned wave_sum_u(unsigned x) {
     return (unsigned)__builtin_amdgcn_readlane((int)wave_incl_scan_u(x), 63);
 }

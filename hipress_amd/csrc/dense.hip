@@ -494,8 +494,10 @@ __global__ __launch_bounds__(kBlock) void terngrad_encode_kernel(Src src) {
 // maximum of every bucket its own elements need.  Maxima meet in LDS as integer keys (the
 // bit pattern of |g| orders like |g|; values that are no number leave no key, as fmaxf
 // passes them over).  A bucket's scale is written by the tile it begins in.
-constexpr unsigned kAnyBucketMax = kTile;
+constexpr unsigned kAnyBucketMax = kTile;  // beyond a tile: the three-launch path, whose tiles lie in at most two buckets
 constexpr unsigned kAnyBuckets = kTile + 2;  // bucket size 1: every element its own, plus none hanging over
+
+__device__ __forceinline__ unsigned umax32(unsigned a, unsigned b) { return a > b ? a : b; }
 
 __device__ __forceinline__ unsigned absmax_key(float x) {
     const unsigned k = __float_as_uint(x) & 0x7fffffffu;
@@ -527,8 +529,19 @@ __device__ __forceinline__ void terngrad_encode_any_tile(const Seg& s, unsigned 
     }
     __syncthreads();
     // what hangs over from the neighbours: fewer than B elements on either side
-    for (long long i = start + threadIdx.x; i < t0; i += kBlock) atomicMax(&mx[0], absmax_key(s.g[i]));
-    for (long long i = t1 + threadIdx.x; i < end; i += kBlock) atomicMax(&mx[nb - 1], absmax_key(s.g[i]));
+    // (every wavefront folds its share before it touches the shared word)
+    if (start < t0) {
+        unsigned k = 0u;
+        for (long long i = start + threadIdx.x; i < t0; i += kBlock) k = umax32(k, absmax_key(s.g[i]));
+        k = wave_umax(k);
+        if (lane == 0) atomicMax(&mx[0], k);
+    }
+    if (t1 < end) {
+        unsigned k = 0u;
+        for (long long i = t1 + threadIdx.x; i < end; i += kBlock) k = umax32(k, absmax_key(s.g[i]));
+        k = wave_umax(k);
+        if (lane == 0) atomicMax(&mx[nb - 1], k);
+    }
     // local bucket and place inside it of each step's first element: one 32-bit division per step
     unsigned lb[4], rem[4];
 #pragma unroll
@@ -538,15 +551,31 @@ __device__ __forceinline__ void terngrad_encode_any_tile(const Seg& s, unsigned 
         rem[j] = x - lb[j] * B;
         const float v[4] = {g[j].x, g[j].y, g[j].z, g[j].w};
         const long long e = base + j * 256 + lane * 4;
-        if (rem[j] + 3u < B) {  // the four elements share a bucket
-            if (e < n) atomicMax(&mx[lb[j]], absmax_key(absmax4(g[j])));  // elements beyond n were loaded as zero
-        } else {
+        const bool shared = rem[j] + 3u < B;  // the four elements share a bucket
+        if (!shared) {
             unsigned b = lb[j], r = rem[j];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 if (e + k < n) atomicMax(&mx[b], absmax_key(v[k]));
                 if (++r == B) { r = 0; ++b; }
             }
+        }
+        const bool mine = shared && e < n;  // elements beyond n were loaded as zero
+        const unsigned key = mine ? absmax_key(absmax4(g[j])) : 0u;
+        if (B >= 128u) {
+            // the step's 256 elements lie in at most three buckets, lane 0's and the two after it: one
+            // fold over the wavefront and one shared-memory maximum each, instead of one per lane
+            const unsigned first = (unsigned)__builtin_amdgcn_readfirstlane((int)lb[j]);
+#pragma unroll
+            for (unsigned d = 0; d < 3u; ++d) {
+                const bool here = mine && lb[j] == first + d;
+                if (__ballot(here)) {  // wavefront-uniform
+                    const unsigned m = wave_umax(here ? key : 0u);
+                    if (lane == 0) atomicMax(&mx[first + d], m);
+                }
+            }
+        } else if (mine) {
+            atomicMax(&mx[lb[j]], key);
         }
     }
     __syncthreads();
@@ -596,16 +625,88 @@ __global__ __launch_bounds__(kBlock) void terngrad_encode_any_kernel(Src src) {
     else terngrad_encode_any_tile<false>(s, tile, mx);
 }
 
-// Bucket sizes beyond a tile: one wavefront per bucket writes the scale ...
+// Bucket sizes beyond a tile, up to the whole tensor: a tile then lies in at most two buckets, and a
+// bucket's maximum is gathered over many tiles.  Three launches, no device-wide read-modify-write
+// (which, a hundred thousand of them on the few cache lines of a short scale array, took a
+// millisecond).  1: every tile folds the magnitudes of its two parts, as bit patterns (which order
+// like the magnitudes; a maximum does not depend on the order it is taken in), into two words that
+// it parks at the start of the payload's word area, words 2t and 2t + 1 for tile t: that area holds
+// 256 words per tile and is written only by launch 3.  (A tensor of a single tile lies in one
+// bucket and parks one word.)  2: the workgroup of the tile in which a bucket begins folds the
+// parked words of the tiles the bucket covers and writes its scale; the first tile also writes the
+// header.  3: a second pass over the gradient quantises with the finished scales.
+struct BigBucketTile {
+    unsigned b0;              // bucket of the tile's first element
+    unsigned long long bnd;   // elements of the tile in front of the next bucket (kTile or more: none follows)
+};
+__device__ __forceinline__ BigBucketTile big_bucket_tile(unsigned tile, unsigned B) {
+    BigBucketTile t;
+    const unsigned t0 = tile * (unsigned)kTile;  // the element count fits 32 bits
+    t.b0 = t0 / B;
+    t.bnd = ((unsigned long long)t.b0 + 1ull) * B - t0;
+    return t;
+}
+
+// maximum over the workgroup of what lane 0 of each wavefront holds; red: one word per wavefront
+__device__ __forceinline__ unsigned block_umax(unsigned wave_value, unsigned* red) {
+    if ((threadIdx.x & 63u) == 0u) red[threadIdx.x >> 6] = wave_value;
+    __syncthreads();
+    unsigned m = red[0];
+#pragma unroll
+    for (int w = 1; w < kBlock / 64; ++w) m = umax32(m, red[w]);
+    __syncthreads();
+    return m;
+}
+
+template <bool FAST>
+__device__ __forceinline__ void terngrad_partial_big_tile(const Seg& s, unsigned tile, unsigned* red) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    const BigBucketTile t = big_bucket_tile(tile, s.bucket);
+    f4 g[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) g[j] = load4<FAST>(s.g, base + j * 256 + lane * 4, n);  // beyond n: zero, which adds nothing
+    unsigned ka = 0u, kb = 0u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const unsigned li = wave * kWaveTile + j * 256 + lane * 4;
+        const float v[4] = {g[j].x, g[j].y, g[j].z, g[j].w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const unsigned key = absmax_key(v[k]);
+            if (li + k < t.bnd) ka = umax32(ka, key);
+            else kb = umax32(kb, key);
+        }
+    }
+    ka = block_umax(wave_umax(ka), red);
+    kb = block_umax(wave_umax(kb), red);
+    if (threadIdx.x == 0) {
+        uint32_t* parked = reinterpret_cast<uint32_t*>(s.pay + s.words_off);
+        if (s.n > (unsigned long long)kTile) {
+            parked[2ull * tile] = ka;
+            parked[2ull * tile + 1ull] = kb;
+        } else {
+            parked[0] = ka;
+        }
+    }
+}
+
 template <class Src>
-__global__ __launch_bounds__(kBlock) void terngrad_scale_generic_kernel(Src src) {
-    // grid: tiles of the tensor; each workgroup walks the buckets that START in its tile
+__global__ __launch_bounds__(kBlock) void terngrad_partial_big_kernel(Src src) {
+    __shared__ unsigned red[kBlock / 64];
     unsigned tile;
     const Seg s = src.get(tile, blockIdx.x);
-    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const long long n = (long long)s.n, B = s.bucket;
-    const long long lo = (long long)tile * kTile, hi = lo + kTile < n ? lo + kTile : n;
-    float* scales = reinterpret_cast<float*>(s.pay + kHeaderBytes);
+    if ((unsigned long long)tile * kTile >= s.n) return;  // an empty tensor has one tile and nothing in it
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) terngrad_partial_big_tile<true>(s, tile, red);
+    else terngrad_partial_big_tile<false>(s, tile, red);
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void terngrad_scale_big_kernel(Src src) {
+    __shared__ unsigned red[kBlock / 64];
+    unsigned tile;
+    const Seg s = src.get(tile, blockIdx.x);
     if (tile == 0 && threadIdx.x == 0) {
         uint32_t* h = reinterpret_cast<uint32_t*>(s.pay);
         h[0] = (uint32_t)s.n;
@@ -614,41 +715,73 @@ __global__ __launch_bounds__(kBlock) void terngrad_scale_generic_kernel(Src src)
         h[3] = 0;
     }
     terngrad_zero_scale_pad(s, tile);
-    long long first = (lo + B - 1) / B;  // first bucket starting at or after lo
-    for (long long b = first + wave; b * B < hi; b += 4) {
-        long long e0 = b * B, e1 = e0 + B < n ? e0 + B : n;
-        float m = 0.f;
-        for (long long e = e0 + lane; e < e1; e += 64) m = fmaxf(m, fabsf(s.g[e]));
-        m = wave_max(m);
-        if (lane == 0) scales[b] = m;
+    const unsigned long long B = s.bucket, lo = (unsigned long long)tile * kTile;
+    const unsigned long long hi = lo + kTile < s.n ? lo + kTile : s.n;
+    const unsigned long long first = (lo + B - 1) / B;  // the bucket that begins at or after lo
+    const unsigned long long e0 = first * B;
+    if (e0 >= hi) return;  // no bucket begins in this tile
+    const unsigned long long e1 = e0 + B < s.n ? e0 + B : s.n;
+    const unsigned long long last_tile = (e1 - 1) / kTile;
+    const uint32_t* parked = reinterpret_cast<const uint32_t*>(s.pay + s.words_off);
+    unsigned k = 0u;
+    if (s.n > (unsigned long long)kTile) {
+        // this tile holds the bucket's beginning: in its second part unless the bucket begins with the
+        // tile; every further tile the bucket reaches holds it in its first part
+        for (unsigned long long t = tile + threadIdx.x; t <= last_tile; t += kBlock)
+            k = umax32(k, parked[2ull * t + ((t == tile && e0 != lo) ? 1ull : 0ull)]);
+    } else if (threadIdx.x == 0) {
+        k = parked[0];
     }
+    k = block_umax(wave_umax(k), red);
+    if (threadIdx.x == 0) reinterpret_cast<float*>(s.pay + kHeaderBytes)[first] = __uint_as_float(k);
 }
 
-// ... and a second pass quantises with a per-element scale lookup.
-template <class Src>
-__global__ __launch_bounds__(kBlock) void terngrad_quant_generic_kernel(Src src) {
-    unsigned tile;
-    const Seg s = src.get(tile, blockIdx.x);
+template <bool FAST>
+__device__ __forceinline__ void terngrad_quant_big_tile(const Seg& s, unsigned tile) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const long long n = (long long)s.n, B = s.bucket;
+    const long long n = (long long)s.n;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
+    if (base >= n) return;
+    const BigBucketTile t = big_bucket_tile(tile, s.bucket);
     const float* scales = reinterpret_cast<const float*>(s.pay + kHeaderBytes);
     uint32_t* words = reinterpret_cast<uint32_t*>(s.pay + s.words_off);
+    f4 g[4], u[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const long long e = base + j * 256 + lane * 4;
+        g[j] = load4<FAST>(s.g, e, n);
+        u[j] = load4<FAST>(s.u, e, n);
+    }
+    const float sa = scales[t.b0];
+    const float sb = (unsigned long long)tile * kTile + t.bnd < (unsigned long long)n && t.bnd < (unsigned long long)kTile ? scales[t.b0 + 1u] : 0.f;
     unsigned myword = 0;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        long long e = base + j * 256 + lane * 4;
-        unsigned byte = 0;
+        const unsigned li = wave * kWaveTile + j * 256 + lane * 4;
+        unsigned byte;
+        if (li + 3u < t.bnd) {
+            byte = tern_code4(g[j], u[j], sa);  // pad elements are 0: u*s < 0 is false
+        } else if (li >= t.bnd) {
+            byte = tern_code4(g[j], u[j], sb);
+        } else {
+            const float gv[4] = {g[j].x, g[j].y, g[j].z, g[j].w}, uv[4] = {u[j].x, u[j].y, u[j].z, u[j].w};
+            byte = 0;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            long long i = e + k;
-            if (i < n) byte |= tern_code(s.g[i], s.u[i], scales[i / B]) << (2 * k);
+            for (int k = 0; k < 4; ++k) byte |= tern_code(gv[k], uv[k], li + k < t.bnd ? sa : sb) << (2 * k);
         }
-        unsigned w = quad_pack8(byte);
+        const unsigned w = quad_pack8(byte);
         myword = ((lane & 3u) == (unsigned)j) ? w : myword;
     }
-    long long widx = (base >> 4) + (lane & 3u) * 16 + (lane >> 2);
-    if (widx < (long long)((n + 15) >> 4)) words[widx] = myword;
+    const long long widx = (base >> 4) + (lane & 3u) * 16 + (lane >> 2);
+    if (FAST || widx < (long long)((n + 15) >> 4)) words[widx] = myword;
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void terngrad_quant_big_kernel(Src src) {
+    unsigned tile;
+    const Seg s = src.get(tile, blockIdx.x);
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) terngrad_quant_big_tile<true>(s, tile);
+    else terngrad_quant_big_tile<false>(s, tile);
 }
 
 // Decode.  The bucket size is in the payload header, and with it the place of the
@@ -864,8 +997,9 @@ static hipError_t terngrad_encode_src(const Src& src, unsigned ntiles, unsigned 
     else if (bucket == 1024) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 1>), dim3(ntiles), dim3(kBlock), kLdsFor5, st, src);
     else if (bucket <= kAnyBucketMax) hipLaunchKernelGGL((terngrad_encode_any_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);
     else {
-        hipLaunchKernelGGL((terngrad_scale_generic_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);
-        hipLaunchKernelGGL((terngrad_quant_generic_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);
+        hipLaunchKernelGGL((terngrad_partial_big_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);
+        hipLaunchKernelGGL((terngrad_scale_big_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);
+        hipLaunchKernelGGL((terngrad_quant_big_kernel<Src>), dim3(ntiles), dim3(kBlock), kLdsFor5, st, src);
     }
     return hipGetLastError();
 }

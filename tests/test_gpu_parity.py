@@ -200,8 +200,9 @@ def test_onebit_zero_tensor(hp):
 # 256 / 512 / 1024: the bucket maximum is a wavefront reduction; every other size up to a tile
 # (1, 3, 16, 100, 2048, 4095, 4096) goes through the single-pass encoder whose maxima meet in
 # LDS, buckets hanging over into the neighbouring tiles included; beyond a tile (4097, 5000,
-# 70000: a bucket longer than most of these tensors) two passes.
-@pytest.mark.parametrize("bucket", [512, 256, 1024, 100, 16, 2048, 1, 3, 4095, 4096, 4097, 5000, 70000])
+# 8192: buckets that begin with a tile, 70000: a bucket longer than most of these tensors,
+# 2000000: one bucket for all of them) per-tile maxima are folded per bucket by a launch of its own.
+@pytest.mark.parametrize("bucket", [512, 256, 1024, 100, 16, 2048, 1, 3, 4095, 4096, 4097, 5000, 8192, 70000, 2000000])
 @pytest.mark.parametrize("n", [1, 17, 511, 512, 513, 4097, 70001, 1000003])
 def test_terngrad_encode_decode(hp, n, bucket):
     rng = np.random.default_rng(n * 7 + bucket)
@@ -218,7 +219,7 @@ def test_terngrad_encode_decode(hp, n, bucket):
     np.testing.assert_array_equal(host(out), oracle.terngrad_decode(want, n))
 
 
-@pytest.mark.parametrize("bucket", [100, 3000, 4096, 6000])
+@pytest.mark.parametrize("bucket", [100, 3000, 4096, 6000, 8192, 50000])
 def test_terngrad_any_bucket_with_special_values_and_batches(hp, bucket):
     """The LDS maxima of the single-pass encoder on values fmaxf treats specially (NaN is
     passed over, infinities and signed zeros are not), through a batch whose tensors begin at
@@ -246,6 +247,30 @@ def test_terngrad_any_bucket_with_special_values_and_batches(hp, bucket):
         np.testing.assert_array_equal(np.isnan(got), np.isnan(ref))
         np.testing.assert_array_equal(got[~np.isnan(ref)], ref[~np.isnan(ref)], err_msg=f"decode n={n}")
     b.close()
+
+
+@pytest.mark.parametrize("bucket", [1_000_000, 4096 * 1000, 20_000_003, 2**31 - 1])
+def test_terngrad_buckets_over_thousands_of_tiles(hp, bucket):
+    """Buckets that cover hundreds to thousands of tiles, up to one bucket for the whole tensor
+    (the per-layer scale of the original TernGrad), on a tensor that starts 4 bytes into its
+    allocation; the largest magnitudes sit where a fold over tiles could lose them: in the
+    first and the last element and either side of a bucket border."""
+    n = 20_000_003
+    rng = np.random.default_rng(bucket % 1000)
+    g = rng.normal(0, 1e-3, n).astype(F)
+    g[0], g[n - 1] = 0.5, -0.75
+    if bucket < n:
+        g[bucket - 1], g[bucket] = 0.25, -0.375
+    u = rng.random(n, dtype=F)
+    gd = torch.empty(n + 1, device="cuda")[1:]
+    gd.copy_(torch.from_numpy(g))
+    pay = payload(hp.terngrad_payload_bytes(n, bucket))
+    hp.terngrad_encode(gd, dev(u), pay, bucket)
+    want = oracle.terngrad_encode(g, u, bucket)
+    np.testing.assert_array_equal(host(pay), want)
+    out = torch.full((n,), 7.0, device="cuda")
+    hp.terngrad_decode(pay, out)
+    np.testing.assert_array_equal(host(out), oracle.terngrad_decode(want, n))
 
 
 def test_terngrad_decode_rejects_header_that_overruns_buffer(hp):
