@@ -542,22 +542,39 @@ __global__ __launch_bounds__(kScanBlock) void sparse_scan_kernel(SegSrc src, Spa
     unsigned tot_gt, tot_eq;
     block_scan_pairs(c, nw, sh, stage, tot_gt, tot_eq);
     unsigned long long total = (unsigned long long)tot_gt + tot_eq;
-    if (total > s.cap) {
-        // More candidates than slots: the threshold becomes the capacity-th largest
-        // key of the whole tensor (all of those keys are >= the sampled threshold,
-        // hence inside flagged groups); ties at the new threshold are taken in
-        // ascending index order until the slots are full.
+    if (total > s.cap && tot_gt < s.cap) {
+        // More candidates than slots, but only because of ties at the threshold (gradients
+        // clipped by value do this): the capacity-th largest key of the tensor is the threshold
+        // itself, so it stays, the tile counts stand, and the ties are taken in ascending index
+        // order until the slots are full.
+        quota = s.cap - tot_gt;
+        total = s.cap;
+    } else if (total > s.cap) {
+        // More keys above the threshold than slots (the sample misjudged the tensor): the
+        // threshold becomes the capacity-th largest key of the whole tensor (all of those keys
+        // are >= the sampled threshold, hence inside flagged groups), found by this one
+        // workgroup; ties at the new threshold are rationed as above.
         const unsigned old = thr;
         const long long n = (long long)s.n;
-        const unsigned long long ngroups = (unsigned long long)s.ntiles * 64;
         const uint2* grec = ws.grec + (unsigned long long)s.tile0 * 64;
+        // a wavefront per tile: lane l looks at the record of group l, then the flagged groups are
+        // read eight at a time (lane l their element l), all eight loads in flight together
         thr = block_kth_largest(sc, s.cap, [&](auto f) {
-            for (unsigned long long g = wave; g < ngroups; g += kScanWaves) {
-                unsigned gm = grec[g].x & 0x7fffffffu;
-                if (gm >= old && gm > 0u) {
-                    long long e = (long long)g * 64 + lane;
-                    unsigned key = e < n ? key_of(s.s1[e]) : 0u;
-                    if (key >= old && key > 0u) f(key);
+            for (unsigned t = wave; t < nw; t += kScanWaves) {
+                const unsigned gm = grec[(unsigned long long)t * 64 + lane].x & 0x7fffffffu;
+                unsigned long long m = __ballot(gm >= old && gm > 0u);
+                const long long tb = (long long)t * kTile + lane;
+                while (m) {
+                    unsigned key[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        const unsigned gi = pop_bit(m);
+                        const long long e = tb + (long long)gi * 64;
+                        key[u] = (gi < 64u && e < n) ? key_of(s.s1[e]) : 0u;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        if (key[u] >= old && key[u] > 0u) f(key[u]);
                 }
             }
         });

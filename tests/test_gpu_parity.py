@@ -362,6 +362,33 @@ def test_sparse_overflow_ties(hp):
     assert oracle.sparse_unpack(want_pay)[0] == 64
 
 
+@pytest.mark.parametrize("alg", ["dgc", "graddrop"])
+def test_sparse_overflow_by_clipped_gradients(hp, alg):
+    """Gradients clipped by value: 5 % of a 3 M-element tensor sit at exactly +-0.01, far more
+    than the slots hold, and nothing lies above them.  The threshold stays at the clip value
+    and the ties go out in index order, step after step as the accumulator releases them; the
+    second step mixes released ties with accumulated values."""
+    n, ratio = 3_000_001, 0.001
+    rng = np.random.default_rng(17)
+    mom_ref, acc_ref = np.zeros(n, F), np.zeros(n, F)
+    mom, acc = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    for step in range(3):
+        g = np.clip(rng.normal(0, 5e-3, n), -0.01, 0.01).astype(F)
+        pay = payload(hp.sparse_payload_bytes(n, ratio))
+        if alg == "dgc":
+            hp.dgc_encode(dev(g), mom, acc, pay, 0.9, ratio)
+            want, mom_ref, acc_ref = oracle.dgc_encode(g, mom_ref, acc_ref, 0.9, ratio)
+            np.testing.assert_array_equal(host(mom), mom_ref, err_msg=f"momentum, step {step}")
+        else:
+            hp.graddrop_encode(dev(g), acc, pay, ratio)
+            want, acc_ref = oracle.graddrop_encode(g, acc_ref, ratio)
+        check_sparse(host(pay), want)
+        np.testing.assert_array_equal(host(acc), acc_ref, err_msg=f"accumulator, step {step}")
+        nnz, _, cap, *_ = oracle.sparse_unpack(want)
+        if step == 0:
+            assert nnz == cap  # the case meant: every slot used
+
+
 def test_sparse_overflow_rethreshold(hp):
     n = 262144
     rng = np.random.default_rng(11)
