@@ -211,8 +211,8 @@ int hipress_terngrad_decode_merge(const void *const *payloads, const int64_t *pa
 /* Sparse payloads must hold their pairs in ascending index order (the encoders
  * here write them so); a payload that does not is still merged correctly, but
  * every tile then looks through that peer's whole payload: time grows with
- * tiles x pairs, which is nothing for chunks of a few MB (the decode-and-merge
- * shape) and 27 ms for one 400 MB chunk with 4 x 100,000 pairs.  workspace: hipress_sparse_merge_workspace_bytes(n, npeers, ratio,
+ * tiles x pairs (168 chunks of 4 MB with 8 x 1,100 pairs each: 2.5 ms instead of
+ * 0.4 ms; one 400 MB chunk with 4 x 100,000 pairs: 27 ms).  workspace: hipress_sparse_merge_workspace_bytes(n, npeers, ratio,
  * accumulator != NULL); it needs no initialisation.  Every call stamps what it
  * finds out of order with a number of its own (a process-wide counter), which a
  * HIP graph freezes: in replays a peer whose payload was once out of order keeps
