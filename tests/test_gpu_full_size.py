@@ -392,6 +392,39 @@ def test_hip_graph_replay_matches_eager(hp):
         np.testing.assert_array_equal(host(out), eager[step][2], err_msg=f"decode, replay {step}")
 
 
+@pytest.mark.parametrize("bucket", [777, 100_000, 3_000_000])
+def test_hip_graph_replay_of_terngrad_with_long_buckets(hp, bucket):
+    """The encoders for bucket sizes that no wavefront covers (maxima gathered in LDS; beyond
+    a tile, three launches that park per-tile maxima in the payload's word area) captured
+    with the decode: each replay sees a new gradient in the same buffers and must give what
+    the oracle gives for it, also where the scales shrink from one replay to the next."""
+    n = 2_500_003
+    rng = np.random.default_rng(bucket)
+    g, u = torch.empty(n, device="cuda"), torch.empty(n, device="cuda")
+    pay = torch.zeros(hp.terngrad_payload_bytes(n, bucket), dtype=torch.uint8, device="cuda")
+    out = torch.empty(n, device="cuda")
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        g.zero_(); u.zero_()
+        hp.terngrad_encode(g, u, pay, bucket)  # warm-up on the capture stream
+        hp.terngrad_decode(pay, out)
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            hp.terngrad_encode(g, u, pay, bucket)
+            hp.terngrad_decode(pay, out)
+    for step, sigma in enumerate([1e-2, 1e-3, 1e-4]):
+        gh, uh = rng.normal(0, sigma, n).astype(np.float32), rng.random(n, dtype=np.float32)
+        g.copy_(torch.from_numpy(gh)); u.copy_(torch.from_numpy(uh))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        _ = (out * 2).sum().item()  # unrelated eager work between replays
+        want = oracle.terngrad_encode(gh, uh, bucket)
+        np.testing.assert_array_equal(host(pay), want, err_msg=f"payload, replay {step}")
+        np.testing.assert_array_equal(host(out), oracle.terngrad_decode(want, n), err_msg=f"decode, replay {step}")
+
+
 def test_hip_graph_replay_of_a_sparse_batch(hp):
     """The batched DGC encode + decode (ten launches, idle dynamic LDS on some, a per-call
     counter in the decode) captured once and replayed: every replay equals the eager run
