@@ -156,8 +156,9 @@ class SetWorkload:
     """encode+decode of one compressor over a list of tensor sizes through a Batch."""
 
     def __init__(self, name, alg, sizes, data, params, enc_bytes, dec_bytes, dominant_phase, dominant_kernel,
-                 dominant_bytes, rotate=1, nphases=1):
+                 dominant_bytes, rotate=1, nphases=1, seeded=False):
         self.name, self.alg, self.sizes, self.data, self.params = name, alg, sizes, data, params
+        self.seeded = seeded  # terngrad: no noise tensors, the kernels draw from a seed that changes every step
         self.enc_bytes, self.dec_bytes = enc_bytes, dec_bytes  # algorithmic bytes per element
         self.dominant_phase, self.dominant_kernel, self.dominant_bytes = dominant_phase, dominant_kernel, dominant_bytes
         self.rotate, self.nphases = rotate, nphases
@@ -206,7 +207,7 @@ class SetWorkload:
                     nb = hp.graddrop_payload_bytes(n, ratio)
                 t["compressed"] = torch.zeros(nb, dtype=torch.uint8, device=dev)
                 ts.append(t)
-            if self.alg == "terngrad":
+            if self.alg == "terngrad" and not self.seeded:
                 for t, u in zip(ts, W.uniform_set(self.sizes, dev, 1000 + seed)):
                     t["uniform"] = u
             self.tensors.append(ts)
@@ -216,7 +217,13 @@ class SetWorkload:
     def step(self, ev=None):
         b = self.batches[self.k % self.rotate]
         self.k += 1
-        if ev is None:
+        if self.seeded:
+            if ev is not None:
+                ev[0].record()
+            b.encode(seed=self.k)
+            if ev is not None:
+                ev[1].record()
+        elif ev is None:
             b.encode()
         else:
             for ph in range(self.nphases):
@@ -238,7 +245,10 @@ class SetWorkload:
         picks, total = _sample_front(self.sizes)
         ts = self.tensors[0]
         g = [ts[i]["gradient"][:k].cpu().numpy() for i, k in picks]
-        u = [ts[i]["uniform"][:k].cpu().numpy() for i, k in picks] if self.alg == "terngrad" else None
+        u = None
+        if self.alg == "terngrad":
+            u = [np.empty(k, np.float32) if self.seeded else ts[i]["uniform"][:k].cpu().numpy() for i, k in picks]
+        seeded = self.seeded
         zeros = lambda: [np.zeros(k, np.float32) for _, k in picks]
         s0, s1 = zeros(), zeros()
         out = [np.empty(k, np.float32) for _, k in picks]
@@ -260,6 +270,8 @@ class SetWorkload:
                     L.hpo_onebit_encode(_vp(g[j]), _vp(s0[j]), k, _vp(pay[j]))
                     L.hpo_onebit_decode(_vp(pay[j]), _vp(out[j]), k)
                 elif alg == "terngrad":
+                    if seeded:  # the draws are part of the operator
+                        L.hpo_uniform_draws(1, j, _vp(u[j]), k)
                     L.hpo_terngrad_encode(_vp(g[j]), _vp(u[j]), k, _vp(pay[j]), pr.get("bucket", 512))
                     L.hpo_terngrad_decode(_vp(pay[j]), _vp(out[j]), k)
                 elif alg == "dgc":
@@ -549,6 +561,10 @@ def make_workload(name):
         return SetWorkload(name, "tbq", vgg, "vgg", {"threshold": 0.05}, 12.25, 4.25, 0, "tbq_encode_kernel", 12.25)
     if name == "terngrad_vgg19":
         return SetWorkload(name, "terngrad", vgg, "vgg", {"bucket": 512}, 8.2578, 4.2578, 0, "terngrad_encode_kernel", 8.2578)
+    if name == "terngrad_seeded_vgg19":
+        # no noise tensor: 4 bytes per element fewer for the encoder to read
+        return SetWorkload(name, "terngrad", vgg, "vgg", {"bucket": 512}, 4.2578, 4.2578, 0, "terngrad_encode_kernel", 4.2578,
+                           seeded=True)
     if name == "dgc_vgg19":
         return SetWorkload(name, "dgc", vgg, "vgg", {"momentum_factor": 0.9, "ratio": 0.001}, 20.0, 4.0, 0,
                            "sparse_accum_kernel", 20.0, nphases=7)
@@ -597,6 +613,7 @@ ALL_WORKLOADS = [
     "tbq_262144", "tbq_262144_x512", "terngrad_resnet50", "dgc_bert_large", "graddrop_bert_large",
     "merge_tbq_vgg19", "merge_dgc_vgg19", "compll_b2_fc6", "compll_generated_b2_fc6", "tbq_fc6", "tbq_generated_fc6",
     "merge_tbq_vgg19_payload_only", "merge_dgc_vgg19_payload_only", "tbq_vgg19_planned", "hop_tbq_vgg19",
+    "terngrad_seeded_vgg19",
 ]
 # any workload with the suffix _graph: the same step captured once into a HIP graph and replayed
 EXTRA_WORKLOADS = [w + "_graph" for w in ALL_WORKLOADS]

@@ -65,11 +65,14 @@ SIGNATURES = {
     "hipress_onebit_encode_deferred": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "hipress_onebit_residual": (ctypes.c_int, [_vp, _vp, _i64, _vp, _vp]),
     "hipress_terngrad_encode": (ctypes.c_int, [_vp, _vp, _i64, _vp, _i64, _i32, _vp]),
+    "hipress_terngrad_encode_seeded": (ctypes.c_int, [_vp, _i64, _vp, _i64, _i32, ctypes.c_uint64, _vp]),
+    "hipress_uniform_fill": (ctypes.c_int, [_vp, _i64, ctypes.c_uint64, ctypes.c_uint32, _vp]),
     "hipress_terngrad_decode": (ctypes.c_int, [_vp, _i64, _vp, _i64, _vp]),
     "hipress_compll_payload_bytes": (_i64, [_i64, _i32]),
     "hipress_compll_workspace_bytes": (_i64, [_i64]),
     "hipress_compll_decoded_count": (_i64, [_i64, _i32]),
     "hipress_compll_encode": (ctypes.c_int, [_vp, _vp, _i64, _vp, _i64, _i32, _vp, _i64, _vp]),
+    "hipress_compll_encode_seeded": (ctypes.c_int, [_vp, _i64, _vp, _i64, _i32, ctypes.c_uint64, _vp, _i64, _vp]),
     "hipress_compll_decode": (ctypes.c_int, [_vp, _i64, _vp, _i64, _vp]),
     "hipress_dgc_encode": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp, _i64, _f32, _f64, _vp, _i64, _vp]),
     "hipress_graddrop_encode": (ctypes.c_int, [_vp, _vp, _i64, _vp, _i64, _f64, _vp, _i64, _vp]),
@@ -84,6 +87,7 @@ SIGNATURES = {
     "hipress_sparse_decode_merge_local": (ctypes.c_int, [_vp, _vp, _i32, _vp, _vp, _i64, _vp, _vp, _i64, _f64, _vp, _i64, _vp]),
     "hipress_batch_create": (ctypes.c_int, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(Tensor), _i32, ctypes.POINTER(Params)]),
     "hipress_batch_encode": (ctypes.c_int, [_vp, _vp]),
+    "hipress_batch_encode_seeded": (ctypes.c_int, [_vp, ctypes.c_uint64, _vp]),
     "hipress_batch_decode": (ctypes.c_int, [_vp, _vp]),
     "hipress_batch_encode_phase": (ctypes.c_int, [_vp, _i32, _vp]),
     "hipress_batch_destroy": (ctypes.c_int, [_vp]),

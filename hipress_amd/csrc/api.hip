@@ -146,7 +146,8 @@ int check_params(int alg, const hipress_params& pr) {
 }
 
 // Fills the fields of `s` that do not depend on the tensor's place in a launch.
-int build_encode_seg(int alg, const hipress_tensor& t, const hipress_params& pr, Seg* s) {
+// drawn: the stochastic rounding's noise is drawn in the kernel, so no noise tensor is asked for.
+int build_encode_seg(int alg, const hipress_tensor& t, const hipress_params& pr, Seg* s, bool drawn = false) {
     std::memset(s, 0, sizeof(Seg));
     if (bad_n(t.n) || (is_sparse(alg) && bad_sparse_n(t.n))) return HIPRESS_ERR_SIZE;
     int rc = check_params(alg, pr);
@@ -158,7 +159,7 @@ int build_encode_seg(int alg, const hipress_tensor& t, const hipress_params& pr,
     if (t.payload_bytes < need) return HIPRESS_ERR_SIZE;
     const bool need_s0 = alg != HIPRESS_TERNGRAD;
     const bool need_s1 = alg == HIPRESS_DGC || alg == HIPRESS_ONEBIT_DEFERRED;
-    const bool need_u = alg == HIPRESS_TERNGRAD;
+    const bool need_u = alg == HIPRESS_TERNGRAD && !drawn;
     if (t.n > 0) {
         if (!t.grad || (need_s0 && !t.state0) || (need_s1 && !t.state1) || (need_u && !t.uniform)) return HIPRESS_ERR_NULL;
     }
@@ -180,8 +181,8 @@ int build_encode_seg(int alg, const hipress_tensor& t, const hipress_params& pr,
             s->words_off = HIPRESS_HEADER_BYTES;
             break;
         case HIPRESS_TERNGRAD: {
-            s->u = t.uniform;
-            s->aligned = s->aligned && vec_ok(t.uniform);
+            s->u = drawn ? nullptr : t.uniform;
+            s->aligned = s->aligned && (drawn || vec_ok(t.uniform));
             s->bucket = (unsigned)pr.bucket;
             int64_t off = HIPRESS_HEADER_BYTES + tg_scale_bytes(t.n, pr.bucket);
             if (off > 0xffffffffLL) return HIPRESS_ERR_SIZE;
@@ -332,6 +333,7 @@ struct hipress_batch {
     hipress_params params{};
     std::vector<Seg> enc, dec;
     bool can_encode = false, can_decode = false;
+    bool drawn = false;  // terngrad: no tensor brings a noise tensor, the encode call brings a seed
     Seg* d_enc = nullptr;
     Seg* d_dec = nullptr;
     uint2* d_map = nullptr;
@@ -544,7 +546,27 @@ int hipress_terngrad_encode(const float* grad, const float* uniform, int64_t n, 
     Seg s;
     int rc = build_encode_seg(HIPRESS_TERNGRAD, t, pr, &s);
     if (rc) return rc;
-    return hiperr(launch_terngrad_encode(single_launch(s), (unsigned)bucket, static_cast<hipStream_t>(stream)));
+    return hiperr(launch_terngrad_encode(single_launch(s), (unsigned)bucket, false, 0u, static_cast<hipStream_t>(stream)));
+}
+
+int hipress_terngrad_encode_seeded(const float* grad, int64_t n, void* payload, int64_t payload_bytes, int32_t bucket,
+                                   uint64_t seed, void* stream) {
+    hipress_tensor t{grad, nullptr, nullptr, nullptr, payload, nullptr, n, payload_bytes};
+    hipress_params pr{};
+    pr.bucket = bucket;
+    Seg s;
+    int rc = build_encode_seg(HIPRESS_TERNGRAD, t, pr, &s, true);
+    if (rc) return rc;
+    return hiperr(launch_terngrad_encode(single_launch(s), (unsigned)bucket, true, uniform_key(seed),
+                                         static_cast<hipStream_t>(stream)));
+}
+
+int hipress_uniform_fill(float* out, int64_t n, uint64_t seed, uint32_t tensor, void* stream) {
+    if (bad_n(n)) return HIPRESS_ERR_SIZE;
+    if (n > 0 && !out) return HIPRESS_ERR_NULL;
+    if (mis(out, 4)) return HIPRESS_ERR_ALIGN;
+    return hiperr(launch_uniform_fill(out, (unsigned long long)n, tensor_key(uniform_key(seed), tensor),
+                                      static_cast<hipStream_t>(stream)));
 }
 
 // The bucket size is read from the payload header on the device and the scale
@@ -580,12 +602,12 @@ int64_t hipress_compll_workspace_bytes(int64_t n) {
     return bad_n(n) ? HIPRESS_ERR_SIZE : round_up(8 * (int64_t)tiles_of(n), 256);
 }
 
-int hipress_compll_encode(const float* grad, const float* uniform, int64_t n, void* compressed,
-                          int64_t compressed_bytes, int32_t bitwidth, void* workspace, int64_t workspace_bytes,
-                          void* stream) {
+static int compll_encode_impl(const float* grad, const float* uniform, bool drawn, uint64_t seed, int64_t n,
+                              void* compressed, int64_t compressed_bytes, int32_t bitwidth, void* workspace,
+                              int64_t workspace_bytes, void* stream) {
     int64_t need = hipress_compll_payload_bytes(n, bitwidth);
     if (need < 0) return (int)need;
-    if (!compressed || (n > 0 && (!grad || !uniform))) return HIPRESS_ERR_NULL;
+    if (!compressed || (n > 0 && (!grad || (!drawn && !uniform)))) return HIPRESS_ERR_NULL;
     if (mis(grad, 4) || mis(uniform, 4)) return HIPRESS_ERR_ALIGN;
     if (compressed_bytes < need) return HIPRESS_ERR_SIZE;
     if (!workspace || workspace_bytes < hipress_compll_workspace_bytes(n)) return HIPRESS_ERR_WORKSPACE;
@@ -593,14 +615,28 @@ int hipress_compll_encode(const float* grad, const float* uniform, int64_t n, vo
     Seg s;
     std::memset(&s, 0, sizeof s);
     s.g = grad;
-    s.u = uniform;
+    s.u = drawn ? nullptr : uniform;
     s.pay = static_cast<uint8_t*>(compressed);
     s.n = (unsigned long long)n;
     s.ntiles = tiles_of(n);
-    s.aligned = vec_ok(grad) && vec_ok(uniform);
+    s.aligned = vec_ok(grad) && (drawn || vec_ok(uniform));
     s.bucket = (unsigned)bitwidth;
-    return hiperr(launch_compll_encode(single_launch(s), bitwidth, static_cast<float*>(workspace),
-                                       static_cast<hipStream_t>(stream)));
+    return hiperr(launch_compll_encode(single_launch(s), bitwidth, static_cast<float*>(workspace), drawn,
+                                       drawn ? uniform_key(seed) : 0u, static_cast<hipStream_t>(stream)));
+}
+
+int hipress_compll_encode(const float* grad, const float* uniform, int64_t n, void* compressed,
+                          int64_t compressed_bytes, int32_t bitwidth, void* workspace, int64_t workspace_bytes,
+                          void* stream) {
+    return compll_encode_impl(grad, uniform, false, 0, n, compressed, compressed_bytes, bitwidth, workspace,
+                              workspace_bytes, stream);
+}
+
+int hipress_compll_encode_seeded(const float* grad, int64_t n, void* compressed, int64_t compressed_bytes,
+                                 int32_t bitwidth, uint64_t seed, void* workspace, int64_t workspace_bytes,
+                                 void* stream) {
+    return compll_encode_impl(grad, nullptr, true, seed, n, compressed, compressed_bytes, bitwidth, workspace,
+                              workspace_bytes, stream);
 }
 
 int hipress_compll_decode(const void* compressed, int64_t compressed_bytes, float* out, int64_t n, void* stream) {
@@ -861,6 +897,14 @@ static int batch_create_impl(hipress_batch** out, int32_t alg, const hipress_ten
         if (t.n > 0 && !t.out) dec_ok = false;
     }
     if (!enc_ok && !dec_ok) { delete b; return HIPRESS_ERR_NULL; }
+    if (alg == HIPRESS_TERNGRAD && enc_ok) {
+        // either every tensor brings its noise, or none does and the encode calls bring a seed
+        int with = 0, without = 0;
+        for (int i = 0; i < count; ++i)
+            if (tensors[i].n > 0) (tensors[i].uniform ? with : without)++;
+        if (with && without) { delete b; return HIPRESS_ERR_NULL; }
+        b->drawn = without > 0;
+    }
     b->can_encode = enc_ok;
     b->can_decode = dec_ok;
     struct Guard {  // frees the half-built batch on every way out but the last
@@ -872,7 +916,7 @@ static int batch_create_impl(hipress_batch** out, int32_t alg, const hipress_ten
         const hipress_tensor& t = tensors[i];
         Seg s;
         if (enc_ok) {
-            if ((rc = build_encode_seg(alg, t, *params, &s))) return fail(rc);
+            if ((rc = build_encode_seg(alg, t, *params, &s, b->drawn))) return fail(rc);
             b->enc.push_back(s);
         }
         if (dec_ok) {
@@ -943,9 +987,10 @@ static Launch batch_launch(const hipress_batch* b, bool encode) {
     return L;
 }
 
-static int batch_encode_impl(hipress_batch* b, int phase, void* stream) {
+static int batch_encode_impl(hipress_batch* b, int phase, void* stream, bool seeded = false, uint64_t seed = 0) {
     if (!b) return HIPRESS_ERR_NULL;
     if (!b->can_encode) return HIPRESS_ERR_NULL;
+    if (seeded != b->drawn) return HIPRESS_ERR_PARAM;  // a seed goes with a batch without noise tensors, and only with it
     if (b->enc.empty()) return HIPRESS_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
     Launch L = batch_launch(b, true);
@@ -961,7 +1006,7 @@ static int batch_encode_impl(hipress_batch* b, int phase, void* stream) {
             return hiperr(launch_tbq_encode(L, st));
         case HIPRESS_TERNGRAD:
             if (phase > 0) return HIPRESS_ERR_PARAM;
-            return hiperr(launch_terngrad_encode(L, (unsigned)b->params.bucket, st));
+            return hiperr(launch_terngrad_encode(L, (unsigned)b->params.bucket, b->drawn, b->drawn ? uniform_key(seed) : 0u, st));
         case HIPRESS_DGC:
         case HIPRESS_GRADDROP:
             if (phase > 6) return HIPRESS_ERR_PARAM;
@@ -971,6 +1016,10 @@ static int batch_encode_impl(hipress_batch* b, int phase, void* stream) {
 }
 
 int hipress_batch_encode(hipress_batch* b, void* stream) { return batch_encode_impl(b, -1, stream); }
+
+int hipress_batch_encode_seeded(hipress_batch* b, uint64_t seed, void* stream) {
+    return batch_encode_impl(b, -1, stream, true, seed);
+}
 
 int hipress_batch_encode_phase(hipress_batch* b, int32_t phase, void* stream) {
     if (phase < 0) return HIPRESS_ERR_PARAM;

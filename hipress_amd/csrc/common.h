@@ -12,6 +12,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "uniform_draw.h"
+
 namespace hp {
 
 typedef float f4 __attribute__((ext_vector_type(4)));
@@ -170,6 +172,21 @@ template <bool FAST>
 __device__ __forceinline__ void store4(float* p, long long e, long long n, f4 v) {
     if (FAST) st4(p + e, v);
     else st4_guard(p, e, n, v);
+}
+// The noise of the stochastic quantisers for the four elements from e on: read from the noise
+// tensor, or (DRAW) drawn from the tensor's key and the element's index (uniform_draw.h).
+template <bool FAST, bool DRAW>
+__device__ __forceinline__ f4 noise4(const float* u, long long e, long long n, unsigned key) {
+    if (DRAW) {
+        const uint32_t i = (uint32_t)e;  // element counts fit 32 bits
+        f4 v;
+        v.x = uniform_at(i, key);
+        v.y = uniform_at(i + 1u, key);
+        v.z = uniform_at(i + 2u, key);
+        v.w = uniform_at(i + 3u, key);
+        return v;
+    }
+    return load4<FAST>(u, e, n);
 }
 // bit k set when element e+k exists
 __device__ __forceinline__ unsigned valid4(long long e, long long n) {

@@ -109,8 +109,10 @@ __device__ __forceinline__ unsigned compll_code(float g, float u, float mn, floa
     return !(f > 0.f) ? 0u : (f >= top ? (unsigned)top : (unsigned)f);  // NaN -> 0
 }
 
-template <class Src, int B>
-__global__ __launch_bounds__(kBlock) void compll_quant_kernel(Src src) {
+// DRAW: the noise is drawn in the kernel from `key` and the element's index (uniform_draw.h);
+// otherwise it is read from the tensor the descriptor names.
+template <class Src, int B, bool DRAW>
+__global__ __launch_bounds__(kBlock) void compll_quant_kernel(Src src, unsigned key) {
     unsigned tile;
     const Seg s = src.get(tile, xcd_reversed(blockIdx.x, gridDim.x));  // begins where the min/max pass ended
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
@@ -122,12 +124,13 @@ __global__ __launch_bounds__(kBlock) void compll_quant_kernel(Src src) {
     const float gap = (mx - mn) / top;
     uint8_t* Q = s.pay + 10;
     const long long nbytes = (n * B + 7) / 8;
+    const unsigned tkey = DRAW ? tensor_key(key, s.id) : 0u;
     f4 g[4], u[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         long long e = base + j * 256 + lane * 4;
         g[j] = fast ? ld4(s.g + e) : ld4_guard(s.g, e, n);
-        u[j] = fast ? ld4(s.u + e) : ld4_guard(s.u, e, n);
+        u[j] = DRAW ? noise4<true, true>(nullptr, e, n, tkey) : (fast ? ld4(s.u + e) : ld4_guard(s.u, e, n));
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -208,23 +211,27 @@ __global__ __launch_bounds__(kBlock) void compll_decode_kernel(Src src) {
     }
 }
 
-template <class Src, class SegSrcT>
+template <class Src, class SegSrcT, bool DRAW>
 static hipError_t compll_encode_src(const Src& src, const SegSrcT& ssrc, unsigned ntiles, unsigned nsegs, int b,
-                                    float* partial, hipStream_t st) {
+                                    float* partial, unsigned key, hipStream_t st) {
     hipLaunchKernelGGL((compll_minmax_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src, partial);
     hipLaunchKernelGGL((compll_header_kernel<SegSrcT>), dim3(nsegs), dim3(kHeaderBlock), 0, st, ssrc, partial);
-    if (b == 1) hipLaunchKernelGGL((compll_quant_kernel<Src, 1>), dim3(ntiles), dim3(kBlock), 0, st, src);
-    else if (b == 2) hipLaunchKernelGGL((compll_quant_kernel<Src, 2>), dim3(ntiles), dim3(kBlock), 0, st, src);
-    else if (b == 4) hipLaunchKernelGGL((compll_quant_kernel<Src, 4>), dim3(ntiles), dim3(kBlock), 0, st, src);
-    else hipLaunchKernelGGL((compll_quant_kernel<Src, 8>), dim3(ntiles), dim3(kBlock), 0, st, src);
+    if (b == 1) hipLaunchKernelGGL((compll_quant_kernel<Src, 1, DRAW>), dim3(ntiles), dim3(kBlock), 0, st, src, key);
+    else if (b == 2) hipLaunchKernelGGL((compll_quant_kernel<Src, 2, DRAW>), dim3(ntiles), dim3(kBlock), 0, st, src, key);
+    else if (b == 4) hipLaunchKernelGGL((compll_quant_kernel<Src, 4, DRAW>), dim3(ntiles), dim3(kBlock), 0, st, src, key);
+    else hipLaunchKernelGGL((compll_quant_kernel<Src, 8, DRAW>), dim3(ntiles), dim3(kBlock), 0, st, src, key);
     return hipGetLastError();
 }
 
-// partial: two floats per tile
-hipError_t launch_compll_encode(const Launch& L, int bitwidth, float* partial, hipStream_t st) {
+// partial: two floats per tile.  draw: the noise comes from `key`, not from the descriptors' tensors.
+hipError_t launch_compll_encode(const Launch& L, int bitwidth, float* partial, bool draw, unsigned key, hipStream_t st) {
     if (L.ntiles == 0) return hipSuccess;
-    if (L.single) return compll_encode_src(SingleSrc{L.seg}, SingleSegSrc{L.seg}, L.ntiles, 1, bitwidth, partial, st);
-    return compll_encode_src(BatchSrc{L.dsegs, L.dmap}, BatchSegSrc{L.dsegs}, L.ntiles, L.nsegs, bitwidth, partial, st);
+    if (L.single) {
+        if (draw) return compll_encode_src<SingleSrc, SingleSegSrc, true>(SingleSrc{L.seg}, SingleSegSrc{L.seg}, L.ntiles, 1, bitwidth, partial, key, st);
+        return compll_encode_src<SingleSrc, SingleSegSrc, false>(SingleSrc{L.seg}, SingleSegSrc{L.seg}, L.ntiles, 1, bitwidth, partial, 0u, st);
+    }
+    if (draw) return compll_encode_src<BatchSrc, BatchSegSrc, true>(BatchSrc{L.dsegs, L.dmap}, BatchSegSrc{L.dsegs}, L.ntiles, L.nsegs, bitwidth, partial, key, st);
+    return compll_encode_src<BatchSrc, BatchSegSrc, false>(BatchSrc{L.dsegs, L.dmap}, BatchSegSrc{L.dsegs}, L.ntiles, L.nsegs, bitwidth, partial, 0u, st);
 }
 
 hipError_t launch_compll_decode(const Launch& L, hipStream_t st) {

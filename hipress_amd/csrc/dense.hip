@@ -423,8 +423,8 @@ __device__ __forceinline__ unsigned tern_code4(f4 g, f4 u, float s) {
 // Bucket sizes 256, 512 and 1024 divide a wavefront's 1024 elements, so the
 // bucket maximum is a wavefront reduction over values already in registers and
 // the whole encode is a single pass.  BPW = buckets per wavefront tile.
-template <bool FAST, int BPW>
-__device__ __forceinline__ void terngrad_encode_tile(const Seg& s, unsigned tile) {
+template <bool FAST, int BPW, bool DRAW>
+__device__ __forceinline__ void terngrad_encode_tile(const Seg& s, unsigned tile, unsigned key) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long n = (long long)s.n;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
@@ -436,7 +436,7 @@ __device__ __forceinline__ void terngrad_encode_tile(const Seg& s, unsigned tile
     for (int j = 0; j < 4; ++j) {
         long long e = base + j * 256 + lane * 4;
         g[j] = load4<FAST>(s.g, e, n);
-        u[j] = load4<FAST>(s.u, e, n);
+        u[j] = noise4<FAST, DRAW>(s.u, e, n, key);
     }
     float sc[4];
     constexpr int SPB = 4 / BPW;  // steps per bucket
@@ -471,8 +471,11 @@ __device__ __forceinline__ void terngrad_zero_scale_pad(const Seg& s, unsigned t
     }
 }
 
-template <class Src, int BPW>
-__global__ __launch_bounds__(kBlock) void terngrad_encode_kernel(Src src) {
+// DRAW: the noise is drawn in the kernel from `key` (the call's), the tensor's place in the
+// launch's table and the element's index; otherwise it is read from the tensor the descriptor
+// names and `key` is not used.
+template <class Src, int BPW, bool DRAW>
+__global__ __launch_bounds__(kBlock) void terngrad_encode_kernel(Src src, unsigned key) {
     unsigned tile;
     const Seg s = src.get(tile, blockIdx.x);
     if (tile == 0 && threadIdx.x == 0) {
@@ -483,8 +486,9 @@ __global__ __launch_bounds__(kBlock) void terngrad_encode_kernel(Src src) {
         h[3] = 0;
     }
     terngrad_zero_scale_pad(s, tile);
-    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) terngrad_encode_tile<true, BPW>(s, tile);
-    else terngrad_encode_tile<false, BPW>(s, tile);
+    const unsigned tkey = DRAW ? tensor_key(key, s.id) : 0u;
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) terngrad_encode_tile<true, BPW, DRAW>(s, tile, tkey);
+    else terngrad_encode_tile<false, BPW, DRAW>(s, tile, tkey);
 }
 
 // Any other bucket size up to a tile (4096): still a single pass.  A tile's elements lie in
@@ -504,8 +508,8 @@ __device__ __forceinline__ unsigned absmax_key(float x) {
     return k > 0x7f800000u ? 0u : k;  // NaN contributes nothing
 }
 
-template <bool FAST>
-__device__ __forceinline__ void terngrad_encode_any_tile(const Seg& s, unsigned tile, unsigned* mx) {
+template <bool FAST, bool DRAW>
+__device__ __forceinline__ void terngrad_encode_any_tile(const Seg& s, unsigned tile, unsigned* mx, unsigned key) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long n = (long long)s.n;
     const unsigned B = s.bucket;
@@ -525,7 +529,7 @@ __device__ __forceinline__ void terngrad_encode_any_tile(const Seg& s, unsigned 
     for (int j = 0; j < 4; ++j) {
         const long long e = base + j * 256 + lane * 4;
         g[j] = load4<FAST>(s.g, e, n);
-        u[j] = load4<FAST>(s.u, e, n);
+        u[j] = noise4<FAST, DRAW>(s.u, e, n, key);
     }
     __syncthreads();
     // what hangs over from the neighbours: fewer than B elements on either side
@@ -607,8 +611,8 @@ __device__ __forceinline__ void terngrad_encode_any_tile(const Seg& s, unsigned 
     if (FAST || widx < (long long)((n + 15) >> 4)) words[widx] = myword;
 }
 
-template <class Src>
-__global__ __launch_bounds__(kBlock) void terngrad_encode_any_kernel(Src src) {
+template <class Src, bool DRAW>
+__global__ __launch_bounds__(kBlock) void terngrad_encode_any_kernel(Src src, unsigned key) {
     __shared__ unsigned mx[kAnyBuckets];
     unsigned tile;
     const Seg s = src.get(tile, blockIdx.x);
@@ -621,8 +625,9 @@ __global__ __launch_bounds__(kBlock) void terngrad_encode_any_kernel(Src src) {
     }
     terngrad_zero_scale_pad(s, tile);
     if ((unsigned long long)tile * kTile >= s.n) return;  // an empty tensor has one tile and nothing in it
-    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) terngrad_encode_any_tile<true>(s, tile, mx);
-    else terngrad_encode_any_tile<false>(s, tile, mx);
+    const unsigned tkey = DRAW ? tensor_key(key, s.id) : 0u;
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) terngrad_encode_any_tile<true, DRAW>(s, tile, mx, tkey);
+    else terngrad_encode_any_tile<false, DRAW>(s, tile, mx, tkey);
 }
 
 // Bucket sizes beyond a tile, up to the whole tensor: a tile then lies in at most two buckets, and a
@@ -736,8 +741,8 @@ __global__ __launch_bounds__(kBlock) void terngrad_scale_big_kernel(Src src) {
     if (threadIdx.x == 0) reinterpret_cast<float*>(s.pay + kHeaderBytes)[first] = __uint_as_float(k);
 }
 
-template <bool FAST>
-__device__ __forceinline__ void terngrad_quant_big_tile(const Seg& s, unsigned tile) {
+template <bool FAST, bool DRAW>
+__device__ __forceinline__ void terngrad_quant_big_tile(const Seg& s, unsigned tile, unsigned key) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const long long n = (long long)s.n;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
@@ -750,7 +755,7 @@ __device__ __forceinline__ void terngrad_quant_big_tile(const Seg& s, unsigned t
     for (int j = 0; j < 4; ++j) {
         const long long e = base + j * 256 + lane * 4;
         g[j] = load4<FAST>(s.g, e, n);
-        u[j] = load4<FAST>(s.u, e, n);
+        u[j] = noise4<FAST, DRAW>(s.u, e, n, key);
     }
     const float sa = scales[t.b0];
     const float sb = (unsigned long long)tile * kTile + t.bnd < (unsigned long long)n && t.bnd < (unsigned long long)kTile ? scales[t.b0 + 1u] : 0.f;
@@ -776,12 +781,13 @@ __device__ __forceinline__ void terngrad_quant_big_tile(const Seg& s, unsigned t
     if (FAST || widx < (long long)((n + 15) >> 4)) words[widx] = myword;
 }
 
-template <class Src>
-__global__ __launch_bounds__(kBlock) void terngrad_quant_big_kernel(Src src) {
+template <class Src, bool DRAW>
+__global__ __launch_bounds__(kBlock) void terngrad_quant_big_kernel(Src src, unsigned key) {
     unsigned tile;
     const Seg s = src.get(tile, blockIdx.x);
-    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) terngrad_quant_big_tile<true>(s, tile);
-    else terngrad_quant_big_tile<false>(s, tile);
+    const unsigned tkey = DRAW ? tensor_key(key, s.id) : 0u;
+    if (s.aligned && (unsigned long long)(tile + 1) * kTile <= s.n) terngrad_quant_big_tile<true, DRAW>(s, tile, tkey);
+    else terngrad_quant_big_tile<false, DRAW>(s, tile, tkey);
 }
 
 // Decode.  The bucket size is in the payload header, and with it the place of the
@@ -990,25 +996,53 @@ hipError_t launch_onebit_encode_deferred(const Launch& L, float* partial, int ph
 
 hipError_t launch_onebit_materialize(const Launch& L, hipStream_t st) { HP_LAUNCH(onebit_materialize_kernel, kLdsFor5, L, st); }
 
-template <class Src>
-static hipError_t terngrad_encode_src(const Src& src, unsigned ntiles, unsigned bucket, hipStream_t st) {
-    if (bucket == 256) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 4>), dim3(ntiles), dim3(kBlock), kLdsFor5, st, src);
-    else if (bucket == 512) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 2>), dim3(ntiles), dim3(kBlock), kLdsFor5, st, src);
-    else if (bucket == 1024) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 1>), dim3(ntiles), dim3(kBlock), kLdsFor5, st, src);
-    else if (bucket <= kAnyBucketMax) hipLaunchKernelGGL((terngrad_encode_any_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);
+template <class Src, bool DRAW>
+static hipError_t terngrad_encode_src(const Src& src, unsigned ntiles, unsigned bucket, unsigned key, hipStream_t st) {
+    const dim3 g(ntiles), b(kBlock);
+    if (bucket == 256) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 4, DRAW>), g, b, kLdsFor5, st, src, key);
+    else if (bucket == 512) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 2, DRAW>), g, b, kLdsFor5, st, src, key);
+    else if (bucket == 1024) hipLaunchKernelGGL((terngrad_encode_kernel<Src, 1, DRAW>), g, b, kLdsFor5, st, src, key);
+    else if (bucket <= kAnyBucketMax) hipLaunchKernelGGL((terngrad_encode_any_kernel<Src, DRAW>), g, b, 0, st, src, key);
     else {
-        hipLaunchKernelGGL((terngrad_partial_big_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);
-        hipLaunchKernelGGL((terngrad_scale_big_kernel<Src>), dim3(ntiles), dim3(kBlock), 0, st, src);
-        hipLaunchKernelGGL((terngrad_quant_big_kernel<Src>), dim3(ntiles), dim3(kBlock), kLdsFor5, st, src);
+        hipLaunchKernelGGL((terngrad_partial_big_kernel<Src>), g, b, 0, st, src);
+        hipLaunchKernelGGL((terngrad_scale_big_kernel<Src>), g, b, 0, st, src);
+        hipLaunchKernelGGL((terngrad_quant_big_kernel<Src, DRAW>), g, b, kLdsFor5, st, src, key);
     }
     return hipGetLastError();
 }
 
-// All tensors of one launch share the bucket size.
-hipError_t launch_terngrad_encode(const Launch& L, unsigned bucket, hipStream_t st) {
+// All tensors of one launch share the bucket size.  draw: the noise is drawn in the kernels from
+// `key` (uniform_draw.h) instead of being read from the tensors the descriptors name.
+hipError_t launch_terngrad_encode(const Launch& L, unsigned bucket, bool draw, unsigned key, hipStream_t st) {
     if (L.ntiles == 0) return hipSuccess;
-    if (L.single) return terngrad_encode_src(SingleSrc{L.seg}, L.ntiles, bucket, st);
-    return terngrad_encode_src(BatchSrc{L.dsegs, L.dmap}, L.ntiles, bucket, st);
+    if (L.single) {
+        if (draw) return terngrad_encode_src<SingleSrc, true>(SingleSrc{L.seg}, L.ntiles, bucket, key, st);
+        return terngrad_encode_src<SingleSrc, false>(SingleSrc{L.seg}, L.ntiles, bucket, 0u, st);
+    }
+    if (draw) return terngrad_encode_src<BatchSrc, true>(BatchSrc{L.dsegs, L.dmap}, L.ntiles, bucket, key, st);
+    return terngrad_encode_src<BatchSrc, false>(BatchSrc{L.dsegs, L.dmap}, L.ntiles, bucket, 0u, st);
+}
+
+// out[i] = the draw an encoder makes for element i of the tensor with this key.
+__global__ __launch_bounds__(kBlock) void uniform_fill_kernel(float* out, unsigned long long n, unsigned key, unsigned aligned) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const long long base = (long long)blockIdx.x * kTile + wave * kWaveTile;
+    const bool fast = aligned && (unsigned long long)(blockIdx.x + 1) * kTile <= n;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const long long e = base + j * 256 + lane * 4;
+        const f4 v = noise4<true, true>(nullptr, e, (long long)n, key);
+        if (fast) st4(out + e, v);
+        else st4_guard(out, e, (long long)n, v);
+    }
+}
+
+hipError_t launch_uniform_fill(float* out, unsigned long long n, unsigned key, hipStream_t st) {
+    if (n == 0) return hipSuccess;
+    const unsigned ntiles = (unsigned)((n + kTile - 1) / kTile);
+    hipLaunchKernelGGL(uniform_fill_kernel, dim3(ntiles), dim3(kBlock), 0, st, out, n, key,
+                       (unsigned)((reinterpret_cast<uintptr_t>(out) & 3u) == 0));
+    return hipGetLastError();
 }
 
 }  // namespace hp

@@ -10,11 +10,12 @@ hipError_t launch_onebit_encode(const Launch& L, float* partial, int phase, hipS
 hipError_t launch_onebit_decode(const Launch& L, hipStream_t st);
 hipError_t launch_onebit_encode_deferred(const Launch& L, float* partial, int phase, hipStream_t st);
 hipError_t launch_onebit_materialize(const Launch& L, hipStream_t st);
-hipError_t launch_terngrad_encode(const Launch& L, unsigned bucket, hipStream_t st);
+hipError_t launch_terngrad_encode(const Launch& L, unsigned bucket, bool draw, unsigned key, hipStream_t st);  // draw: noise from key, not from the tensors
+hipError_t launch_uniform_fill(float* out, unsigned long long n, unsigned key, hipStream_t st);
 hipError_t launch_terngrad_decode(const Launch& L, unsigned bucket, hipStream_t st);  // bucket: what the launch's descriptors name, 0 = unknown
 
 // The in-tree CompLL operator (10-byte header, b-bit min/max quantiser).
-hipError_t launch_compll_encode(const Launch& L, int bitwidth, float* partial, hipStream_t st);
+hipError_t launch_compll_encode(const Launch& L, int bitwidth, float* partial, bool draw, unsigned key, hipStream_t st);
 hipError_t launch_compll_decode(const Launch& L, hipStream_t st);
 
 // Dense decode-and-merge; alg is a hipress_alg value (onebit, tbq, terngrad).

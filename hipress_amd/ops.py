@@ -29,6 +29,7 @@ __all__ = [
     "sparse_payload_bytes", "dgc_payload_bytes", "graddrop_payload_bytes",
     "onebit_encode", "onebit_decode", "onebit_encode_deferred", "onebit_residual", "tbq_encode", "tbq_decode", "terngrad_encode", "terngrad_decode",
     "dgc_encode", "dgc_decode", "graddrop_encode", "graddrop_decode",
+    "terngrad_encode_seeded", "uniform_fill", "compll_terngrad_encode_seeded",
     "compll_payload_bytes", "compll_decoded_count", "compll_terngrad_encode", "compll_terngrad_decode",
     "onebit_decode_merge", "tbq_decode_merge", "terngrad_decode_merge", "dgc_decode_merge",
     "graddrop_decode_merge", "Batch", "MergeBatch", "PlannedSet", "PlannedMerge", "ALIASES",
@@ -211,6 +212,32 @@ def terngrad_encode(gradient, uniform, compressed, bucket=512):
                                                  compressed.numel(), int(bucket), _stream(gradient)), "terngrad_encode")
 
 
+def _seed(seed):
+    """A caller's seed as the C ABI takes it (64 bits); None draws one from torch's CPU
+    generator, so that torch.manual_seed makes a run repeatable and every call differs."""
+    if seed is None:
+        return int(torch.randint(0, 2 ** 62, (1,)).item())
+    return int(seed) & 0xFFFFFFFFFFFFFFFF
+
+
+def terngrad_encode_seeded(gradient, compressed, bucket=512, seed=None):
+    """terngrad_encode with the noise drawn inside the kernel from `seed` (a new one every
+    step; None takes one from torch's CPU generator): no noise tensor is made, kept or read.
+    The payload equals that of terngrad_encode with uniform_fill(seed)'s values."""
+    _f32(gradient, "gradient"); _u8(compressed, "compressed", gradient)
+    with _on(gradient.device):
+        check(_lib.lib().hipress_terngrad_encode_seeded(_p(gradient), gradient.numel(), _p(compressed), compressed.numel(),
+                                                        int(bucket), _seed(seed), _stream(gradient)), "terngrad_encode_seeded")
+
+
+def uniform_fill(out, seed, tensor=0):
+    """out[i] = the noise a seeded encoder draws for element i of tensor number `tensor` of its
+    launch (0 for a per-tensor call, the place in the table for a Batch)."""
+    _f32(out, "out")
+    with _on(out.device):
+        check(_lib.lib().hipress_uniform_fill(_p(out), out.numel(), _seed(seed), int(tensor), _stream(out)), "uniform_fill")
+
+
 def terngrad_decode(compressed, gradient):
     _u8(compressed, "compressed"); _f32(gradient, "gradient", compressed)
     with _on(gradient.device):
@@ -241,6 +268,18 @@ def compll_terngrad_encode(gradient, uniform, compressed, bitwidth=2):
         ws = _workspace(gradient, size(L.hipress_compll_workspace_bytes(n), "compll_workspace_bytes"))
         check(L.hipress_compll_encode(_p(gradient), _p(uniform), n, _p(compressed), compressed.numel(), int(bitwidth),
                                       _p(ws), ws.numel(), _stream(gradient)), "compll_encode")
+
+
+def compll_terngrad_encode_seeded(gradient, compressed, bitwidth=2, seed=None):
+    """compll_terngrad_encode with the noise drawn inside the kernel from `seed`, as the
+    reference's operator draws its own: the signature the reference registers, plus the seed."""
+    _f32(gradient, "gradient"); _u8(compressed, "compressed", gradient)
+    L = _lib.lib()
+    n = gradient.numel()
+    with _on(gradient.device):
+        ws = _workspace(gradient, size(L.hipress_compll_workspace_bytes(n), "compll_workspace_bytes"))
+        check(L.hipress_compll_encode_seeded(_p(gradient), n, _p(compressed), compressed.numel(), int(bitwidth), _seed(seed),
+                                             _p(ws), ws.numel(), _stream(gradient)), "compll_encode_seeded")
 
 
 def compll_terngrad_decode(compressed, gradient):
@@ -293,18 +332,19 @@ graddrop_decode = dgc_decode
 
 
 # ---------------------------------------------------------------- the reference's own operator names
-def TernGradEncode(gradient, compressed, bitwidth=2, uniform=None):
+def TernGradEncode(gradient, compressed, bitwidth=2, uniform=None, seed=None):
     """The operator the reference registers under this name
     (/root/reference/src/CompLL/GCGen/output/TernGradEncode/TernGradEncode.cc:10-24):
     arguments (gradient, compressed, bitwidth), the min/max `bitwidth`-bit stochastic
     quantiser with the 10-byte [bitwidth][tail][min][max] header.  The reference draws its
     rounding noise inside the operator from a clock-seeded generator
-    (TernGradEncode_body.h:49,119); here `uniform` supplies it, and when it is left out one
-    U[0,1) draw per element is taken from torch's generator for the gradient's device."""
+    (TernGradEncode_body.h:49,119); here `uniform` supplies it, and when it is left out the
+    kernel draws it itself from `seed` (None: a seed from torch's CPU generator, a new one
+    every call)."""
     if uniform is None:
-        _f32(gradient, "gradient")
-        uniform = torch.rand_like(gradient)
-    compll_terngrad_encode(gradient, uniform, compressed, bitwidth)
+        compll_terngrad_encode_seeded(gradient, compressed, bitwidth, seed)
+    else:
+        compll_terngrad_encode(gradient, uniform, compressed, bitwidth)
 
 
 def TernGradDecode(compressed, gradient):
@@ -411,6 +451,8 @@ class Batch:
     gradient, residual (onebit, tbq), momentum + accumulator (dgc), accumulator
     (graddrop), uniform (terngrad), compressed, and ``out`` for decode.  The
     tensors must stay alive and keep their addresses for the life of the batch.
+    A terngrad batch none of whose tensors has ``uniform`` draws its noise in the
+    kernel: ``encode(seed=...)``.
     """
 
     def __init__(self, alg, tensors, threshold=0.0, bucket=512, momentum_factor=0.9, ratio=0.001):
@@ -445,10 +487,18 @@ class Batch:
         with _on(dev):
             check(_lib.lib().hipress_batch_create(ctypes.byref(h), alg_id, arr, len(tensors), ctypes.byref(pr)), "batch_create")
         self._h = h
+        self.seeded = alg == "terngrad" and any(t.get("gradient") is not None for t in tensors) and \
+            all(t.get("uniform") is None for t in tensors)
 
-    def encode(self):
+    def encode(self, seed=None):
+        """``seed``: for a terngrad batch without noise tensors (None: one from torch's CPU
+        generator); tensor k of the table draws with tensor = k."""
         with _on(self.device):
-            check(_lib.lib().hipress_batch_encode(self._h, _device_stream(self.device)), "batch_encode")
+            if self.seeded:
+                check(_lib.lib().hipress_batch_encode_seeded(self._h, _seed(seed), _device_stream(self.device)),
+                      "batch_encode_seeded")
+            else:
+                check(_lib.lib().hipress_batch_encode(self._h, _device_stream(self.device)), "batch_encode")
 
     def encode_phase(self, phase):
         """One launch of the encode sequence (measurement aid)."""
@@ -560,7 +610,8 @@ class PlannedSet:
     name: ``state[name]`` (dict of whole-gradient tensors: residual / momentum,
     accumulator / state, scale_state per partition), ``compressed[name]`` (one uint8
     payload per partition), ``out[name]`` (the decoded gradient, whole).  TernGrad reads
-    its rounding noise from ``uniform[name]``, one float32 tensor per compressed gradient.
+    its rounding noise from ``uniform[name]``, one float32 tensor per compressed gradient,
+    or, with ``uniform=None``, draws it in the kernel: ``encode(seed=...)``.
     """
 
     def __init__(self, alg, plan, gradients, uniform=None, threshold=0.0, bucket=512, momentum_factor=0.9,
@@ -597,8 +648,8 @@ class PlannedSet:
             if alg == "onebit_deferred":
                 st["scale_state"] = torch.zeros(max(len(bounds), 1), device=g.device)
             u = None
-            if alg == "terngrad":
-                if uniform is None or name not in uniform:
+            if alg == "terngrad" and uniform is not None:
+                if name not in uniform:
                     raise KeyError(f"terngrad needs uniform[{name!r}]")
                 u = _f32(uniform[name], "uniform", g).view(-1)
                 _same_numel(u, flat, "uniform", name)
@@ -620,9 +671,9 @@ class PlannedSet:
         self._batch = Batch(alg, tensors, threshold=threshold, bucket=bucket, momentum_factor=momentum_factor,
                             ratio=ratio) if tensors else None
 
-    def encode(self):
+    def encode(self, seed=None):
         if self._batch is not None:
-            self._batch.encode()
+            self._batch.encode(seed)
 
     def decode(self):
         if self._batch is not None:
@@ -730,6 +781,8 @@ _SCHEMAS = {
     "tbq_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
     "terngrad_encode": "(Tensor gradient, Tensor uniform, Tensor(a!) compressed, int bucket=512) -> ()",
     "terngrad_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
+    "terngrad_encode_seeded": "(Tensor gradient, Tensor(a!) compressed, int bucket=512, int? seed=None) -> ()",
+    "uniform_fill": "(Tensor(a!) out, int seed, int tensor=0) -> ()",
     "dgc_encode": "(Tensor gradient, Tensor(a!) momentum, Tensor(b!) accumulator, Tensor(c!) compressed, "
                   "float momentum_factor=0.9, float ratio=0.001) -> ()",
     "dgc_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
@@ -737,7 +790,8 @@ _SCHEMAS = {
     "graddrop_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
     "compll_terngrad_encode": "(Tensor gradient, Tensor uniform, Tensor(a!) compressed, int bitwidth=2) -> ()",
     "compll_terngrad_decode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
-    "TernGradEncode": "(Tensor gradient, Tensor(a!) compressed, int bitwidth=2, Tensor? uniform=None) -> ()",
+    "compll_terngrad_encode_seeded": "(Tensor gradient, Tensor(a!) compressed, int bitwidth=2, int? seed=None) -> ()",
+    "TernGradEncode": "(Tensor gradient, Tensor(a!) compressed, int bitwidth=2, Tensor? uniform=None, int? seed=None) -> ()",
     "TernGradDecode": "(Tensor compressed, Tensor(a!) gradient) -> ()",
     "onebit_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate, Tensor? local=None) -> ()",
     "terngrad_decode_merge": "(Tensor[] compressed, Tensor(a!) aggregate, Tensor? local=None) -> ()",

@@ -152,6 +152,22 @@ int hipress_terngrad_encode(const float *grad, const float *uniform, int64_t n, 
                             int64_t payload_bytes, int32_t bucket, void *stream);
 int hipress_terngrad_decode(const void *payload, int64_t payload_bytes, float *out, int64_t n,
                             void *stream);
+/* The same encoder with the noise drawn inside the kernel, as the body this replaces draws
+ * its own (TernGradEncode_body.h:49,119: a generator per output byte, seeded from the
+ * clock): no noise tensor to fill, keep and read, 4 of the encoder's 8.26 bytes per element
+ * less.  Where the reference's seed is the time of the call, here the caller passes it, so
+ * that a call can be repeated: element i takes
+ *     u_i = (mix32(i ^ tensor_key(uniform_key(seed), tensor)) >> 8) * 2^-24,
+ * a counter-based draw on the 24-bit grid in [0, 1) (hipress_amd/csrc/uniform_draw.h states
+ * the three functions; tensor = 0 here, the tensor's place in the table for a batch), and
+ * the payload equals, byte for byte, that of hipress_terngrad_encode with those values as
+ * its noise tensor.  hipress_uniform_fill writes them out (for a check, or for a peer that
+ * needs the tensor).  Use a new seed every step.  A call captured in a HIP graph replays
+ * the seed it was captured with. */
+int hipress_terngrad_encode_seeded(const float *grad, int64_t n, void *payload,
+                                   int64_t payload_bytes, int32_t bucket, uint64_t seed,
+                                   void *stream);
+int hipress_uniform_fill(float *out, int64_t n, uint64_t seed, uint32_t tensor, void *stream);
 
 /* ---- the in-tree CompLL operator, in its own wire format ---------------------- */
 /* Replaces TernGradEncode_body / TernGradDecode_body as generated in the tree
@@ -174,6 +190,14 @@ int64_t hipress_compll_workspace_bytes(int64_t n);
 int hipress_compll_encode(const float *grad, const float *uniform, int64_t n, void *compressed,
                           int64_t compressed_bytes, int32_t bitwidth, void *workspace,
                           int64_t workspace_bytes, void *stream);
+/* The encoder with the signature of the body it replaces, (gradient, size, compressed, size,
+ * bitwidth, ..., stream), plus the seed that the reference takes from the clock
+ * (TernGradEncode_body.h:119): the noise is drawn in the kernel as described at
+ * hipress_terngrad_encode_seeded (tensor = 0), and the result equals hipress_compll_encode
+ * with hipress_uniform_fill's values as its noise tensor. */
+int hipress_compll_encode_seeded(const float *grad, int64_t n, void *compressed,
+                                 int64_t compressed_bytes, int32_t bitwidth, uint64_t seed,
+                                 void *workspace, int64_t workspace_bytes, void *stream);
 int hipress_compll_decode(const void *compressed, int64_t compressed_bytes, float *out, int64_t n,
                           void *stream);
 
@@ -286,6 +310,12 @@ typedef struct hipress_batch hipress_batch;
 int hipress_batch_create(hipress_batch **out, int32_t alg, const hipress_tensor *tensors,
                          int32_t count, const hipress_params *params);
 int hipress_batch_encode(hipress_batch *batch, void *stream);
+/* For a terngrad batch none of whose tensors names a noise tensor (`uniform` NULL in all of
+ * them; a batch with some and not others is refused): the noise is drawn in the kernel from
+ * this seed, tensor k of the table with tensor = k (hipress_terngrad_encode_seeded).
+ * hipress_batch_encode refuses such a batch, and this call any other
+ * (HIPRESS_ERR_PARAM). */
+int hipress_batch_encode_seeded(hipress_batch *batch, uint64_t seed, void *stream);
 int hipress_batch_decode(hipress_batch *batch, void *stream);
 /* Measurement aid: enqueues only launch number `phase` of the encode sequence, so
  * that a caller can bracket one kernel with events.  onebit: 0 magnitude sum,

@@ -89,6 +89,8 @@ _SIG = {
     "hpo_compll_payload_bytes": (_i64, [_i64, ctypes.c_int]),
     "hpo_compll_encode": (_i64, [_ptr, _ptr, _i64, _ptr, ctypes.c_int]),
     "hpo_lcg_uniform": (None, [ctypes.c_uint32, _f32, _f32, _ptr, _i64]),
+    "hpo_uniform_tensor_key": (ctypes.c_uint32, [ctypes.c_uint64, ctypes.c_uint32]),
+    "hpo_uniform_draws": (None, [ctypes.c_uint64, ctypes.c_uint32, _ptr, _i64]),
 }
 
 
@@ -343,3 +345,15 @@ def lcg_uniform(seed, n, lo=0.0, hi=1.0):
     out = np.empty(n, dtype=np.float32)
     lib().hpo_lcg_uniform(seed, lo, hi, _p(out), n)
     return out
+
+
+def uniform_draws(seed, n, tensor=0):
+    """The noise an encoder called with `seed` draws for the n elements of tensor `tensor`
+    of its launch (0 for a per-tensor call)."""
+    out = np.empty(n, dtype=np.float32)
+    lib().hpo_uniform_draws(seed, tensor, _p(out), n)
+    return out
+
+
+def uniform_tensor_key(seed, tensor=0):
+    return int(lib().hpo_uniform_tensor_key(seed, tensor))

@@ -673,6 +673,47 @@ void hpo_lcg_uniform(uint32_t seed, float lo, float hi, float *out, int64_t n)
     }
 }
 
+/* The noise the encoders draw themselves when they are called with a seed instead of a
+ * noise tensor (include/hipress_amd.h, hipress_terngrad_encode_seeded).  A definition of
+ * this library's own, with no counterpart in the reference, whose generator is seeded from
+ * the clock (TernGradEncode_body.h:119): element i of tensor t takes the top 24 bits of
+ * h(i xor k) as a fraction, h being the 32-bit mixer "triple32" (xor-shift 17, times
+ * 0xed5ad4bb, xor-shift 11, times 0xac4c1b51, xor-shift 15, times 0x31848bab, xor-shift 14)
+ * and k = h(fold(seed) +
+ * t * 0x9e3779b9), where fold xors the two halves of the SplitMix64 output function
+ * applied to seed + 0x9e3779b97f4a7c15.  Pinned by tests/test_uniform_draw.py: the
+ * published first SplitMix64 output, an independent big-integer restatement, and the
+ * header the kernels compile, built for the host. */
+static uint32_t hpo_triple32(uint32_t x)
+{
+    x = x ^ (x >> 17);
+    x = x * 0xed5ad4bbU;
+    x = x ^ (x >> 11);
+    x = x * 0xac4c1b51U;
+    x = x ^ (x >> 15);
+    x = x * 0x31848babU;
+    x = x ^ (x >> 14);
+    return x;
+}
+
+uint32_t hpo_uniform_tensor_key(uint64_t seed, uint32_t tensor)
+{
+    uint64_t z = seed + 0x9e3779b97f4a7c15ULL;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ULL;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebULL;
+    z = z ^ (z >> 31);
+    uint32_t folded = (uint32_t)(z & 0xffffffffULL) ^ (uint32_t)(z >> 32);
+    return hpo_triple32(folded + tensor * 0x9e3779b9U);
+}
+
+void hpo_uniform_draws(uint64_t seed, uint32_t tensor, float *out, int64_t n)
+{
+    const uint32_t k = hpo_uniform_tensor_key(seed, tensor);
+    HPO_PARALLEL_FOR
+    for (int64_t i = 0; i < n; ++i)
+        out[i] = (float)(hpo_triple32((uint32_t)i ^ k) >> 8) / 16777216.0f;
+}
+
 /* Threads the all-cores build runs its parallel loops on (1 for the plain build). */
 #ifdef HPO_OMP
 #include <omp.h>

@@ -82,6 +82,13 @@ def test_null_and_range_checks_need_no_gpu(lib):
     assert L.hipress_tbq_encode(None, None, -1, None, 100, 0.05, None) == -2
     assert L.hipress_tbq_decode(None, 100, None, 10, None) == -1
     assert L.hipress_batch_encode(None, None) == -1
+    assert L.hipress_batch_encode_seeded(None, 1, None) == -1
+    assert L.hipress_terngrad_encode_seeded(None, 10, None, 100, 512, 1, None) == -1
+    assert L.hipress_terngrad_encode_seeded(None, -1, None, 100, 512, 1, None) == -2
+    assert L.hipress_uniform_fill(None, 10, 1, 0, None) == -1
+    assert L.hipress_uniform_fill(None, -1, 1, 0, None) == -2
+    assert L.hipress_compll_encode_seeded(None, 10, None, 100, 2, 1, None, 0, None) == -1
+    assert L.hipress_compll_encode_seeded(None, 10, None, 100, 3, 1, None, 0, None) == -4
     assert L.hipress_merge_batch_run(None, None) == -1
     # a merge without the re-encode needs its aggregate
     import ctypes
