@@ -184,6 +184,12 @@ __device__ __forceinline__ f4 noise4(const float* u, long long e, long long n, u
         v.y = uniform_at(i + 1u, key);
         v.z = uniform_at(i + 2u, key);
         v.w = uniform_at(i + 3u, key);
+        if (!FAST) {  // places beyond the tensor draw 0, as they read 0 from a noise tensor
+            if (e + 3 >= n) v.w = 0.f;
+            if (e + 2 >= n) v.z = 0.f;
+            if (e + 1 >= n) v.y = 0.f;
+            if (e >= n) v.x = 0.f;
+        }
         return v;
     }
     return load4<FAST>(u, e, n);

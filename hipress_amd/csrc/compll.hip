@@ -130,7 +130,7 @@ __global__ __launch_bounds__(kBlock) void compll_quant_kernel(Src src, unsigned 
     for (int j = 0; j < 4; ++j) {
         long long e = base + j * 256 + lane * 4;
         g[j] = fast ? ld4(s.g + e) : ld4_guard(s.g, e, n);
-        u[j] = DRAW ? noise4<true, true>(nullptr, e, n, tkey) : (fast ? ld4(s.u + e) : ld4_guard(s.u, e, n));
+        u[j] = DRAW ? noise4<true, true>(nullptr, e, n, tkey) : (fast ? ld4(s.u + e) : ld4_guard(s.u, e, n));  // codes beyond n are masked below
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
