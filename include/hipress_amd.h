@@ -313,8 +313,8 @@ int hipress_batch_encode(hipress_batch *batch, void *stream);
 /* For a terngrad batch none of whose tensors names a noise tensor (`uniform` NULL in all of
  * them; a batch with some and not others is refused): the noise is drawn in the kernel from
  * this seed, tensor k of the table with tensor = k (hipress_terngrad_encode_seeded).
- * hipress_batch_encode refuses such a batch, and this call any other
- * (HIPRESS_ERR_PARAM). */
+ * hipress_batch_encode and hipress_batch_encode_phase refuse such a batch, and this
+ * call any other (HIPRESS_ERR_PARAM). */
 int hipress_batch_encode_seeded(hipress_batch *batch, uint64_t seed, void *stream);
 int hipress_batch_decode(hipress_batch *batch, void *stream);
 /* Measurement aid: enqueues only launch number `phase` of the encode sequence, so
