@@ -284,3 +284,35 @@ def test_views_buckets_and_dense_merges_random_cases(hp):
         np.testing.assert_array_equal(host(agg), want_agg, err_msg="sparse merge " + where)
         check_sparse(host(outp), want_out, "sparse merge payload " + where)
         np.testing.assert_array_equal(host(acc), want_acc, err_msg="sparse merge accumulator " + where)
+
+
+def test_seeded_quantisers_random_cases(hp):
+    """The encoders that draw their own noise, at random sizes, bucket sizes, bit widths, seeds
+    and view offsets, per tensor and as a table: equal to the oracle run on oracle.uniform_draws."""
+    rng = seeded(2029)
+    for case, n in enumerate(sizes(rng, 60, top=700_000)):
+        bucket = int(rng.choice([int(rng.integers(1, 6000)), 256, 512, 1024, 4096, int(rng.integers(6000, 200000))]))
+        seed, off, b = int(rng.integers(0, 2 ** 63)), int(rng.integers(0, 4)), int(rng.choice([1, 2, 4, 8]))
+        where = f"case {case}: n={n} bucket={bucket} seed={seed} offset={off} b={b}"
+        g = rng.normal(0, 1e-3, n).astype(F)
+        t = torch.empty(n + off, device="cuda")
+        gv = t[off:]
+        gv.copy_(torch.from_numpy(g))
+        u = oracle.uniform_draws(seed, n)
+        pay = payload(hp.terngrad_payload_bytes(n, bucket))
+        hp.terngrad_encode_seeded(gv, pay, bucket, seed)
+        np.testing.assert_array_equal(host(pay), oracle.terngrad_encode(g, u, bucket), err_msg="terngrad " + where)
+        pay = payload(hp.compll_payload_bytes(n, b))
+        hp.compll_terngrad_encode_seeded(gv, pay, b, seed)
+        np.testing.assert_array_equal(host(pay), oracle.compll_encode(g, u, b), err_msg="min/max quantiser " + where)
+    for table in range(6):
+        ns = sizes(rng, int(rng.integers(2, 25)), top=400_000)
+        bucket, seed = int(rng.choice([512, 100, 777, 5000])), int(rng.integers(0, 2 ** 63))
+        gs = [rng.normal(0, 1e-3, n).astype(F) for n in ns]
+        ts = [{"gradient": dev(g), "compressed": payload(hp.terngrad_payload_bytes(g.size, bucket))} for g in gs]
+        bt = hp.Batch("terngrad", ts, bucket=bucket)
+        bt.encode(seed=seed)
+        for k, (tt, g) in enumerate(zip(ts, gs)):
+            want = oracle.terngrad_encode(g, oracle.uniform_draws(seed, g.size, k), bucket)
+            np.testing.assert_array_equal(host(tt["compressed"]), want, err_msg=f"table {table} tensor {k} n={g.size} bucket={bucket}")
+        bt.close()
