@@ -13,7 +13,8 @@ primitive kernels of hipress_amd/csrc/compll_prims.h:
   device-known ones are evaluated by a one-thread kernel and stay in `Dev`;
 * neighbouring `reduce` statements over the same vector share one sweep;
 * a packed vector that only feeds `concat` is produced in place behind the header;
-* `random<float>(lo, hi)` reads an explicit uniform[0,1) input tensor.
+* `random<float>(lo, hi)` reads an explicit uniform[0,1) input tensor, or, when the caller passes
+  NULL for it, is drawn in the kernel from the caller's seed and the element's index.
 
 The emitted entry point mirrors the reference's body signature (vectors in the
 order of declaration, each followed by its length, then the scalar parameters),
@@ -259,7 +260,7 @@ class FunctionGen:
             self.needs_uniform = True
             if self.streams is not None:
                 return Value(f"cl::uniform_from(s[{self._stream('a.uniform')}], (float)({lo.code}), (float)({hi.code}))", "float", "dev")
-            return Value(f"cl::uniform_draw(a.uniform, {_local(index_name)}, (float)({lo.code}), (float)({hi.code}))", "float", "dev")
+            return Value(f"cl::uniform_draw(a.uniform, a.ukey, {_local(index_name)}, (float)({lo.code}), (float)({hi.code}))", "float", "dev")
         if isinstance(e, F.Call):
             args = [self.expr(x, scope, index_name) for x in e.args]
             cls = "dev" if any(x.cls == "dev" for x in args) else "host"
@@ -727,7 +728,7 @@ class FunctionGen:
                 sig.append((_SCALAR_C[p.type.base], p.name))
                 man.append({"name": p.name, "kind": p.type.base})
         if self.needs_uniform:
-            sig.append(("const float*", "uniform"))
+            sig += [("const float*", "uniform"), ("uint64_t", "seed")]
         sig += [("void*", "workspace"), ("int64_t", "workspace_bytes"), ("void*", "stream")]
         return sig, man
 
@@ -743,6 +744,7 @@ class FunctionGen:
             if s.cls == "host":
                 o.append(f"    {s.ctype} v_{s.name};")
         o.append("    const float* uniform;")
+        o.append("    unsigned ukey;")
         o.append("};")
         o.append("struct Dev {")
         dev = [s for s in self.scalars.values() if s.cls == "dev"]
@@ -878,7 +880,7 @@ class FunctionGen:
         o.append("}")
         o.append("")
         o.append(f"// {name}: vectors with their lengths in elements, then the scalar parameters" +
-                 (", then `uniform`: one uniform[0,1) float per element of the longest mapped range" if self.needs_uniform else "") +
+                 (", then `uniform`: one uniform[0,1) float per element of the longest mapped range, or NULL: the values are then drawn in the kernels from `seed`" if self.needs_uniform else "") +
                  f"; workspace of at least {name}_workspace_bytes(longest float vector) bytes, 16-byte aligned;")
         o.append("// returns 0, -1 null pointer, -2 a buffer too small, -3 misaligned workspace, -4 bad parameter, -5 HIP error, -6 workspace.")
         o.append(f'extern "C" int {name}({", ".join(t + " " + n for t, n in sig)}) {{')
@@ -894,11 +896,11 @@ class FunctionGen:
             if s.is_param:
                 o.append(f"    a.v_{s.name} = {s.name};")
         if self.needs_uniform:
-            some = " || ".join(f"{v.name}_size > 0" for v in self.vectors.values() if v.is_param and v.elem == "float") or "true"
-            o.append(f"    if (!uniform && ({some})) return -1;")
             o.append("    a.uniform = uniform;")
+            o.append("    a.ukey = hp::tensor_key(hp::uniform_key(seed), 0u);")
         else:
             o.append("    a.uniform = nullptr;")
+            o.append("    a.ukey = 0u;")
         o += ["    " + ln for ln in self.host_lines]
         o += ["    " + ln for ln in self.checks]
         biggest = " , ".join(f"(long long){v.size}" for v in self.reduced) or "0ll"

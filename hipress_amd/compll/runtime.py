@@ -3,7 +3,8 @@ on torch tensors: in-place operators over caller-allocated buffers, vectors firs
 the order the operator declares them, then its scalars, as the reference's generated
 operators are called (`TernGradEncode(gradient, compressed, bitwidth=b)`,
 /root/reference/src/CompLL/GCGen/output/TernGradEncode/TernGradEncode.cc:10-24).
-An operator that draws random numbers takes the uniform[0,1) tensor as `uniform=`.
+An operator that draws random numbers takes the uniform[0,1) tensor as `uniform=`, or,
+without one, draws in its kernels from `seed=` (left out: a seed from torch's CPU generator).
 There is no CPU path: loading fails loudly if the generated library was not built.
 """
 import ctypes
@@ -51,7 +52,7 @@ class Operators:
                     argtypes += [ctypes.c_void_p, ctypes.c_int32]
             argtypes += [_C[p["kind"]] for p in m["params"] if not p["kind"].endswith("*")]
             if m["uniform"]:
-                argtypes.append(ctypes.c_void_p)
+                argtypes += [ctypes.c_void_p, ctypes.c_uint64]
             argtypes += [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
             fn.argtypes, fn.restype = argtypes, ctypes.c_int
             ws = getattr(self._lib, name + "_workspace_bytes")
@@ -65,7 +66,7 @@ class Operators:
         vectors = [p for p in m["params"] if p["kind"].endswith("*")]
         scalars = [p for p in m["params"] if not p["kind"].endswith("*")]
 
-        def call(*args, uniform=None, **kw):
+        def call(*args, uniform=None, seed=None, **kw):
             if len(args) > len(vectors) + len(scalars):
                 raise TypeError(f"{name} takes {len(vectors) + len(scalars)} positional arguments")
             values = dict(zip([p["name"] for p in vectors + scalars], args))
@@ -92,12 +93,17 @@ class Operators:
                     floats = max(floats, t.numel())
                 cargs += [t.data_ptr(), t.numel()]
             cargs += [values[p["name"]] for p in scalars]
-            if m["uniform"]:
+            if m["uniform"] and uniform is None:
+                # no noise tensor: the kernels draw from a seed (the caller's, or one from torch's CPU generator)
+                if seed is None:
+                    seed = int(torch.randint(0, 2 ** 62, (1,)).item())
+                cargs += [None, int(seed) & 0xFFFFFFFFFFFFFFFF]
+            elif m["uniform"]:
                 if not isinstance(uniform, torch.Tensor) or uniform.dtype != torch.float32 or not uniform.is_cuda or not uniform.is_contiguous():
                     raise TypeError(f"{name}: uniform= must be a contiguous float32 tensor on the GPU")
                 if uniform.numel() < floats:
                     raise ValueError(f"{name}: uniform= is shorter than the float vectors")
-                cargs.append(uniform.data_ptr())
+                cargs += [uniform.data_ptr(), 0]
             need = ws_bytes(biggest)
             stream = _raw_stream(device.index) if _raw_stream is not None else torch.cuda.current_stream(device).cuda_stream
             key = (device, stream, name)  # scratch is per stream: calls on one stream are ordered, others are not

@@ -19,6 +19,8 @@
 
 #include <type_traits>
 
+#include "uniform_draw.h"
+
 namespace cl {
 
 typedef float f4 __attribute__((ext_vector_type(4)));
@@ -74,10 +76,12 @@ __device__ __forceinline__ T get(const uint8_t* p) {
 
 // ---- rounding noise -------------------------------------------------------------------
 // random<float>(lo, hi) of the language reads an explicit uniform[0,1) tensor at
-// the element being mapped, so that an operator is a function of its inputs.
+// the element being mapped, so that an operator is a function of its inputs; without such
+// a tensor (NULL) the value is drawn from the call's key and the element's index
+// (uniform_draw.h), which the caller's seed fixes: still a function of the inputs.
 __device__ __forceinline__ float uniform_from(float u, float lo, float hi) { return lo + (hi - lo) * u; }
-__device__ __forceinline__ float uniform_draw(const float* u, long long i, float lo, float hi) {
-    return uniform_from(u[i], lo, hi);
+__device__ __forceinline__ float uniform_draw(const float* u, unsigned key, long long i, float lo, float hi) {
+    return uniform_from(u ? u[i] : hp::uniform_at((uint32_t)i, key), lo, hi);
 }
 
 struct Nothing {
@@ -96,8 +100,10 @@ __global__ void serial_kernel(Args a, Dev* d) {
 // ---- streamed operands ---------------------------------------------------------------------
 // A lane owns four consecutive indices of each of four rows of 256 of its
 // wavefront's 1024.  Fn::stream(a, k), k < Fn::NS, are the float vectors a lambda
+// reads at its own index; they are loaded as 16-byte vectors, whole rows per wavefront.  A
+// stream without a vector (NULL: the noise of random<float> when the caller passed a seed and
+// no noise tensor) is drawn instead, element i taking hp::uniform_at(i, a.ukey).
 // KEEP: plain loads, which leave their lines on the chip for the sweep that follows; the others are
-// KEEP: plain loads, which leave their lines in L2 for the sweep that follows; the others are
 // streamed.  (The empty statement keeps the compiler from folding the two otherwise identical
 // branches into one, which would drop the streaming hint from both.)
 template <class Args, class Fn, bool KEEP>
@@ -109,7 +115,13 @@ __device__ __forceinline__ void load_streams_as(const Args& a, long long base, l
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const long long e = base + j * 256;
-            if (e + 3 < count && vec_ok) {
+            if (p == nullptr) {  // the same for every lane of the launch
+                const uint32_t i = (uint32_t)e;
+                x[k][j].x = e < count ? hp::uniform_at(i, a.ukey) : 0.f;
+                x[k][j].y = e + 1 < count ? hp::uniform_at(i + 1u, a.ukey) : 0.f;
+                x[k][j].z = e + 2 < count ? hp::uniform_at(i + 2u, a.ukey) : 0.f;
+                x[k][j].w = e + 3 < count ? hp::uniform_at(i + 3u, a.ukey) : 0.f;
+            } else if (e + 3 < count && vec_ok) {
                 if (KEEP) {
                     asm volatile("");
                     x[k][j] = *reinterpret_cast<const f4u*>(p + e);

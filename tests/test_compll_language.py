@@ -67,7 +67,7 @@ def test_plan_classifies_scalars_and_fuses_reductions():
     assert len(g.stages[0].folds) == 2 and g.needs_uniform
     src, man = compll.compile_text(PROGRAM)
     assert 'extern "C" int Enc(float* g, int32_t g_size, uint8_t* out, int32_t out_size, uint8_t b, const float* uniform, ' \
-           "void* workspace, int64_t workspace_bytes, void* stream)" in src
+           "uint64_t seed, void* workspace, int64_t workspace_bytes, void* stream)" in src  # uniform NULL: drawn from seed
     assert "cl::put<float>(a.v_out + 2, (float)d.v_bottom);" in src  # header offsets 0, 1, 2, 6; codes behind byte 10
     assert "(a.v_out + 10)" in src
     assert man[0]["params"] == [{"name": "g", "kind": "float*"}, {"name": "out", "kind": "uint8*"}, {"name": "b", "kind": "uint8"}]

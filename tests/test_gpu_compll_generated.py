@@ -50,6 +50,13 @@ def test_minmax_quant_matches_the_oracle(ops, n, b):
     pay2 = torch.zeros(hp.compll_payload_bytes(n, b), dtype=torch.uint8, device="cuda")
     hp.compll_terngrad_encode(dev(g), dev(u), pay2, b)
     np.testing.assert_array_equal(host(pay2), want)
+    # without a noise tensor both draw the same values from the same seed
+    seed = 31 * n + b
+    ops.MinMaxQuantEncode(dev(g), pay2, b, seed=seed)
+    np.testing.assert_array_equal(host(pay2), oracle.compll_encode(g, oracle.uniform_draws(seed, n), b))
+    pay3 = torch.zeros_like(pay2)
+    hp.compll_terngrad_encode_seeded(dev(g), pay3, b, seed)
+    np.testing.assert_array_equal(host(pay3), host(pay2))
     # decode: as many elements as the payload says, bounded by the output
     ref = oracle.compll_decode(want, n + 8)
     out = torch.full((n + 8,), 7.0, device="cuda")
@@ -184,7 +191,8 @@ def test_generated_ops_report_errors(ops):
     with pytest.raises(GeneratedOpError, match="bad parameter"):
         ops.MinMaxQuantEncode(g, torch.zeros(200, dtype=torch.uint8, device="cuda"), 3, uniform=u)
     with pytest.raises(TypeError):
-        ops.MinMaxQuantEncode(g, torch.zeros(200, dtype=torch.uint8, device="cuda"), 2)  # no uniform tensor
+        ops.MinMaxQuantEncode(g, torch.zeros(200, dtype=torch.uint8, device="cuda"), 2, uniform=u.cpu())  # noise not on the GPU
+    ops.MinMaxQuantEncode(g, torch.zeros(200, dtype=torch.uint8, device="cuda"), 2)  # no noise tensor: drawn in the kernel
     with pytest.raises(TypeError):
         ops.MinMaxQuantEncode(g.double(), torch.zeros(200, dtype=torch.uint8, device="cuda"), 2, uniform=u)
     # a payload whose header names an impossible width decodes to nothing
@@ -232,3 +240,8 @@ def test_the_reference_s_own_programs_match_the_oracle(reference_ops, n, b):
     assert dec.size == k
     np.testing.assert_array_equal(host(out)[:k], dec)
     assert (host(out)[k:] == 7.0).all()
+    # with the reference's own argument list - no noise tensor - the kernels draw from the seed
+    seed = 1000 * n + b
+    pay.fill_(0xAB)
+    reference_ops.TernGradEncode(dev(g), pay, b, seed=seed)
+    np.testing.assert_array_equal(host(pay), oracle.compll_encode(g, oracle.uniform_draws(seed, n), b))
