@@ -809,6 +809,7 @@ class FunctionGen:
                 else:
                     streams, call = [st.vec.ptr], "s[0]"
                 o.append(f"    static constexpr int NS = {len(streams)};")
+                o.append(f"    static constexpr int UNIFORM = {streams.index('a.uniform') if 'a.uniform' in streams else -1};  // the stream that may come without a vector")
                 o.append("    static __device__ __forceinline__ const float* stream(const Args& a, int k) {")
                 for i, ptr in enumerate(streams):
                     o.append(f"        if (k == {i}) return {ptr};")
@@ -833,6 +834,7 @@ class FunctionGen:
                         if ptr not in streams:
                             streams.append(ptr)
                 o.append(f"    static constexpr int NS = {len(streams)};  // float vectors read at the index itself")
+                o.append(f"    static constexpr int UNIFORM = {streams.index('a.uniform') if 'a.uniform' in streams else -1};  // the stream that may come without a vector")
                 o.append("    static __device__ __forceinline__ const float* stream(const Args& a, int k) {")
                 for i, ptr in enumerate(streams):
                     o.append(f"        if (k == {i}) return {ptr};")

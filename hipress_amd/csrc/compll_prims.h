@@ -102,7 +102,8 @@ __global__ void serial_kernel(Args a, Dev* d) {
 // wavefront's 1024.  Fn::stream(a, k), k < Fn::NS, are the float vectors a lambda
 // reads at its own index; they are loaded as 16-byte vectors, whole rows per wavefront.  A
 // stream without a vector (NULL: the noise of random<float> when the caller passed a seed and
-// no noise tensor) is drawn instead, element i taking hp::uniform_at(i, a.ukey).
+// no noise tensor; Fn::UNIFORM names that stream, -1: none) is drawn instead, element i taking
+// hp::uniform_at(i, a.ukey).
 // KEEP: plain loads, which leave their lines on the chip for the sweep that follows; the others are
 // streamed.  (The empty statement keeps the compiler from folding the two otherwise identical
 // branches into one, which would drop the streaming hint from both.)
@@ -115,7 +116,7 @@ __device__ __forceinline__ void load_streams_as(const Args& a, long long base, l
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const long long e = base + j * 256;
-            if (p == nullptr) {  // the same for every lane of the launch
+            if (k == Fn::UNIFORM && p == nullptr) {  // the same for every lane of the launch
                 const uint32_t i = (uint32_t)e;
                 x[k][j].x = e < count ? hp::uniform_at(i, a.ukey) : 0.f;
                 x[k][j].y = e + 1 < count ? hp::uniform_at(i + 1u, a.ukey) : 0.f;
