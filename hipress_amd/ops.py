@@ -487,8 +487,10 @@ class Batch:
         with _on(dev):
             check(_lib.lib().hipress_batch_create(ctypes.byref(h), alg_id, arr, len(tensors), ctypes.byref(pr)), "batch_create")
         self._h = h
-        self.seeded = alg == "terngrad" and any(t.get("gradient") is not None for t in tensors) and \
-            all(t.get("uniform") is None for t in tensors)
+        # as the library decides it: some tensor with elements comes without a noise tensor (all of them, or the
+        # library has refused the batch)
+        self.seeded = alg == "terngrad" and any(
+            t.get("gradient") is not None and t["gradient"].numel() > 0 and t.get("uniform") is None for t in tensors)
 
     def encode(self, seed=None):
         """``seed``: for a terngrad batch without noise tensors (None: one from torch's CPU

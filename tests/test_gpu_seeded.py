@@ -144,6 +144,12 @@ def test_batches_take_a_seed_exactly_when_they_have_no_noise_tensors(hp):
     assert L.hipress_batch_encode_seeded(tb._h, 1, st) == -4
     for b in (drawn, plain, tb):
         b.close()
+    # a table of empty tensors has nothing to draw for: the plain call serves it, with or without noise tensors
+    e = torch.zeros(0, device="cuda")
+    empty = hp.Batch("terngrad", [{"gradient": e, "compressed": payload(hp.terngrad_payload_bytes(0, 512))}], bucket=512)
+    assert not empty.seeded
+    empty.encode()
+    empty.close()
 
 
 def test_planned_set_without_noise_tensors(hp):
