@@ -169,3 +169,29 @@ def test_planned_set_without_noise_tensors(hp):
         ref[off:off + length] = oracle.terngrad_decode(want, length)
     np.testing.assert_array_equal(host(ps.out["w"]), ref)
     ps.close()
+
+
+def test_seeded_terngrad_is_unbiased_over_seeds(hp):
+    """What the noise is for: averaged over many seeds the decoded value of every element
+    approaches the gradient (E[code] = g / s when u is uniform).  256 seeds, every element
+    that is kept often enough for a normal bound within 5.5 standard errors, no drift over the
+    tensor, and the spread of independent draws."""
+    n, bucket, seeds = 20000, 512, 256
+    g = np.random.default_rng(3).normal(0, 1e-3, n).astype(F)
+    gd, pay, out = dev(g), payload(hp.terngrad_payload_bytes(n, bucket)), torch.empty(n, device="cuda")
+    acc = torch.zeros(n, device="cuda", dtype=torch.float64)
+    for seed in range(seeds):
+        hp.terngrad_encode_seeded(gd, pay, bucket, seed)
+        hp.terngrad_decode(pay, out)
+        acc += out.double()
+    mean = host(acc) / seeds
+    s = np.empty(n)
+    for b0 in range(0, n, bucket):
+        s[b0:b0 + bucket] = np.abs(g[b0:b0 + bucket]).max()
+    p = np.abs(g) / s                                  # the probability that an element is kept
+    se = s * np.sqrt(p * (1 - p) / seeds) + 1e-12      # standard error of the mean of seeds draws of +-s or 0
+    z = (mean - g) / se
+    near_normal = (p * seeds >= 10) & ((1 - p) * seeds >= 10)  # elsewhere the count of kept draws is too skewed for a z bound
+    assert near_normal.sum() > n // 2 and np.abs(z[near_normal]).max() < 5.5, np.abs(z[near_normal]).max()
+    assert abs(z.mean()) < 5 / np.sqrt(n)              # no common drift
+    assert 0.9 < z.std() < 1.1                         # and the spread of independent draws
