@@ -316,3 +316,100 @@ def test_seeded_quantisers_random_cases(hp):
             want = oracle.terngrad_encode(g, oracle.uniform_draws(seed, g.size, k), bucket)
             np.testing.assert_array_equal(host(tt["compressed"]), want, err_msg=f"table {table} tensor {k} n={g.size} bucket={bucket}")
         bt.close()
+
+
+SPECIALS = np.array([np.nan, np.inf, -np.inf, 0.0, -0.0, 1e-40, -3e-42, 1.4e-45, np.finfo(F).max, -np.finfo(F).max,
+                     np.finfo(F).tiny, -np.finfo(F).tiny], F)
+
+
+def feq(got, want, msg=""):
+    """Equal as floats, NaN matching NaN, and the sign of zero respected."""
+    np.testing.assert_array_equal(got, want, err_msg=msg)
+    z = want == 0
+    np.testing.assert_array_equal(np.signbit(got[z]), np.signbit(want[z]), err_msg=msg + " (sign of zero)")
+
+
+def sprinkled(rng, n, sigma):
+    """N(0, sigma) data with special values at random places (about one in fifty, and the ends)."""
+    g = rng.normal(0, sigma, n).astype(F)
+    k = max(1, n // 50)
+    at = np.concatenate([rng.integers(0, n, k), [0, n - 1]])
+    g[at] = rng.choice(SPECIALS, at.size)
+    return g
+
+
+def test_special_values_random_cases(hp):
+    """NaN, infinities, signed zeros, denormals and FLT_MAX at random places of tensors of random
+    sizes, through the encoders that have no per-tensor sum (TBQ, TernGrad at any bucket size,
+    DGC, GradDrop), their decoders and the merges, state carried over two steps."""
+    rng = seeded(2030)
+    for case, n in enumerate(sizes(rng, 50, top=500_000)):
+        bucket = int(rng.choice([int(rng.integers(1, 6000)), 256, 512, 1024, 4096, int(rng.integers(6000, 100000))]))
+        ratio, P = float(10 ** rng.uniform(-3, -1.5)), int(rng.integers(1, 9))
+        where = f"case {case}: n={n} bucket={bucket} ratio={ratio:.3g} peers={P}"
+        r_ref, mom_ref, acc_ref, gacc_ref = sprinkled(rng, n, 0.02), np.zeros(n, F), np.zeros(n, F), np.zeros(n, F)
+        r, mom, acc, gacc = dev(r_ref), dev(mom_ref), dev(acc_ref), dev(gacc_ref)
+        out = torch.full((n,), 7.0, device="cuda")
+        for step in range(2):
+            g, u = sprinkled(rng, n, 0.02), rng.random(n, dtype=F)
+            pay = payload(hp.tbq_payload_bytes(n))
+            hp.tbq_encode(dev(g), r, pay, 0.05)
+            want, r_ref = oracle.tbq_encode(g, r_ref, 0.05)
+            np.testing.assert_array_equal(host(pay), want, err_msg="tbq " + where)
+            feq(host(r), r_ref, "tbq residual " + where)
+            hp.tbq_decode(pay, out)
+            feq(host(out), oracle.tbq_decode(want, n), "tbq decode " + where)
+            pay = payload(hp.terngrad_payload_bytes(n, bucket))
+            hp.terngrad_encode(dev(g), dev(u), pay, bucket)
+            want = oracle.terngrad_encode(g, u, bucket)
+            got, nb = host(pay), (n + bucket - 1) // bucket
+            feq(got[16:16 + 4 * nb].view(F), want[16:16 + 4 * nb].view(F), "terngrad scales " + where)
+            np.testing.assert_array_equal(got[:16], want[:16], err_msg="terngrad header " + where)
+            off = 16 + oracle.terngrad_scale_bytes(n, bucket)
+            np.testing.assert_array_equal(got[off:], want[off:], err_msg="terngrad codes " + where)
+            hp.terngrad_decode(pay, out)
+            feq(host(out), oracle.terngrad_decode(want, n), "terngrad decode " + where)
+            gs = sprinkled(rng, n, 1e-3)
+            pay = payload(hp.sparse_payload_bytes(n, ratio))
+            hp.dgc_encode(dev(gs), mom, acc, pay, 0.9, ratio)
+            want, mom_ref, acc_ref = oracle.dgc_encode(gs, mom_ref, acc_ref, 0.9, ratio)
+            gp, wp = oracle.sparse_unpack(host(pay)), oracle.sparse_unpack(want)
+            assert gp[:3] == wp[:3] and gp[3].view(np.uint32) == wp[3].view(np.uint32), ("dgc " + where, gp[:4], wp[:4])
+            np.testing.assert_array_equal(gp[4], wp[4], err_msg="dgc indices " + where)
+            feq(gp[5], wp[5], "dgc values " + where)
+            feq(host(mom), mom_ref, "dgc momentum " + where)
+            feq(host(acc), acc_ref, "dgc accumulator " + where)
+            hp.dgc_decode(pay, out)
+            feq(host(out), oracle.sparse_decode(want, n), "sparse decode " + where)
+            pay = payload(hp.sparse_payload_bytes(n, ratio))
+            hp.graddrop_encode(dev(gs), gacc, pay, ratio)
+            want, gacc_ref = oracle.graddrop_encode(gs, gacc_ref, ratio)
+            gp, wp = oracle.sparse_unpack(host(pay)), oracle.sparse_unpack(want)
+            assert gp[:3] == wp[:3] and gp[3].view(np.uint32) == wp[3].view(np.uint32), ("graddrop " + where, gp[:4], wp[:4])
+            np.testing.assert_array_equal(gp[4], wp[4], err_msg="graddrop indices " + where)
+            feq(gp[5], wp[5], "graddrop values " + where)
+            feq(host(gacc), gacc_ref, "graddrop accumulator " + where)
+        # merges of peers that carry such values
+        z = np.zeros(n, F)
+        tp = [oracle.tbq_encode(sprinkled(rng, n, 0.04), z, 0.05)[0] for _ in range(P)]
+        r0 = sprinkled(rng, n, 0.02)
+        agg, res, outp = torch.full((n,), 7.0, device="cuda"), dev(r0), payload(hp.tbq_payload_bytes(n))
+        hp.tbq_decode_merge([dev(p) for p in tp], agg, res, outp, 0.05)
+        want_agg, want_out, want_r = oracle.tbq_decode_merge(tp, n, r0, 0.05)
+        feq(host(agg), want_agg, "tbq merge " + where)
+        np.testing.assert_array_equal(host(outp), want_out, err_msg="tbq merge payload " + where)
+        feq(host(res), want_r, "tbq merge residual " + where)
+        tg = [oracle.terngrad_encode(sprinkled(rng, n, 1e-3), rng.random(n, dtype=F), bucket) for _ in range(P)]
+        hp.terngrad_decode_merge([dev(p) for p in tg], agg)
+        feq(host(agg), oracle.terngrad_decode_merge(tg, n), "terngrad merge " + where)
+        sp = [oracle.graddrop_encode(sprinkled(rng, n, 1e-3), z, ratio)[0] for _ in range(P)]
+        a0 = sprinkled(rng, n, 1e-4)
+        acc2, outp = dev(a0), payload(hp.sparse_payload_bytes(n, ratio))
+        hp.dgc_decode_merge([dev(p) for p in sp], agg, acc2, outp, ratio)
+        want_agg, want_out, want_acc = oracle.sparse_decode_merge(sp, n, a0, ratio)
+        feq(host(agg), want_agg, "sparse merge " + where)
+        gp, wp = oracle.sparse_unpack(host(outp)), oracle.sparse_unpack(want_out)
+        assert gp[:3] == wp[:3] and gp[3].view(np.uint32) == wp[3].view(np.uint32), ("sparse merge payload " + where, gp[:4], wp[:4])
+        np.testing.assert_array_equal(gp[4], wp[4], err_msg="sparse merge indices " + where)
+        feq(gp[5], wp[5], "sparse merge values " + where)
+        feq(host(acc2), want_acc, "sparse merge accumulator " + where)
