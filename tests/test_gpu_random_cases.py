@@ -413,3 +413,65 @@ def test_special_values_random_cases(hp):
         np.testing.assert_array_equal(gp[4], wp[4], err_msg="sparse merge indices " + where)
         feq(gp[5], wp[5], "sparse merge values " + where)
         feq(host(acc2), want_acc, "sparse merge accumulator " + where)
+
+
+def test_merge_batches_of_random_chunk_tables(hp):
+    """MergeBatch over tables of chunks of random sizes: every dense algorithm and the sparse
+    merge, 1-16 peers, with and without the re-encode, some chunks starting from a local
+    gradient, some re-encoding chunks without an aggregate buffer, run twice on the same table."""
+    rng = seeded(2031)
+    for table in range(10):
+        alg = ("tbq", "onebit", "terngrad", "dgc")[table % 4]
+        P = int(rng.integers(1, 17))
+        reenc = alg in ("tbq", "dgc") and rng.random() < 0.7
+        tau, ratio = float(F(rng.uniform(0.01, 0.1))), float(10 ** rng.uniform(-3, -1.5))
+        bucket = int(rng.choice([512, 256, 100, 3000, 5000]))
+        ns = sizes(rng, int(rng.integers(2, 14)), top=600_000)
+        chunks, pays_all, locals_, states = [], [], [], []
+        z = lambda n: np.zeros(n, F)
+        for n in ns:
+            if alg == "tbq":
+                pays = [oracle.tbq_encode(rng.normal(0, 0.04, n).astype(F), z(n), tau)[0] for _ in range(P)]
+            elif alg == "onebit":
+                pays = [oracle.onebit_encode(rng.normal(0, 1e-2, n).astype(F), z(n))[0] for _ in range(P)]
+            elif alg == "terngrad":
+                pays = [oracle.terngrad_encode(rng.normal(0, 1e-3, n).astype(F), rng.random(n, dtype=F), bucket) for _ in range(P)]
+            else:
+                pays = [oracle.graddrop_encode(rng.normal(0, 1e-3, n).astype(F), z(n), ratio)[0] for _ in range(P)]
+            local = rng.normal(0, 1e-2, n).astype(F) if rng.random() < 0.4 else None
+            st = rng.normal(0, 1e-3, n).astype(F)
+            c = {"compressed": [dev(p) for p in pays]}
+            if not (reenc and rng.random() < 0.3):
+                c["aggregate"] = torch.full((n,), 7.0, device="cuda")
+            else:
+                c["aggregate"] = None
+            if reenc:
+                nb = hp.tbq_payload_bytes(n) if alg == "tbq" else hp.sparse_payload_bytes(n, ratio)
+                c["state"], c["out_compressed"] = dev(st), payload(nb)
+            if local is not None:
+                c["local"] = dev(local)
+            chunks.append(c); pays_all.append(pays); locals_.append(local); states.append(st)
+        mb = hp.MergeBatch(alg, chunks, threshold=tau, bucket=bucket, ratio=ratio)
+        for rnd in range(2):
+            mb.run()
+            for k, (c, n, pays, local) in enumerate(zip(chunks, ns, pays_all, locals_)):
+                where = f"table {table} ({alg}, {P} peers, re-encode {reenc}) round {rnd} chunk {k} n={n}"
+                if alg == "tbq":
+                    want = oracle.tbq_decode_merge(pays, n, states[k] if reenc else None, tau if reenc else 0.0, local=local)
+                elif alg == "onebit":
+                    want = oracle.onebit_decode_merge(pays, n, local=local)
+                elif alg == "terngrad":
+                    want = oracle.terngrad_decode_merge(pays, n, local=local)
+                else:
+                    want = oracle.sparse_decode_merge(pays, n, states[k] if reenc else None, ratio if reenc else 0.0, local=local)
+                agg, outp, st = want if reenc else (want, None, None)
+                if c["aggregate"] is not None:
+                    np.testing.assert_array_equal(host(c["aggregate"]), agg, err_msg="aggregate " + where)
+                if reenc:
+                    if alg == "tbq":
+                        np.testing.assert_array_equal(host(c["out_compressed"]), outp, err_msg="payload " + where)
+                    else:
+                        check_sparse(host(c["out_compressed"]), outp, "payload " + where)
+                    np.testing.assert_array_equal(host(c["state"]), st, err_msg="state " + where)
+                    states[k] = st  # the next round starts from the state this one left
+        mb.close()
