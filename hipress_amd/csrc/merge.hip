@@ -21,6 +21,34 @@ __device__ __forceinline__ f4 expand_codes(unsigned byte, float sc) {
     return o;
 }
 
+// The same sum for a scale that is finite and not negative ("plain": its bits, read as an unsigned
+// number, lie below those of +Inf), at two thirds of the instructions.  A code is then worth a
+// multiplier 0, +1 or -1, and agg + value is one fused multiply-add: the product is exact, so the
+// result is rounded once like the addition of +-s, and a code of 0 adds the product +0 like the
+// addition of 0.f (sc = NaN or an infinity would turn 0 * sc into NaN, a negative sc into -0:
+// those scales take expand_codes).  The multipliers of a byte's four codes are made together as
+// two-bit signed fields: 00 -> 00, 01 -> 01, 10 -> 11, and the unused 11 -> 00.  Used for TBQ
+// peers, whose scale is one number per peer (8 peers over the VGG19 chunks without re-encode
+// 200 -> 184 us); with TernGrad's per-bucket scales the decision costs more than it saves
+// (377 -> 396 us per lane, 409 us per wavefront and peer).
+__device__ __forceinline__ bool plain_scale(float sc) { return __float_as_uint(sc) < 0x7f800000u; }
+
+__device__ __forceinline__ unsigned code_multipliers(unsigned byte) {
+    const unsigned hi = byte >> 1;
+    const unsigned one = (byte ^ hi) & 0x55u;    // exactly one bit of the code set: the low bit of the field
+    const unsigned neg = hi & ~byte & 0x55u;     // code 10: also the high bit
+    return one | (neg << 1);
+}
+
+__device__ __forceinline__ f4 add_codes_plain(f4 agg, unsigned byte, float sc) {
+    const int m = (int)code_multipliers(byte);
+    agg.x = __fmaf_rn((float)(int)__builtin_amdgcn_sbfe(m, 0, 2), sc, agg.x);
+    agg.y = __fmaf_rn((float)(int)__builtin_amdgcn_sbfe(m, 2, 2), sc, agg.y);
+    agg.z = __fmaf_rn((float)(int)__builtin_amdgcn_sbfe(m, 4, 2), sc, agg.z);
+    agg.w = __fmaf_rn((float)(int)__builtin_amdgcn_sbfe(m, 6, 2), sc, agg.w);
+    return agg;
+}
+
 __device__ __forceinline__ unsigned tbq_q(float v, float tau, float& keep) {
     unsigned c = v >= tau ? 1u : (v <= -tau ? 2u : 0u);
     keep = c == 1u ? v - tau : (c == 2u ? v + tau : v);
@@ -82,6 +110,7 @@ __device__ __forceinline__ void merge_tile(const MergeSeg& m, unsigned tile, int
 #pragma unroll
         for (int q = 0; q < kPeerChunk; ++q) {
             if (!use[q]) continue;  // wavefront-uniform
+            const bool plain = ALG == HIPRESS_TBQ && plain_scale(sc[q]);  // the same for the whole launch of a peer
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 if (ALG == HIPRESS_ONEBIT) {
@@ -97,7 +126,8 @@ __device__ __forceinline__ void merge_tile(const MergeSeg& m, unsigned tile, int
                     const uint32_t w = (uint32_t)__shfl((int)wq[q], j * 16 + (int)(lane >> 2), 64);
                     const unsigned byte = (w >> (8 * (lane & 3u))) & 0xffu;
                     if (ALG == HIPRESS_TBQ) {
-                        agg[j] = agg[j] + expand_codes(byte, sc[q]);
+                        if (plain) agg[j] = add_codes_plain(agg[j], byte, sc[q]);
+                        else agg[j] = agg[j] + expand_codes(byte, sc[q]);
                     }
                 }
             }
