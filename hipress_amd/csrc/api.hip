@@ -365,6 +365,7 @@ struct hipress_merge_batch {
     void* ws = nullptr;
     SparseWsLayout swl{};
     void* iws = nullptr;  // sparse: per tile a head and one run record per peer
+    unsigned* tgflags = nullptr;  // terngrad with a bucket size that is a multiple of 256: per chunk, does a header disagree
     unsigned slices = 1;  // sparse: the largest peer buffer's slots / 1024, rounded up
     unsigned long long expect_pairs = 0;  // sparse re-encode: sum over the chunks
     std::atomic<unsigned> epoch{0};
@@ -1052,6 +1053,7 @@ int hipress_merge_batch_destroy(hipress_merge_batch* b) {
     if (!b) return HIPRESS_OK;
     (void)hipFree(b->d_segs);
     (void)hipFree(b->iws);
+    (void)hipFree(b->tgflags);
     (void)hipFree(b->d_renc);
     (void)hipFree(b->d_map);
     (void)hipFree(b->d_smap);
@@ -1129,6 +1131,10 @@ static int merge_batch_create_impl(hipress_merge_batch** out, int32_t alg, const
         for (const MergeSeg& m : b->segs)
             for (int p = 0; p < npeers; ++p) b->slices = std::max(b->slices, slices_of(m.peer_slots[p]));
     }
+    if (alg == HIPRESS_TERNGRAD && params->bucket >= 256 && params->bucket % 256 == 0 && !b->segs.empty()) {
+        // the lean merge kernel (every descriptor names this bucket size): one flag per chunk, written by every run
+        if (hipMalloc(reinterpret_cast<void**>(&b->tgflags), 4 * b->segs.size()) != hipSuccess) return fail(HIPRESS_ERR_HIP);
+    }
     if ((rc = upload(b->segs, &b->d_segs))) return fail(rc);
     if ((rc = upload(b->renc, &b->d_renc))) return fail(rc);
     if ((rc = upload(map, &b->d_map))) return fail(rc);
@@ -1164,6 +1170,7 @@ static int merge_batch_run_impl(hipress_merge_batch* b, int phase, void* stream)
     L.reencode = b->reencode;
     L.aggregate = b->aggregate;
     L.local = b->local;
+    L.tgflags = b->tgflags;
     if (b->alg == HIPRESS_DGC || b->alg == HIPRESS_GRADDROP) {
         if (phase > 2) return HIPRESS_ERR_PARAM;
         PeerRun* runs = static_cast<PeerRun*>(b->iws);

@@ -408,6 +408,7 @@ struct MergeLaunch {
     bool reencode;
     bool aggregate;  // some chunk of the launch writes its fp32 sum
     bool local;      // some chunk of the launch starts its sum from a local gradient
+    unsigned* tgflags;  // terngrad batch whose descriptors name a bucket size that is a multiple of 256: one word per chunk
 };
 
 }  // namespace hp

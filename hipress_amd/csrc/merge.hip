@@ -242,6 +242,68 @@ __device__ __forceinline__ bool tg_request(const uint8_t* pay, unsigned long lon
     return true;
 }
 
+// The tile function for a launch whose bucket size is named by the host and is a multiple of 256
+// (512, the usual one, among them): a step's 256 elements then share a bucket, so nothing below
+// looks at single elements, and no peer is set up a second time - which is what makes the general
+// function further down take 121 registers and 365 us for 8 peers over the VGG19 chunks, against
+// 90 registers and 230 us here.  It holds no code for a peer whose header names another bucket size
+// and does not even read the headers (eight more scalar loads per wavefront and tile cost 35 us):
+// a launch of one wavefront per chunk looks at them first and flags the chunks in which some
+// header disagrees (terngrad_headers_kernel); a flagged chunk's tiles store nothing here - the flag
+// is asked for at the start and looked at before the stores - and are written by a third launch,
+// a few workgroups per chunk that run the general function over the flagged chunks' tiles and
+// return at once from the others (terngrad_others_kernel).
+template <bool FAST, bool LOCAL>
+__device__ __forceinline__ void merge_tile_terngrad_lean(const MergeSeg& m, unsigned tile, int npeers, const unsigned* flags) {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const Seg s = m.s;
+    const long long n = (long long)s.n;
+    const long long base = (long long)tile * kTile + wave * kWaveTile;
+    if (base >= n) return;
+    const unsigned B = s.bucket;  // a multiple of 256, at least 256: the host has seen to it
+    const unsigned flagged = flags[s.id];
+    const TgGeom g = tg_geom(B, (unsigned)n, (unsigned)base);
+    unsigned pq[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const unsigned long long x = (unsigned long long)g.r0 + (unsigned)(j * 256);
+        pq[j] = g.q0 + (unsigned)(x >= B) + (unsigned)(x >= 2ull * B) + (unsigned)(x >= 3ull * B);
+    }
+    f4 agg[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        agg[j] = (f4){0.f, 0.f, 0.f, 0.f};
+        if (LOCAL && s.g) agg[j] = load4<FAST>(s.g, base + j * 256 + lane * 4, n);
+    }
+    constexpr int kPeerChunk = 8;
+    for (int p0 = 0; p0 < npeers; p0 += kPeerChunk) {
+        uint32_t wq[kPeerChunk];
+        float tsc[kPeerChunk][4];
+        unsigned usemask = 0u;
+#pragma unroll
+        for (int q = 0; q < kPeerChunk; ++q) {
+            wq[q] = 0u;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) tsc[q][j] = 0.f;
+            if (p0 + q >= npeers) continue;
+            if (tg_request<FAST>(m.peer[p0 + q], m.peer_bytes[p0 + q], g, pq, n, base, lane, wq[q], tsc[q])) usemask |= 1u << q;
+        }
+#pragma unroll
+        for (int q = 0; q < kPeerChunk; ++q) {
+            if (!((usemask >> q) & 1u)) continue;  // wavefront-uniform
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t w = (uint32_t)__shfl((int)wq[q], j * 16 + (int)(lane >> 2), 64);
+                const unsigned byte = (w >> (8 * (lane & 3u))) & 0xffu;
+                agg[j] = agg[j] + expand_codes(byte, tsc[q][j]);  // codes beyond n are 0
+            }
+        }
+    }
+    if (flagged) return;  // wavefront-uniform: the third launch writes this chunk's tiles
+#pragma unroll
+    for (int j = 0; j < 4; ++j) store4<FAST>(s.out, base + j * 256 + lane * 4, n, agg[j]);
+}
+
 template <bool FAST, bool LOCAL>
 __device__ __forceinline__ void merge_tile_terngrad(const MergeSeg& m, unsigned tile, int npeers) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
@@ -338,8 +400,9 @@ __device__ __forceinline__ void merge_tile_terngrad(const MergeSeg& m, unsigned 
     for (int j = 0; j < 4; ++j) store4<FAST>(s.out, base + j * 256 + lane * 4, n, agg[j]);
 }
 
-template <class MSrc, int ALG, bool REENC, bool LOCAL>
-__global__ __launch_bounds__(kBlock) void dense_merge_kernel(MSrc src, int npeers) {
+// LEAN (TernGrad only): the lean tile function; flags: one word per chunk, not zero where a header disagrees.
+template <class MSrc, int ALG, bool REENC, bool LOCAL, bool LEAN = false>
+__global__ __launch_bounds__(kBlock) void dense_merge_kernel(MSrc src, int npeers, const unsigned* flags) {
     unsigned tile;
     const MergeSeg& m = src.get(tile, blockIdx.x);
     if (REENC && tile == 0 && threadIdx.x == 0) {
@@ -351,11 +414,38 @@ __global__ __launch_bounds__(kBlock) void dense_merge_kernel(MSrc src, int npeer
     }
     const bool fast = m.s.aligned && (unsigned long long)(tile + 1) * kTile <= m.s.n;
     if constexpr (ALG == HIPRESS_TERNGRAD) {
-        if (fast) merge_tile_terngrad<true, LOCAL>(m, tile, npeers);
-        else merge_tile_terngrad<false, LOCAL>(m, tile, npeers);
+        if constexpr (LEAN) {
+            if (fast) merge_tile_terngrad_lean<true, LOCAL>(m, tile, npeers, flags);
+            else merge_tile_terngrad_lean<false, LOCAL>(m, tile, npeers, flags);
+        } else {
+            if (fast) merge_tile_terngrad<true, LOCAL>(m, tile, npeers);
+            else merge_tile_terngrad<false, LOCAL>(m, tile, npeers);
+        }
     } else {
         if (fast) merge_tile<true, ALG, REENC, LOCAL>(m, tile, npeers);
         else merge_tile<false, ALG, REENC, LOCAL>(m, tile, npeers);
+    }
+}
+
+// One wavefront per chunk: flags[chunk] = some peer's header names another bucket size than the launch.
+template <class SegSrc>
+__global__ __launch_bounds__(64) void terngrad_headers_kernel(SegSrc src, int npeers, unsigned* flags) {
+    const MergeSeg& m = src.at(blockIdx.x);
+    const unsigned B = m.s.bucket;
+    unsigned differ = 0u;
+    for (int p = (int)threadIdx.x; p < npeers; p += 64) differ |= reinterpret_cast<const uint32_t*>(m.peer[p])[1] ^ B;
+    const bool any = __any(differ != 0u);
+    if (threadIdx.x == 0) flags[m.s.id] = any ? 1u : 0u;
+}
+
+// The general function over the tiles of the flagged chunks; gridDim.y workgroups share a chunk's tiles.
+template <class SegSrc, bool LOCAL>
+__global__ __launch_bounds__(kBlock) void terngrad_others_kernel(SegSrc src, int npeers, const unsigned* flags) {
+    const MergeSeg& m = src.at(blockIdx.x);
+    if (!flags[m.s.id]) return;
+    for (unsigned tile = blockIdx.y; tile < m.s.ntiles; tile += gridDim.y) {
+        if (m.s.aligned && (unsigned long long)(tile + 1) * kTile <= m.s.n) merge_tile_terngrad<true, LOCAL>(m, tile, npeers);
+        else merge_tile_terngrad<false, LOCAL>(m, tile, npeers);
     }
 }
 
@@ -363,13 +453,19 @@ template <class MSrc, bool LOCAL>
 static hipError_t dense_merge_src(const MSrc& src, const MergeLaunch& L, int alg, hipStream_t st) {
     dim3 g(L.ntiles), b(kBlock);
     if (alg == HIPRESS_ONEBIT)
-        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_ONEBIT, false, LOCAL>), g, b, 0, st, src, L.npeers);
+        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_ONEBIT, false, LOCAL>), g, b, 0, st, src, L.npeers, static_cast<const unsigned*>(nullptr));
+    else if (alg == HIPRESS_TERNGRAD && L.tgflags) {  // a batch whose bucket size is a multiple of 256
+        const MergeBatchSegSrc segs{L.dsegs};
+        hipLaunchKernelGGL((terngrad_headers_kernel<MergeBatchSegSrc>), dim3(L.nsegs), dim3(64), 0, st, segs, L.npeers, L.tgflags);
+        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TERNGRAD, false, LOCAL, true>), g, b, 0, st, src, L.npeers, L.tgflags);
+        hipLaunchKernelGGL((terngrad_others_kernel<MergeBatchSegSrc, LOCAL>), dim3(L.nsegs, 8), b, 0, st, segs, L.npeers, L.tgflags);
+    }
     else if (alg == HIPRESS_TERNGRAD)
-        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TERNGRAD, false, LOCAL>), g, b, 0, st, src, L.npeers);
+        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TERNGRAD, false, LOCAL>), g, b, 0, st, src, L.npeers, static_cast<const unsigned*>(nullptr));
     else if (L.reencode)
-        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TBQ, true, LOCAL>), g, b, 0, st, src, L.npeers);
+        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TBQ, true, LOCAL>), g, b, 0, st, src, L.npeers, static_cast<const unsigned*>(nullptr));
     else
-        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TBQ, false, LOCAL>), g, b, 0, st, src, L.npeers);
+        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TBQ, false, LOCAL>), g, b, 0, st, src, L.npeers, static_cast<const unsigned*>(nullptr));
     return hipGetLastError();
 }
 

@@ -511,6 +511,43 @@ def test_terngrad_merge_batch_with_peers_of_other_bucket_sizes(hp, expected, roo
     mb.close()
 
 
+@pytest.mark.parametrize("bucket", [512, 4096])
+def test_terngrad_merge_batch_where_only_some_chunks_hold_another_bucket_size(hp, bucket):
+    """With a bucket size that is a multiple of 256 the batch runs a kernel that knows nothing of
+    other sizes; chunks in which some header disagrees are flagged by a launch before it and written
+    by a launch after it.  Six chunks (one of them starting from a local gradient, 16 peers in two
+    rounds), the odd ones with one peer of another size; then the payloads change places in the same
+    buffers, so that the flags of the second run are the opposite of the first's."""
+    rng = np.random.default_rng(bucket)
+    P, sizes = 16, [4096 * 3 + 5, 100003, 4096, 70001, 300007, 17]
+    room = {n: max(hp.terngrad_payload_bytes(n, b) for b in (bucket, 100, 64)) for n in sizes}
+    grads = {n: [(rng.normal(0, 1e-3, n).astype(F), rng.random(n, dtype=F)) for _ in range(P)] for n in sizes}
+    local = rng.normal(0, 1e-3, sizes[1]).astype(F)
+    chunks = []
+    for k, n in enumerate(sizes):
+        c = {"compressed": [torch.zeros(room[n], dtype=torch.uint8, device="cuda") for _ in range(P)],
+             "aggregate": torch.full((n,), 7.0, device="cuda")}
+        if k == 1:
+            c["local"] = dev(local)
+        chunks.append(c)
+    mb = hp.MergeBatch("terngrad", chunks, bucket=bucket)
+    for rnd in range(3):
+        for k, (c, n) in enumerate(zip(chunks, sizes)):
+            odd_one = (k + rnd) % 2 == 1
+            pays = []
+            for p, (g, u) in enumerate(grads[n]):
+                b = (100 if p == 11 else 64) if odd_one and p in (3, 11) and (p == 3 or rnd == 2) else bucket
+                pays.append(oracle.terngrad_encode(g, u, b))
+                c["compressed"][p].zero_()
+                c["compressed"][p][: pays[-1].size] = dev(pays[-1])
+            c["want"] = oracle.terngrad_decode_merge(pays, n, local=local if k == 1 else None)
+            c["aggregate"].fill_(7.0)
+        mb.run()
+        for k, (c, n) in enumerate(zip(chunks, sizes)):
+            np.testing.assert_array_equal(host(c["aggregate"]), c["want"], err_msg=f"round {rnd} chunk {k} n={n}")
+    mb.close()
+
+
 @pytest.mark.parametrize("n", [1000, 1048576])
 def test_sparse_decode_merge(hp, n):
     P, ratio = 8, 0.001
