@@ -347,6 +347,9 @@ class MergeWorkload:
         if alg == "tbq":
             self.enc_bytes, self.dec_bytes = 0.25 * npeers + agg_bytes + 8.25, 0.0
             self.dominant_kernel, self.dominant_bytes = "dense_merge_kernel", self.enc_bytes
+        elif alg == "terngrad":  # sum only: TernGrad keeps no state to re-encode against (buckets of 512)
+            self.enc_bytes, self.dec_bytes = (0.25 + 4.0 / 512) * npeers + agg_bytes, 0.0
+            self.dominant_kernel, self.dominant_bytes = "dense_merge_kernel", self.enc_bytes
         else:
             self.enc_bytes, self.dec_bytes = 8.0 + agg_bytes, 0.0  # + 8*(P*rho + rho'), added after the run
             self.dominant_kernel, self.dominant_bytes = "sparse_merge_kernel", 8.0 + agg_bytes
@@ -361,11 +364,12 @@ class MergeWorkload:
         self.ratio = ratio
         chunks = []
         for n in self.sizes:
-            nb = hp.tbq_payload_bytes(n) if self.alg == "tbq" else hp.dgc_payload_bytes(n, ratio)
-            chunks.append({"compressed": [torch.zeros(nb, dtype=torch.uint8, device=dev) for _ in range(self.npeers)],
-                           "aggregate": torch.empty(n, device=dev) if self.aggregate else None,
-                           "state": torch.zeros(n, device=dev),
-                           "out_compressed": torch.zeros(nb, dtype=torch.uint8, device=dev)})
+            nb = {"tbq": hp.tbq_payload_bytes(n), "terngrad": hp.terngrad_payload_bytes(n, 512)}.get(self.alg) or hp.dgc_payload_bytes(n, ratio)
+            c = {"compressed": [torch.zeros(nb, dtype=torch.uint8, device=dev) for _ in range(self.npeers)],
+                 "aggregate": torch.empty(n, device=dev) if self.aggregate else None}
+            if self.alg != "terngrad":
+                c["state"], c["out_compressed"] = torch.zeros(n, device=dev), torch.zeros(nb, dtype=torch.uint8, device=dev)
+            chunks.append(c)
         if self.local:
             for c, g in zip(chunks, W.normal_set(self.sizes, dev, 0, sigma=0.02 if self.alg == "tbq" else 1e-3)):
                 c["local"] = g
@@ -376,20 +380,24 @@ class MergeWorkload:
                 ts = [{"gradient": g, "residual": torch.zeros_like(g), "compressed": c["compressed"][p]}
                       for g, c in zip(grads, chunks)]
                 b = hp.Batch("tbq", ts, threshold=tau)
+            elif self.alg == "terngrad":
+                grads = W.normal_set(self.sizes, dev, p + 1, sigma=1e-3)
+                ts = [{"gradient": g, "compressed": c["compressed"][p]} for g, c in zip(grads, chunks)]
+                b = hp.Batch("terngrad", ts, bucket=512)  # no noise tensors: the peers draw from seed p
             else:
                 grads = W.normal_set(self.sizes, dev, p + 1, sigma=1e-3)
                 ts = [{"gradient": g, "momentum": torch.zeros_like(g), "accumulator": torch.zeros_like(g),
                        "compressed": c["compressed"][p]} for g, c in zip(grads, chunks)]
                 b = hp.Batch("dgc", ts, momentum_factor=0.9, ratio=ratio)
-            b.encode()
+            b.encode(seed=p) if self.alg == "terngrad" else b.encode()
             torch.cuda.synchronize()
             b.close()
             del grads, ts
         self.chunks = chunks
-        self.mb = hp.MergeBatch(self.alg, chunks, threshold=tau, ratio=ratio)
+        self.mb = hp.MergeBatch(self.alg, chunks, threshold=tau, bucket=512, ratio=ratio)
 
     def step(self, ev=None):
-        if ev is not None and self.alg == "tbq":
+        if ev is not None and self.alg in ("tbq", "terngrad"):
             ev[0].record()
             self.mb.run()
             ev[1].record()
@@ -417,8 +425,8 @@ class MergeWorkload:
             pays = [p.cpu().numpy() for p in self.chunks[i]["compressed"]]
             arr = (ctypes.c_void_p * P)(*[p.ctypes.data for p in pays])
             loc = self.chunks[i]["local"].cpu().numpy() if self.local else None
-            jobs.append((n, pays, arr, np.empty(n, np.float32), np.zeros(n, np.float32),
-                         np.zeros(self.chunks[i]["out_compressed"].numel(), np.uint8), loc))
+            out_bytes = self.chunks[i]["out_compressed"].numel() if "out_compressed" in self.chunks[i] else 0
+            jobs.append((n, pays, arr, np.empty(n, np.float32), np.zeros(n, np.float32), np.zeros(out_bytes, np.uint8), loc))
         total = sum(j[0] for j in jobs)
 
         def run(L):
@@ -426,10 +434,12 @@ class MergeWorkload:
                 lp = _vp(loc) if loc is not None else None
                 if alg == "tbq":
                     L.hpo_tbq_decode_merge_local(arr, P, lp, _vp(agg), n, _vp(state), _vp(outp), 0.05)
+                elif alg == "terngrad":
+                    L.hpo_terngrad_decode_merge_local(arr, P, lp, _vp(agg), n)
                 else:
                     L.hpo_sparse_decode_merge_local(arr, P, lp, _vp(agg), n, _vp(state), _vp(outp), ratio)
 
-        what = (f"{alg} decode-and-merge of {P} peers + re-encode over the {len(jobs)} largest of "
+        what = (f"{alg} decode-and-merge of {P} peers{'' if alg == 'terngrad' else ' + re-encode'} over the {len(jobs)} largest of "
                 f"{len(self.sizes)} chunks ({total:,} elements per pass)")
         return CpuJob(total, what, run)
 
@@ -598,6 +608,8 @@ def make_workload(name):
         return MergeWorkload(name, "tbq", W.chunk_sizes(vgg))
     if name == "merge_dgc_vgg19":
         return MergeWorkload(name, "dgc", W.chunk_sizes(vgg))
+    if name == "merge_terngrad_vgg19":  # the sum alone: TernGrad has no state to re-encode against
+        return MergeWorkload(name, "terngrad", W.chunk_sizes(vgg))
     if name == "merge_tbq_vgg19_payload_only":
         return MergeWorkload(name, "tbq", W.chunk_sizes(vgg), aggregate=False)
     if name == "merge_dgc_vgg19_payload_only":
@@ -613,7 +625,7 @@ ALL_WORKLOADS = [
     "tbq_262144", "tbq_262144_x512", "terngrad_resnet50", "dgc_bert_large", "graddrop_bert_large",
     "merge_tbq_vgg19", "merge_dgc_vgg19", "compll_b2_fc6", "compll_generated_b2_fc6", "tbq_fc6", "tbq_generated_fc6",
     "merge_tbq_vgg19_payload_only", "merge_dgc_vgg19_payload_only", "tbq_vgg19_planned", "hop_tbq_vgg19",
-    "terngrad_seeded_vgg19",
+    "terngrad_seeded_vgg19", "merge_terngrad_vgg19",
 ]
 # any workload with the suffix _graph: the same step captured once into a HIP graph and replayed
 EXTRA_WORKLOADS = [w + "_graph" for w in ALL_WORKLOADS]
