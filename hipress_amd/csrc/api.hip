@@ -365,7 +365,7 @@ struct hipress_merge_batch {
     void* ws = nullptr;
     SparseWsLayout swl{};
     void* iws = nullptr;  // sparse: per tile a head and one run record per peer
-    unsigned* tgflags = nullptr;  // terngrad with a bucket size that is a multiple of 256: per chunk, does a header disagree
+    unsigned* tgflags = nullptr;  // terngrad: per chunk, does some peer's header disagree with the batch's bucket size
     unsigned slices = 1;  // sparse: the largest peer buffer's slots / 1024, rounded up
     unsigned long long expect_pairs = 0;  // sparse re-encode: sum over the chunks
     std::atomic<unsigned> epoch{0};
@@ -1131,8 +1131,8 @@ static int merge_batch_create_impl(hipress_merge_batch** out, int32_t alg, const
         for (const MergeSeg& m : b->segs)
             for (int p = 0; p < npeers; ++p) b->slices = std::max(b->slices, slices_of(m.peer_slots[p]));
     }
-    if (alg == HIPRESS_TERNGRAD && params->bucket >= 256 && params->bucket % 256 == 0 && !b->segs.empty()) {
-        // the lean merge kernel (every descriptor names this bucket size): one flag per chunk, written by every run
+    if (alg == HIPRESS_TERNGRAD && params->bucket >= 1 && !b->segs.empty()) {
+        // the lean merge kernels (every descriptor names this bucket size): one flag per chunk, written by every run
         if (hipMalloc(reinterpret_cast<void**>(&b->tgflags), 4 * b->segs.size()) != hipSuccess) return fail(HIPRESS_ERR_HIP);
     }
     if ((rc = upload(b->segs, &b->d_segs))) return fail(rc);
@@ -1171,6 +1171,7 @@ static int merge_batch_run_impl(hipress_merge_batch* b, int phase, void* stream)
     L.aggregate = b->aggregate;
     L.local = b->local;
     L.tgflags = b->tgflags;
+    L.bucket256 = b->params.bucket >= 256 && b->params.bucket % 256 == 0;
     if (b->alg == HIPRESS_DGC || b->alg == HIPRESS_GRADDROP) {
         if (phase > 2) return HIPRESS_ERR_PARAM;
         PeerRun* runs = static_cast<PeerRun*>(b->iws);

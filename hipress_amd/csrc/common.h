@@ -408,7 +408,8 @@ struct MergeLaunch {
     bool reencode;
     bool aggregate;  // some chunk of the launch writes its fp32 sum
     bool local;      // some chunk of the launch starts its sum from a local gradient
-    unsigned* tgflags;  // terngrad batch whose descriptors name a bucket size that is a multiple of 256: one word per chunk
+    unsigned* tgflags;  // terngrad batch (its descriptors name the bucket size): one word per chunk, does a header disagree
+    bool bucket256;     // and that size is a multiple of 256
 };
 
 }  // namespace hp

@@ -242,32 +242,40 @@ __device__ __forceinline__ bool tg_request(const uint8_t* pay, unsigned long lon
     return true;
 }
 
-// The tile function for a launch whose bucket size is named by the host and is a multiple of 256
-// (512, the usual one, among them): a step's 256 elements then share a bucket, so nothing below
-// looks at single elements, and no peer is set up a second time - which is what makes the general
-// function further down take 121 registers and 365 us for 8 peers over the VGG19 chunks, against
-// 90 registers and 230 us here.  It holds no code for a peer whose header names another bucket size
+// The tile function for a launch whose bucket size is named by the host (a batch).  With a multiple of
+// 256 (512, the usual one, among them) a step's 256 elements share a bucket, so nothing below
+// looks at single elements; and with any size no peer is set up a second time - which is what makes
+// the general function further down take 121 registers and 365 us for 8 peers over the VGG19 chunks,
+// against 94 registers and 235 us here.  It holds no code for a peer whose header names another bucket size
 // and does not even read the headers (eight more scalar loads per wavefront and tile cost 35 us):
 // a launch of one wavefront per chunk looks at them first and flags the chunks in which some
 // header disagrees (terngrad_headers_kernel); a flagged chunk's tiles store nothing here - the flag
 // is asked for at the start and looked at before the stores - and are written by a third launch,
 // a few workgroups per chunk that run the general function over the flagged chunks' tiles and
 // return at once from the others (terngrad_others_kernel).
-template <bool FAST, bool LOCAL>
+// B256: the bucket size is a multiple of 256; otherwise it is any size, the lane's first elements are
+// placed by division and four elements that straddle a bucket border look their scales up one by one
+// (8 peers, buckets of 100: 411 us in the general function, 324 us here).
+template <bool FAST, bool LOCAL, bool B256>
 __device__ __forceinline__ void merge_tile_terngrad_lean(const MergeSeg& m, unsigned tile, int npeers, const unsigned* flags) {
     const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const Seg s = m.s;
     const long long n = (long long)s.n;
     const long long base = (long long)tile * kTile + wave * kWaveTile;
     if (base >= n) return;
-    const unsigned B = s.bucket;  // a multiple of 256, at least 256: the host has seen to it
+    const unsigned B = s.bucket;  // named by the host, at least 1 (B256: a multiple of 256)
     const unsigned flagged = flags[s.id];
     const TgGeom g = tg_geom(B, (unsigned)n, (unsigned)base);
-    unsigned pq[4];
+    unsigned pq[4], pr[4];
+    if (B256) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const unsigned long long x = (unsigned long long)g.r0 + (unsigned)(j * 256);
-        pq[j] = g.q0 + (unsigned)(x >= B) + (unsigned)(x >= 2ull * B) + (unsigned)(x >= 3ull * B);
+        for (int j = 0; j < 4; ++j) {
+            const unsigned long long x = (unsigned long long)g.r0 + (unsigned)(j * 256);
+            pq[j] = g.q0 + (unsigned)(x >= B) + (unsigned)(x >= 2ull * B) + (unsigned)(x >= 3ull * B);
+            pr[j] = 0u;
+        }
+    } else {
+        tg_positions(g, B, lane, pq, pr);
     }
     f4 agg[4];
 #pragma unroll
@@ -295,7 +303,27 @@ __device__ __forceinline__ void merge_tile_terngrad_lean(const MergeSeg& m, unsi
             for (int j = 0; j < 4; ++j) {
                 const uint32_t w = (uint32_t)__shfl((int)wq[q], j * 16 + (int)(lane >> 2), 64);
                 const unsigned byte = (w >> (8 * (lane & 3u))) & 0xffu;
-                agg[j] = agg[j] + expand_codes(byte, tsc[q][j]);  // codes beyond n are 0
+                if (B256 || (B & 255u) == 0u || (unsigned long long)pr[j] + 3ull < B) {
+                    agg[j] = agg[j] + expand_codes(byte, tsc[q][j]);  // the four share a bucket; codes beyond n are 0
+                } else {
+                    const float* scales = reinterpret_cast<const float*>(m.peer[p0 + q] + kHeaderBytes);
+                    const long long e = base + j * 256 + lane * 4;
+                    unsigned bq = pq[j], br = pr[j];
+                    float sck = tsc[q][j], dv[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const unsigned c = (byte >> (2 * k)) & 3u;
+                        dv[k] = (e + k < n && c) ? code_val(c, sck) : 0.f;
+                        if (++br == B) {  // the next element begins a bucket: its scale is looked up here
+                            br = 0u;
+                            ++bq;
+                            if (k < 3 && e + k + 1 < n) sck = scales[bq];
+                        }
+                    }
+                    f4 d;
+                    d.x = dv[0]; d.y = dv[1]; d.z = dv[2]; d.w = dv[3];
+                    agg[j] = agg[j] + d;
+                }
             }
         }
     }
@@ -400,8 +428,9 @@ __device__ __forceinline__ void merge_tile_terngrad(const MergeSeg& m, unsigned 
     for (int j = 0; j < 4; ++j) store4<FAST>(s.out, base + j * 256 + lane * 4, n, agg[j]);
 }
 
-// LEAN (TernGrad only): the lean tile function; flags: one word per chunk, not zero where a header disagrees.
-template <class MSrc, int ALG, bool REENC, bool LOCAL, bool LEAN = false>
+// LEAN (TernGrad only): 1 the lean tile function for bucket sizes that are multiples of 256, 2 the one for any
+// size, 0 the general function; flags: one word per chunk, not zero where a header disagrees.
+template <class MSrc, int ALG, bool REENC, bool LOCAL, int LEAN = 0>
 __global__ __launch_bounds__(kBlock) void dense_merge_kernel(MSrc src, int npeers, const unsigned* flags) {
     unsigned tile;
     const MergeSeg& m = src.get(tile, blockIdx.x);
@@ -414,9 +443,9 @@ __global__ __launch_bounds__(kBlock) void dense_merge_kernel(MSrc src, int npeer
     }
     const bool fast = m.s.aligned && (unsigned long long)(tile + 1) * kTile <= m.s.n;
     if constexpr (ALG == HIPRESS_TERNGRAD) {
-        if constexpr (LEAN) {
-            if (fast) merge_tile_terngrad_lean<true, LOCAL>(m, tile, npeers, flags);
-            else merge_tile_terngrad_lean<false, LOCAL>(m, tile, npeers, flags);
+        if constexpr (LEAN != 0) {
+            if (fast) merge_tile_terngrad_lean<true, LOCAL, LEAN == 1>(m, tile, npeers, flags);
+            else merge_tile_terngrad_lean<false, LOCAL, LEAN == 1>(m, tile, npeers, flags);
         } else {
             if (fast) merge_tile_terngrad<true, LOCAL>(m, tile, npeers);
             else merge_tile_terngrad<false, LOCAL>(m, tile, npeers);
@@ -454,10 +483,13 @@ static hipError_t dense_merge_src(const MSrc& src, const MergeLaunch& L, int alg
     dim3 g(L.ntiles), b(kBlock);
     if (alg == HIPRESS_ONEBIT)
         hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_ONEBIT, false, LOCAL>), g, b, 0, st, src, L.npeers, static_cast<const unsigned*>(nullptr));
-    else if (alg == HIPRESS_TERNGRAD && L.tgflags) {  // a batch whose bucket size is a multiple of 256
+    else if (alg == HIPRESS_TERNGRAD && L.tgflags) {  // a batch: its descriptors name the bucket size
         const MergeBatchSegSrc segs{L.dsegs};
         hipLaunchKernelGGL((terngrad_headers_kernel<MergeBatchSegSrc>), dim3(L.nsegs), dim3(64), 0, st, segs, L.npeers, L.tgflags);
-        hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TERNGRAD, false, LOCAL, true>), g, b, 0, st, src, L.npeers, L.tgflags);
+        if (L.bucket256)
+            hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TERNGRAD, false, LOCAL, 1>), g, b, 0, st, src, L.npeers, L.tgflags);
+        else
+            hipLaunchKernelGGL((dense_merge_kernel<MSrc, HIPRESS_TERNGRAD, false, LOCAL, 2>), g, b, 0, st, src, L.npeers, L.tgflags);
         hipLaunchKernelGGL((terngrad_others_kernel<MergeBatchSegSrc, LOCAL>), dim3(L.nsegs, 8), b, 0, st, segs, L.npeers, L.tgflags);
     }
     else if (alg == HIPRESS_TERNGRAD)
