@@ -339,6 +339,12 @@ typedef struct hipress_merge_chunk {
 
 typedef struct hipress_merge_batch hipress_merge_batch;
 
+/* params: threshold (tbq re-encode), ratio (sparse re-encode), and for terngrad `bucket`, the
+ * bucket size the peers are expected to have used: the merge then works from it without
+ * waiting for the payload headers (8 peers over 168 chunks of 4 MB: 235 us against 365 us
+ * through hipress_terngrad_decode_merge, which learns the size from the headers).  The
+ * headers still decide: a chunk in which some peer's header names another size is summed
+ * from the headers, correctly and more slowly. */
 int hipress_merge_batch_create(hipress_merge_batch **out, int32_t alg,
                                const hipress_merge_chunk *chunks, int32_t count, int32_t npeers,
                                const hipress_params *params);
