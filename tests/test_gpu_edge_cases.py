@@ -795,3 +795,50 @@ def test_hip_graph_replay_of_a_sparse_merge_batch(hp):
             check_sparse(host(c["out_compressed"]), out, f"replay {rep} chunk {i}")
             np.testing.assert_array_equal(host(c["state"]), ref[i], err_msg=f"state, replay {rep} chunk {i}")
     mb.close()
+
+
+@pytest.mark.parametrize("bucket", [512, 100])
+def test_hip_graph_replay_of_a_terngrad_merge_batch(hp, bucket):
+    """The TernGrad merge batch is three launches (headers -> flags, the lean sum, the general sum
+    over flagged chunks).  Captured once, replayed with new peer payloads in the same buffers before
+    every replay; which chunks hold a peer of another bucket size changes from replay to replay,
+    so the flags a replay writes differ from the ones the capture saw."""
+    sizes, P = [1048576, 300007, 4097, 70001], 5
+    rng = np.random.default_rng(bucket)
+    room = {n: max(hp.terngrad_payload_bytes(n, b) for b in (bucket, 64, 300)) for n in sizes}
+    chunks = [{"compressed": [torch.zeros(room[n], dtype=torch.uint8, device="cuda") for _ in range(P)],
+               "aggregate": torch.empty(n, device="cuda")} for n in sizes]
+    mb = hp.MergeBatch("terngrad", chunks, bucket=bucket)
+
+    def new_payloads(odd):
+        want = []
+        for k, (c, n) in enumerate(zip(chunks, sizes)):
+            ps = []
+            for p in range(P):
+                b = (64 if p == 1 else 300) if k % 2 == odd and p in (1, 4) else bucket
+                ps.append(oracle.terngrad_encode(rng.normal(0, 1e-3, n).astype(F), rng.random(n, dtype=F), b))
+                c["compressed"][p].zero_()
+                c["compressed"][p][: ps[-1].size] = dev(ps[-1])
+            want.append(oracle.terngrad_decode_merge(ps, n))
+        return want
+
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    new_payloads(0)
+    with torch.cuda.stream(stream):
+        mb.run()  # warm-up on the capture stream
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            mb.run()
+    for rep in range(4):
+        want = new_payloads(rep % 2 if rep < 3 else 2)  # the last replay: no chunk is flagged
+        for c in chunks:
+            c["aggregate"].fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        _ = (chunks[0]["aggregate"] * 2).sum().item()  # unrelated eager work between replays
+        for i, (c, w) in enumerate(zip(chunks, want)):
+            np.testing.assert_array_equal(host(c["aggregate"]), w, err_msg=f"replay {rep} chunk {i}")
+    mb.close()
+
